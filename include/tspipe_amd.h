@@ -1,0 +1,232 @@
+/*
+ * tspipe_amd.h -- C ABI of the MI355X (gfx950) teacher-student step kernels.
+ *
+ * The reference (kaist-ina/TSPipe) has no native code and no FFI: every
+ * operation below is, there, a chain of eager PyTorch calls made from a Python
+ * plug-in.  Each entry point cites the reference lines whose arithmetic it
+ * replaces; the Python adapters in tspipe_amd/ keep the reference's plug-in
+ * signatures and call these through ctypes.
+ *
+ * Conventions (all entry points):
+ *   - plain C, no C++ or torch types; returns 0 (TS_OK) or a negative TS_ERR_*;
+ *   - every "dev" pointer is device memory owned by the caller and must stay
+ *     alive until the work enqueued on `stream` has run;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream);
+ *   - calls only enqueue work: no implicit synchronisation, no allocation, no
+ *     global mutable state; re-entrant from any thread;
+ *   - workspaces are caller-provided; sizes are stated per function;
+ *   - "plan" functions are pure host code (no GPU needed): they turn tensor
+ *     lists into the chunk tables the kernels walk.
+ */
+#ifndef TSPIPE_AMD_H
+#define TSPIPE_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* ts_stream_t; /* hipStream_t */
+
+enum ts_status {
+  TS_OK = 0,
+  TS_ERR_ARG = -1,      /* null pointer, negative size, unsupported dtype ... */
+  TS_ERR_CAPACITY = -2, /* a plan does not fit the table the caller passed */
+  TS_ERR_LAUNCH = -3,   /* hipLaunchKernel / hipFuncSetAttribute reported an error */
+  TS_ERR_ALIGN = -4,    /* pointer not aligned to its element size */
+  TS_ERR_RANGE = -5     /* size beyond what the kernel's grid/index type covers */
+};
+
+enum ts_dtype { TS_F32 = 0, TS_BF16 = 1, TS_F16 = 2 };
+
+/* Library identification and error text (static strings). */
+const char* ts_version(void);
+const char* ts_error_string(int status);
+/* Last HIP error code recorded by a failed launch in this thread (0 if none). */
+int ts_last_hip_error(void);
+
+/* ------------------------------------------------------------------------ */
+/* Momentum-teacher EMA over a whole parameter list, one launch.         */
+/*                                                                          */
+/* Replaces the per-tensor loop                                              */
+/*     detached = param_k.clone().detach()                                   */
+/*     detached = detached * m + param_q.data * (1. - m)                     */
+/* of benchmarks/byol/trainer.py:198-212 and benchmarks/moco-v3/main.py:     */
+/* 133-144 (in-place twins: byol/trainer.py:43-49, moco/builder.py:57-61).   */
+/* Arithmetic: out = fl32(fl32(t*m32) + fl32(s*c32)), no FMA contraction,    */
+/* m32 = (float)m, c32 = (float)(1.0 - m) with the subtraction in double --  */
+/* the rounding order of the eager fp32 ops, so results are bit-identical.   */
+/* ------------------------------------------------------------------------ */
+
+typedef struct ts_ema_chunk {
+  const float* t; /* teacher (previous target) values of this chunk */
+  const float* s; /* student (online) values */
+  float* out;     /* new teacher values; may alias t for the in-place form */
+  uint32_t n;     /* elements in the chunk (<= chunk_elems) */
+  uint32_t flags; /* bit0: t, s and out are all 16-byte aligned */
+} ts_ema_chunk;   /* 32 bytes */
+
+/* Chunk size the planner picks for `total` elements when chunk_elems == 0. */
+int64_t ts_ema_auto_chunk(int64_t total_elems);
+
+/* Host: split n_tensors (t[i], s[i], out[i], numel[i]) into chunks.
+ * chunk_elems: elements per chunk, a positive multiple of 1024, or 0 = auto.
+ * table == NULL: only count.  Returns the chunk count (>= 0) or TS_ERR_*.
+ * Tensors with numel 0 produce no chunk.  Pointers must be 4-byte aligned. */
+int64_t ts_ema_plan(const void* const* t, const void* const* s, void* const* out,
+                    const int64_t* numel, int64_t n_tensors, int64_t chunk_elems,
+                    ts_ema_chunk* table, int64_t capacity);
+
+/* Device: run the EMA over a table that lives in device memory. */
+int ts_ema_multi(const ts_ema_chunk* table_dev, int64_t n_chunks, float m32, float c32,
+                 ts_stream_t stream);
+
+/* ------------------------------------------------------------------------ */
+/* Multi-segment copy: micro-batch gather (torch.cat on dim 0,      */
+/* tspipe/batch_ops.py:186-205, tspipe/utils.py:280), the owning form of     */
+/* scatter (batch_ops.py:168-183), the student-parameter clone               */
+/* (tspipe/gpu_task.py:398) and the teacher copy-in (gpu_task.py:706-724).   */
+/* Byte-exact for any dtype.                                                 */
+/* ------------------------------------------------------------------------ */
+
+typedef struct ts_copy_chunk {
+  const void* src;
+  void* dst;
+  uint64_t bytes;
+  uint64_t flags; /* bit0: src and dst are both 16-byte aligned */
+} ts_copy_chunk;  /* 32 bytes */
+
+int64_t ts_copy_auto_chunk(int64_t total_bytes);
+
+/* Host: split n_segments (src[i], dst[i], bytes[i]) into chunks of at most
+ * chunk_bytes (positive multiple of 4096, or 0 = auto).  Same return rule as
+ * ts_ema_plan.  Source and destination ranges must not overlap. */
+int64_t ts_copy_plan(const void* const* src, void* const* dst, const int64_t* bytes,
+                     int64_t n_segments, int64_t chunk_bytes, ts_copy_chunk* table,
+                     int64_t capacity);
+
+int ts_copy_segments(const ts_copy_chunk* table_dev, int64_t n_chunks, ts_stream_t stream);
+
+/* ------------------------------------------------------------------------ */
+/* KD soft-target loss, forward and backward in one pass over rows.   */
+/*                                                                          */
+/* Replaces F.kl_div(F.log_softmax(s/T,1), F.softmax(t/T,1), 'batchmean')    */
+/* * T * T (benchmarks/soft_target/kd_losses/st.py:18-23) and the masked     */
+/* wide-vocabulary form of benchmarks/distilbert/distiller.py:719-740        */
+/* (masked_select of rows, KLDivLoss('batchmean'), * temperature**2).        */
+/*                                                                          */
+/*   B       = number of rows with row_mask != 0 (all n_rows if mask NULL)   */
+/*   loss    = loss_scale / B * sum_rows KL(softmax(t/T) || softmax(s/T))    */
+/*   grad_ij = loss_scale * inv_T / B * (q_ij - p_ij) for selected rows,     */
+/*             0 for the others (dense, like masked_select's backward)       */
+/* with loss_scale = T*T*weight chosen by the caller.  B == 0 gives          */
+/* loss = NaN and grad = 0, as the reference's 0/0 does.                     */
+/*                                                                          */
+/* s, t, grad: [n_rows, V] row-major with leading dimensions ld_* in         */
+/* elements; dtype TS_F32 / TS_BF16 / TS_F16 (same for all three);           */
+/* accumulation is fp32.  grad may be NULL (loss only).                      */
+/* workspace: ts_kd_workspace_bytes(n_rows) bytes, 16-byte aligned, contents */
+/* irrelevant on entry.  loss_out: one float.                                */
+/* ------------------------------------------------------------------------ */
+
+size_t ts_kd_workspace_bytes(int64_t n_rows);
+
+int ts_kd_fwd_bwd(const void* s, const void* t, const uint8_t* row_mask, int64_t n_rows,
+                  int64_t V, int64_t ld_s, int64_t ld_t, float inv_T, float loss_scale,
+                  void* workspace, float* loss_out, void* grad, int64_t ld_g, int dtype,
+                  ts_stream_t stream);
+
+/* grad *= *g for the rows the loss touched; returns at once on the device
+ * when *g == 1 (the only value TSPipe's torch.autograd.backward(loss) feeds,
+ * tspipe/gpu_task.py:207-212).  g_dev: one float in device memory. */
+int ts_scale_rows(void* grad, int64_t n_rows, int64_t V, int64_t ld_g, const float* g_dev,
+                  int dtype, ts_stream_t stream);
+
+/* ------------------------------------------------------------------------ */
+/* BYOL normalised-MSE loss, forward and backward.                       */
+/*                                                                          */
+/* Replaces regression_loss (benchmarks/byol/trainer.py:51-55) and           */
+/* contrastive_loss (trainer.py:192-196):                                    */
+/*   rl(x,y)_i = 2 - 2 * <x_i/max(|x_i|,1e-12), y_i/max(|y_i|,1e-12)>        */
+/*   loss = mean_i( rl(x1,y1)_i + rl(x2,y2)_i )      (x2,y2 may be NULL)     */
+/*   gx   = d loss / d x  (teacher side y gets no gradient)                  */
+/* x*, y*, gx*: [n, c] contiguous, same dtype.  workspace: 2*n floats.       */
+/* ------------------------------------------------------------------------ */
+
+int ts_byol_fwd_bwd(const void* x1, const void* y1, const void* x2, const void* y2, int64_t n,
+                    int64_t c, float* workspace, float* loss_out, void* gx1, void* gx2,
+                    int dtype, ts_stream_t stream);
+
+/* ------------------------------------------------------------------------ */
+/* MoCo-v3 InfoNCE loss, forward and backward, logits never stored.      */
+/*                                                                          */
+/* Replaces contrastive_loss.loss (benchmarks/moco-v3/main.py:147-162;       */
+/* single-device twin moco/builder.py:63-71):                                */
+/*   qh = q/max(|q|,1e-12), kh likewise; logits = qh kh^T / tau;             */
+/*   loss = CrossEntropy(logits, arange(N)) * 2 tau   (mean over rows)       */
+/*   dq   = d loss / d q  (k is the detached teacher output)                 */
+/* Up to two (q,k) pairs are summed into one loss (main.py:162); q2,k2,dq2   */
+/* may be NULL.  q*, k*: [n, c] contiguous bf16 (TS_BF16) or fp32 (TS_F32,   */
+/* rounded to bf16 for the MFMA contraction); c a multiple of 32, <= 256.    */
+/* workspace: ts_infonce_workspace_bytes(n, c, n_pairs) bytes, 256-aligned.  */
+/* ------------------------------------------------------------------------ */
+
+size_t ts_infonce_workspace_bytes(int64_t n, int64_t c, int n_pairs);
+
+int ts_infonce_fwd_bwd(const void* q1, const void* k1, const void* q2, const void* k2, int64_t n,
+                       int64_t c, float tau, void* workspace, float* loss_out, void* dq1,
+                       void* dq2, int dtype, ts_stream_t stream);
+
+/* ------------------------------------------------------------------------ */
+/* DeferredBatchNorm (tspipe/batchnorm.py).                           */
+/* x, y, dy, dx: fp32 [N, C, HW] contiguous (NCHW with HW = prod of the      */
+/* trailing dims).                                                           */
+/* ------------------------------------------------------------------------ */
+
+/* _track (batchnorm.py:45-59) fused with the statistics F.batch_norm(
+ * training=True) needs (batchnorm.py:111-120): one read of x gives the
+ * micro-batch's per-channel sum and sum of squares, which are
+ *   - added into the mini-batch accumulators `sum`, `sum_squares` (fp32 +=),
+ *     unless those are NULL;
+ *   - turned into ub_mean = S/cnt and ub_invstd = 1/sqrt(max(Q/cnt - mean^2,0)
+ *     + eps), cnt = N*HW, unless those are NULL.
+ * ws: 2*C floats that are ZERO on entry; the call leaves them zero again. */
+int ts_bn_stats(const float* x, int64_t N, int64_t C, int64_t HW, float* ws, float* sum,
+                float* sum_squares, float* ub_mean, float* ub_invstd, float eps,
+                ts_stream_t stream);
+
+/* _commit (batchnorm.py:61-85): num_batches_tracked += 1;
+ * f = momentum, or 1/num_batches_tracked when momentum < 0 (the reference's
+ * momentum=None); mean = sum/counter; var = sum_squares/counter - mean^2;
+ * running = running*(1-f) + stat*f in the reference's fp32 rounding order;
+ * then sum = sum_squares = 0. */
+int ts_bn_commit(float* sum, float* sum_squares, float* running_mean, float* running_var,
+                 int64_t* num_batches_tracked, int64_t C, double counter, double momentum,
+                 ts_stream_t stream);
+
+/* y = (x - mean[c]) * invstd[c] * gamma[c] + beta[c]; gamma/beta may be NULL
+ * (affine=False).  With is_var != 0 the fourth argument holds variances and
+ * invstd = 1/sqrt(var + eps) is formed on the fly (eval mode with running
+ * statistics, batchnorm.py:88-99). */
+int ts_bn_apply(const float* x, float* y, const float* mean, const float* invstd_or_var,
+                const float* gamma, const float* beta, int64_t N, int64_t C, int64_t HW,
+                int is_var, float eps, ts_stream_t stream);
+
+/* Backward of the normalisation (what autograd derives for F.batch_norm):
+ * dgamma = sum dy*xhat, dbeta = sum dy, and
+ *   training != 0 (batch statistics, batchnorm.py:111-120):
+ *     dx = gamma*invstd*(dy - dbeta/cnt - xhat*dgamma/cnt)
+ *   training == 0 (fixed running statistics, batchnorm.py:88-99):
+ *     dx = gamma*invstd*dy
+ * ws: 2*C floats zero on entry, zero again on return.  dgamma/dbeta: [C]
+ * outputs (required); gamma may be NULL (treated as 1). */
+int ts_bn_backward(const float* x, const float* dy, const float* ub_mean, const float* ub_invstd,
+                   const float* gamma, float* dx, float* dgamma, float* dbeta, float* ws,
+                   int64_t N, int64_t C, int64_t HW, int training, ts_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TSPIPE_AMD_H */

@@ -1,0 +1,169 @@
+"""GPU parity: DeferredBatchNorm statistics, commit, normalisation and backward.
+
+Tolerances: accumulated sums and running statistics within 1e-6 relative of an
+fp64 evaluation; normalised output within 2e-5 absolute of F.batch_norm; the
+state after a commit is also compared with the fp32 oracle.
+"""
+import pytest
+import torch
+import torch.nn.functional as F
+from torch import nn
+
+import tspipe_amd as ta
+from helpers import max_rel_to_peak, seeded
+from oracle import ts_oracle
+
+pytestmark = pytest.mark.gpu
+
+
+def _rel(a, b):
+    a, b = a.detach().cpu().double(), b.detach().cpu().double()
+    return ((a - b).abs() / b.abs().clamp_min(1e-30)).max().item()
+
+
+def _make(shape, seed, mean=0.5, std=1.5):
+    return torch.randn(shape, generator=seeded(seed)) * std + mean
+
+
+@pytest.mark.parametrize("shape,chunks", [((8, 16, 14, 14), 4), ((4, 7, 5, 3), 3), ((2, 3, 9), 2),
+                                          ((3, 5, 2, 2, 3), 2), ((16, 64, 7, 7), 1)])
+def test_deferred_bn_matches_oracle(device, shape, chunks):
+    C = shape[1]
+    g = seeded(40)
+    gamma = torch.rand(C, generator=g) + 0.5
+    beta = torch.randn(C, generator=g) * 0.1
+    bn = ta.DeferredBatchNorm(C, chunks=chunks)
+    with torch.no_grad():
+        bn.weight.copy_(gamma)
+        bn.bias.copy_(beta)
+    bn = bn.to(device)
+    ora = ts_oracle.DeferredBNOracle(C, chunks=chunks, weight=gamma.double(), bias=beta.double(), dtype=torch.float64)
+    for step in range(2 * chunks + 1):
+        x = _make(shape, 50 + step)
+        y = bn(x.to(device))
+        yo = ora.forward(x.double())
+        assert (y.cpu().double() - yo).abs().max().item() < 2e-5
+        assert bn.counter == ora.counter and bn.tracked == ora.tracked
+        if ora.tracked:
+            assert _rel(bn.sum, ora.sum) < 1e-6 and _rel(bn.sum_squares, ora.sum_squares) < 1e-6
+        else:
+            assert (bn.sum == 0).all() and (bn.sum_squares == 0).all()
+        assert _rel(bn.running_mean, ora.running_mean) < 1e-6 or (ora.running_mean == 0).all()
+        assert _rel(bn.running_var, ora.running_var) < 1e-6
+        assert int(bn.num_batches_tracked) == int(ora.num_batches_tracked)
+    assert (bn._ws == 0).all()  # reduction workspace is left clean
+
+
+def test_deferred_bn_cfg5_shape(device):
+    # 8 micro-batches of [32, 256, 56, 56]; oracle in fp64 on per-channel sums
+    C = 256
+    g = seeded(4)
+    gamma = torch.rand(C, generator=g) + 0.5
+    beta = torch.randn(C, generator=g) * 0.1
+    bn = ta.DeferredBatchNorm(C, chunks=8)
+    with torch.no_grad():
+        bn.weight.copy_(gamma)
+        bn.bias.copy_(beta)
+    bn = bn.to(device)
+    S = torch.zeros(C, dtype=torch.float64)
+    Q = torch.zeros(C, dtype=torch.float64)
+    cnt = 0
+    for ub in range(8):
+        x = torch.randn(32, C, 56, 56, generator=g) * 1.5 + 0.5
+        xd = x.to(device)
+        y = bn(xd)
+        xs = x.double()
+        S += xs.sum(dim=(0, 2, 3))
+        Q += (xs * xs).sum(dim=(0, 2, 3))
+        cnt += 32 * 56 * 56
+        if ub in (0, 7):
+            ref = F.batch_norm(xd, None, None, bn.weight, bn.bias, True, 0.0, 1e-5)
+            assert (y - ref).abs().max().item() < 2e-5
+            mu = xs.mean(dim=(0, 2, 3))
+            var = xs.var(dim=(0, 2, 3), unbiased=False)
+            want = (xs - mu[None, :, None, None]) / torch.sqrt(var + 1e-5)[None, :, None, None] \
+                * gamma.double()[None, :, None, None] + beta.double()[None, :, None, None]
+            assert (y.cpu().double() - want).abs().max().item() < 2e-5
+        if ub == 6:
+            assert _rel(bn.sum, S) < 1e-6 and _rel(bn.sum_squares, Q) < 1e-6
+    mean = S / cnt
+    var = Q / cnt - mean * mean  # biased
+    assert _rel(bn.running_mean, 0.1 * mean) < 1e-6
+    assert _rel(bn.running_var, 0.9 + 0.1 * var) < 1e-6
+    assert (bn.sum == 0).all() and (bn.sum_squares == 0).all() and bn.counter == 0 and bn.tracked == 0
+    assert int(bn.num_batches_tracked) == 1
+
+
+def test_deferred_bn_large_mean_is_stable(device):
+    # |mean| >> std: the shifted sums keep the micro-batch variance accurate
+    x = torch.randn(8, 4, 32, 32, generator=seeded(41)) * 0.01 + 100.0
+    bn = ta.DeferredBatchNorm(4, chunks=1, affine=False).to(device)
+    y = bn(x.to(device)).cpu().double()
+    xs = x.double()
+    want = (xs - xs.mean(dim=(0, 2, 3), keepdim=True)) / torch.sqrt(xs.var(dim=(0, 2, 3), unbiased=False, keepdim=True) + 1e-5)
+    assert (y - want).abs().max().item() < 5e-3  # fp32 input spacing at 100 is 7.6e-6, i.e. 7.6e-4 sigma
+    assert _rel(bn.running_mean, 0.1 * xs.mean(dim=(0, 2, 3))) < 1e-6
+
+
+def test_deferred_bn_backward(device):
+    g = seeded(42)
+    shape = (6, 10, 9, 7)
+    x = _make(shape, 43)
+    dy = torch.randn(shape, generator=g)
+    bn = ta.DeferredBatchNorm(10, chunks=2).to(device)
+    with torch.no_grad():
+        bn.weight.copy_(torch.rand(10, generator=g) + 0.5)
+        bn.bias.copy_(torch.randn(10, generator=g) * 0.1)
+    xd = x.to(device).requires_grad_()
+    bn(xd).backward(dy.to(device))
+    x64 = x.double().requires_grad_()
+    w64 = bn.weight.detach().cpu().double().requires_grad_()
+    b64 = bn.bias.detach().cpu().double().requires_grad_()
+    F.batch_norm(x64, None, None, w64, b64, True, 0.0, 1e-5).backward(dy.double())
+    assert max_rel_to_peak(xd.grad, x64.grad) < 1e-5
+    assert max_rel_to_peak(bn.weight.grad, w64.grad) < 1e-5
+    assert max_rel_to_peak(bn.bias.grad, b64.grad) < 1e-5
+    assert (bn._ws == 0).all()
+
+
+def test_deferred_bn_eval_mode_and_momentum_none(device):
+    g = seeded(44)
+    bn = ta.DeferredBatchNorm(5, momentum=None, chunks=2).to(device)
+    ora = ts_oracle.DeferredBNOracle(5, momentum=None, chunks=2, weight=torch.ones(5, dtype=torch.float64),
+                                     bias=torch.zeros(5, dtype=torch.float64), dtype=torch.float64)
+    for step in range(6):
+        x = _make((4, 5, 6, 6), 60 + step)
+        bn(x.to(device))
+        ora.forward(x.double())
+    assert int(bn.num_batches_tracked) == 3
+    assert _rel(bn.running_mean, ora.running_mean) < 1e-6 and _rel(bn.running_var, ora.running_var) < 1e-6
+    bn.eval()
+    ora.training = False
+    x = _make((3, 5, 4, 4), 70)
+    xd = x.to(device).requires_grad_()
+    y = bn(xd)
+    assert (y.detach().cpu().double() - ora.forward(x.double())).abs().max().item() < 2e-5
+    y.sum().backward()
+    want = (bn.weight.detach() * torch.rsqrt(bn.running_var + bn.eps))[None, :, None, None].expand_as(x).cpu()
+    assert (xd.grad.cpu() - want).abs().max().item() < 1e-5
+    assert bn.tracked == 0 and bn.counter == 0  # eval does not track
+
+
+def test_deferred_bn_module_contract(device):
+    bn = ta.DeferredBatchNorm(4, chunks=2)
+    assert set(bn.state_dict().keys()) == {"weight", "bias", "running_mean", "running_var", "num_batches_tracked",
+                                           "sum", "sum_squares"}
+    with pytest.raises(ValueError):
+        bn.to(device)(torch.zeros(3, 4, device=device))  # 2-D input
+    model = nn.Sequential(nn.Conv2d(3, 4, 3), nn.BatchNorm2d(4), nn.Sequential(nn.BatchNorm2d(4, affine=False)),
+                          nn.BatchNorm2d(4, track_running_stats=False))
+    conv = ta.DeferredBatchNorm.convert_deferred_batch_norm(model, chunks=3)
+    assert isinstance(conv[1], ta.DeferredBatchNorm) and isinstance(conv[2][0], ta.DeferredBatchNorm)
+    assert not isinstance(conv[3], ta.DeferredBatchNorm)  # no running stats: left alone
+    assert conv[1].weight is model[1].weight and conv[1].running_mean is model[1].running_mean
+    assert conv[1].chunks == 3 and conv[2][0].affine is False
+    again = ta.DeferredBatchNorm.convert_deferred_batch_norm(conv[1], chunks=3)
+    assert again is conv[1]
+    conv = conv.to(device)
+    out = conv(torch.randn(2, 3, 8, 8, device=device))
+    assert out.shape == (2, 4, 6, 6)

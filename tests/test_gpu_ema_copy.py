@@ -1,0 +1,158 @@
+"""GPU parity: multi-tensor EMA and multi-segment copy (bit-exact vs the oracle)."""
+import pytest
+import torch
+
+import tspipe_amd as ta
+from helpers import bits_equal, param_lists, seeded
+from oracle import ts_oracle
+from shapes import resnet18_shapes, vit_base_shapes
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("name,shapes,m,seed", [("resnet18", resnet18_shapes(), 0.996, 0),
+                                                ("vit_base", vit_base_shapes(), 0.99, 3)])
+def test_ema_bit_exact(device, name, shapes, m, seed):
+    teacher, student = param_lists(shapes, seed)
+    want = ts_oracle.ema_update(m, student, teacher)
+    t_dev = [t.to(device) for t in teacher]
+    s_dev = [s.to(device) for s in student]
+    got = ta.calculate_target_network_parameters(m, s_dev, t_dev)
+    assert len(got) == len(want)
+    for g, w, t0, s0, td, sd in zip(got, want, teacher, student, t_dev, s_dev):
+        assert g.shape == w.shape and g.dtype == torch.float32 and g.is_cuda
+        assert bits_equal(g, w)
+        assert bits_equal(td, t0) and bits_equal(sd, s0)  # inputs untouched
+        assert g.data_ptr() != td.data_ptr()
+
+
+def test_ema_iterated_100(device):
+    shapes = resnet18_shapes()
+    teacher, student = param_lists(shapes, 0)
+    t_dev = [t.to(device) for t in teacher]
+    s_dev = [s.to(device) for s in student]
+    want = teacher
+    for _ in range(100):
+        t_dev = ta.calculate_target_network_parameters(0.996, s_dev, t_dev)
+        want = ts_oracle.ema_update(0.996, student, want)
+    for g, w in zip(t_dev, want):
+        assert bits_equal(g, w)
+
+
+def test_ema_none_entries_unaligned_views_and_momentum_edges(device):
+    g = seeded(11)
+    base_t = torch.randn(4099, generator=g).to(device)
+    base_s = torch.randn(4099, generator=g).to(device)
+    # views that start 4 and 12 bytes into a 16-byte line, odd lengths
+    t_list = [base_t[1:1001], base_t[1003:1004], base_t[1100:4099], torch.randn(7, 3, generator=g).to(device)]
+    s_list = [base_s[3:1003], None, base_s[1100:4099], torch.randn(7, 3, generator=g).to(device)]
+    got = ta.calculate_updated_momentum_encoder(0.9, s_list, t_list)
+    want = ts_oracle.ema_update(0.9, [None if s is None else s.cpu() for s in s_list], [t.cpu() for t in t_list],
+                                skip_none=True)
+    assert len(got) == 3
+    for a, b in zip(got, want):
+        assert bits_equal(a, b)
+    with pytest.raises(TypeError):
+        ta.calculate_target_network_parameters(0.9, s_list, t_list)
+    pairs_t = [t for t, s in zip(t_list, s_list) if s is not None]
+    pairs_s = [s for s in s_list if s is not None]
+    for a, t in zip(ta.momentum_update(1.0, pairs_s, pairs_t), pairs_t):
+        assert bits_equal(a, t)  # m = 1: teacher unchanged
+    for a, s in zip(ta.momentum_update(0.0, pairs_s, pairs_t), pairs_s):
+        assert bits_equal(a, s)  # m = 0: student copied
+    assert ta.momentum_update(0.5, [], []) == []
+
+
+def test_ema_in_place_form(device):
+    teacher, student = param_lists([(33, 17), (5,), (128, 64, 3, 3)], 5)
+    t_dev = [torch.nn.Parameter(t.to(device)) for t in teacher]
+    s_dev = [torch.nn.Parameter(s.to(device)) for s in student]
+    ptrs = [t.data_ptr() for t in t_dev]
+    ta.update_target_network_parameters_(s_dev, t_dev, 0.99)
+    want = ts_oracle.ema_update(0.99, student, teacher)
+    for t, w, p in zip(t_dev, want, ptrs):
+        assert bits_equal(t, w) and t.data_ptr() == p
+
+
+def test_ema_rejects_bad_inputs(device):
+    a = torch.zeros(8, device=device)
+    with pytest.raises(TypeError):
+        ta.momentum_update(0.9, [a.half()], [a.half()])
+    with pytest.raises(ValueError):
+        ta.momentum_update(0.9, [a], [torch.zeros(9, device=device)])
+    with pytest.raises(TypeError):
+        ta.momentum_update(0.9, [a.cpu()], [a.cpu()])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.int64, torch.uint8, torch.bool])
+def test_gather_bit_exact_dtypes(device, dtype):
+    g = seeded(21)
+    pieces = []
+    for rows in (3, 1, 0, 5):
+        x = torch.randn(rows, 7, 13, generator=g) * 100
+        pieces.append((x > 0) if dtype == torch.bool else x.to(dtype))
+    want = torch.cat(pieces)
+    got = ta.gather([ta.Batch(p.to(device)) for p in pieces])
+    assert bits_equal(got, want)
+
+
+def test_gather_scatter_roundtrip_ragged(device):
+    g = seeded(22)
+    for n, k in [(5, 4), (6, 4), (1, 4), (3, 8), (32, 4), (7, 1), (9, 2)]:
+        x = torch.randn(n, 5, 3, generator=g).to(device)
+        pieces = ta.scatter(x, k)
+        want_sizes = [p.shape[0] for p in x.cpu().chunk(k)]
+        assert [b.tensor.shape[0] for b in pieces] == want_sizes
+        assert pieces[0].tensor.data_ptr() == x.data_ptr()  # views, as in the reference
+        assert bits_equal(ta.gather(pieces), x)
+        owned = ta.scatter_copy(x, k)
+        assert [b.tensor.shape[0] for b in owned] == want_sizes
+        assert all(bits_equal(o.tensor, p.tensor) for o, p in zip(owned, pieces))
+        assert owned[0].tensor.data_ptr() != x.data_ptr()
+
+
+def test_gather_tuple_and_unaligned_segments(device):
+    g = seeded(23)
+    a = torch.randn(10, 3, generator=g).to(device)          # 12-byte rows: pieces start off 16-byte lines
+    b = torch.randint(0, 255, (10, 5), generator=g).to(torch.uint8).to(device)  # 5-byte rows
+    pieces = ta.scatter((a, b), 4)
+    assert all(not p.atomic and len(p) == 2 for p in pieces)
+    got = ta.gather(pieces)
+    assert isinstance(got, tuple) and bits_equal(got[0], a) and bits_equal(got[1], b)
+    # non-contiguous piece and odd byte offsets
+    c = torch.randint(0, 255, (9, 7), generator=g).to(torch.uint8).to(device)
+    parts = [c[0:2], c[2:5, :], c[5:9]]
+    assert bits_equal(ta.gather([ta.Batch(p) for p in parts]), c)
+    t = torch.randn(6, 4, generator=g).to(device)
+    parts = [t.t()[0:2], t.t()[2:4]]  # transposed views: not contiguous
+    assert bits_equal(ta.gather([ta.Batch(p) for p in parts]), torch.cat([p.cpu() for p in parts]))
+
+
+def test_gather_autograd_routes_gradients(device):
+    g = seeded(24)
+    leaves = [torch.randn(r, 4, generator=g).to(device).requires_grad_() for r in (2, 3, 1)]
+    out = ta.gather([ta.Batch(x) for x in leaves])
+    assert out.requires_grad
+    w = torch.randn(6, 4, generator=g).to(device)
+    (out * w).sum().backward()
+    r0 = 0
+    for x in leaves:
+        assert bits_equal(x.grad, w[r0:r0 + x.shape[0]])
+        r0 += x.shape[0]
+
+
+def test_gather_large_cfg3_shape(device):
+    # 4 micro-batches of [8, 128, 30522] bf16 -> [32, 128, 30522]
+    g = seeded(2)
+    pieces = [(torch.randn(8, 128, 30522, generator=g) * 2).to(torch.bfloat16).to(device) for _ in range(4)]
+    got = ta.gather([ta.Batch(p) for p in pieces])
+    assert got.shape == (32, 128, 30522)
+    for i, p in enumerate(pieces):
+        assert torch.equal(got[8 * i:8 * i + 8].view(torch.int16), p.view(torch.int16))
+    back = ta.scatter(got, 4)
+    assert all(torch.equal(b.tensor.view(torch.int16), p.view(torch.int16)) for b, p in zip(back, pieces))
+
+
+def test_gather_rejects_host_tensors():
+    with pytest.raises(TypeError):
+        ta.gather([ta.Batch(torch.zeros(2, 2)), ta.Batch(torch.zeros(2, 2))])

@@ -1,0 +1,228 @@
+"""GPU parity: KD soft target (plain and masked), BYOL and InfoNCE losses against the oracle.
+
+Tolerances.  fp32 inputs: loss and gradient within 1e-5 (relative for the
+loss, max-abs over the gradient's peak for the gradient) of the fp64 oracle.
+bf16 inputs: the oracle is evaluated in fp64 on the same bf16 values; loss
+within 1e-3 relative, gradient within 1e-3 of the gradient's peak plus the
+bf16 rounding of the stored gradient itself (2^-9 relative per element).
+"""
+import pytest
+import torch
+
+import tspipe_amd as ta
+from helpers import max_rel_to_peak, rel_err, seeded
+from oracle import ts_oracle
+
+pytestmark = pytest.mark.gpu
+
+
+def _oracle_grad(fn, *student, others=()):
+    xs = [s.detach().double().requires_grad_() for s in student]
+    loss = fn(*xs, *[o.double() for o in others])
+    loss.backward()
+    return loss.item(), [x.grad for x in xs]
+
+
+def test_kd_cfg2_fp32(device):
+    g = seeded(1)
+    s = torch.randn(256, 100, generator=g) * 3
+    t = torch.randn(256, 100, generator=g) * 3
+    want, (gw,) = _oracle_grad(lambda a, b: ts_oracle.kd_soft_target(a, b, 4.0), s, others=(t,))
+    sd = s.to(device).requires_grad_()
+    loss = ta.SoftTarget(4.0)(sd, t.to(device))
+    loss.backward()
+    assert loss.dtype == torch.float32 and loss.dim() == 0
+    assert rel_err(loss.item(), want) < 1e-5
+    assert max_rel_to_peak(sd.grad, gw) < 1e-5
+    # against the fp32 eager chain too (the reference's own arithmetic)
+    s32 = s.clone().requires_grad_()
+    l32 = ts_oracle.kd_soft_target(s32, t, 4.0)
+    l32.backward()
+    assert rel_err(loss.item(), l32.item()) < 1e-5
+    assert max_rel_to_peak(sd.grad, s32.grad) < 1e-5
+
+
+@pytest.mark.parametrize("rows,V", [(1, 1), (3, 5), (7, 63), (5, 64), (4, 65), (9, 1000), (2, 2049), (3, 4099)])
+def test_kd_shapes_fp32(device, rows, V):
+    g = seeded(100 + V)
+    s = torch.randn(rows, V, generator=g) * 3
+    t = torch.randn(rows, V, generator=g) * 3
+    want, (gw,) = _oracle_grad(lambda a, b: ts_oracle.kd_soft_target(a, b, 2.5), s, others=(t,))
+    sd = s.to(device).requires_grad_()
+    loss = ta.kd_soft_target_loss(sd, t.to(device), 2.5)
+    loss.backward()
+    assert rel_err(loss.item(), want) < 2e-5 or abs(loss.item() - want) < 1e-7
+    assert max_rel_to_peak(sd.grad, gw) < 2e-5 or gw.abs().max() < 1e-12
+
+
+def test_kd_identities(device):
+    g = seeded(7)
+    s = (torch.randn(16, 50, generator=g) * 3).to(device)
+    same = s.clone().requires_grad_()
+    loss = ta.kd_soft_target_loss(same, s, 4.0)
+    loss.backward()
+    assert abs(loss.item()) < 1e-6 and same.grad.abs().max().item() < 1e-7  # s == t
+    t = (torch.randn(16, 50, generator=g) * 3).to(device)
+    a = s.clone().requires_grad_()
+    l1 = ta.kd_soft_target_loss(a, t, 4.0)
+    l1.backward()
+    shift = torch.randn(16, 1, generator=g).to(device) * 10
+    b = (s + shift).requires_grad_()
+    l2 = ta.kd_soft_target_loss(b, t - shift, 4.0)
+    l2.backward()
+    assert rel_err(l2.item(), l1.item()) < 1e-4  # per-row constants cancel
+    assert (a.grad - b.grad).abs().max().item() < 1e-6
+    assert a.grad.sum(dim=1).abs().max().item() < 1e-6  # gradient rows sum to zero
+    assert l1.item() >= 0
+
+
+def test_kd_grad_output_scaling_and_no_grad(device):
+    g = seeded(8)
+    s = (torch.randn(8, 33, generator=g)).to(device)
+    t = (torch.randn(8, 33, generator=g)).to(device)
+    a = s.clone().requires_grad_()
+    ta.kd_soft_target_loss(a, t, 2.0).backward()
+    b = s.clone().requires_grad_()
+    (ta.kd_soft_target_loss(b, t, 2.0) * 3.0).backward()
+    assert torch.allclose(b.grad, 3.0 * a.grad, rtol=1e-6, atol=0)
+    c = s.clone().requires_grad_()
+    ta.kd_soft_target_loss(c, t, 2.0, weight=3.0).backward()
+    assert torch.allclose(c.grad, b.grad, rtol=1e-5, atol=1e-9)
+    with torch.no_grad():
+        l = ta.kd_soft_target_loss(s, t, 2.0)
+    assert not l.requires_grad
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_kd_masked_wide_vocab_half(device, dtype):
+    # DistilBERT-shaped rows (vocab 30522: rows are not 16-byte aligned), fewer rows than cfg3
+    g = seeded(2)
+    bs, seq, V = 4, 32, 30522
+    s = (torch.randn(bs, seq, V, generator=g) * 2).to(dtype)
+    t = (torch.randn(bs, seq, V, generator=g) * 2).to(dtype)
+    mask = torch.rand(bs, seq, generator=g) < 0.15
+    assert 0 < mask.sum().item() < bs * seq
+    want, (gw,) = _oracle_grad(lambda a, b: ts_oracle.distil_ce(a, b, mask, 2.0, 0.5), s, others=(t,))
+    sd = s.to(device).requires_grad_()
+    loss = ta.distil_ce_loss(sd, t.to(device), mask.to(device), 2.0, 0.5)
+    loss.backward()
+    assert rel_err(loss.item(), want) < 1e-3
+    peak = gw.abs().max().item()
+    err = (sd.grad.cpu().double() - gw).abs()
+    assert (err <= 1e-3 * peak + gw.abs() * 2.0 ** -8).all()
+    assert sd.grad.dtype == dtype and sd.grad.shape == s.shape
+    unsel = ~mask
+    assert (sd.grad.cpu()[unsel] == 0).all()  # dense gradient, zero outside the mask
+
+
+def test_kd_mask_special_cases(device):
+    g = seeded(3)
+    s = (torch.randn(2, 6, 40, generator=g) * 2)
+    t = (torch.randn(2, 6, 40, generator=g) * 2)
+    sd, td = s.to(device), t.to(device)
+    full = torch.ones(2, 6, dtype=torch.bool)
+    a = ta.distil_ce_loss(sd, td, full.to(device), 2.0).item()
+    b = ta.kd_soft_target_loss(sd.view(-1, 40), td.view(-1, 40), 2.0).item()
+    assert rel_err(a, b) < 1e-6  # all-true mask == unmasked over all rows
+    one = torch.zeros(2, 6, dtype=torch.bool)
+    one[1, 2] = True
+    want = ts_oracle.distil_ce(s.double(), t.double(), one, 2.0).item()
+    assert rel_err(ta.distil_ce_loss(sd, td, one.to(device), 2.0).item(), want) < 1e-5
+    none = torch.zeros(2, 6, dtype=torch.bool)
+    x = sd.clone().requires_grad_()
+    l = ta.distil_ce_loss(x, td, none.to(device), 2.0)
+    l.backward()
+    assert torch.isnan(l).item() and torch.isnan(ts_oracle.distil_ce(s, t, none, 2.0)).item()  # 0/0 like the reference
+    assert (x.grad == 0).all()
+    # integer attention mask is accepted like a bool one
+    att = torch.tensor([[1, 1, 0, 0, 1, 0], [0, 1, 1, 1, 0, 0]])
+    want = ts_oracle.distil_ce(s.double(), t.double(), att.bool(), 2.0).item()
+    assert rel_err(ta.distil_ce_loss(sd, td, att.to(device), 2.0).item(), want) < 1e-5
+
+
+def test_byol_fp32(device):
+    g = seeded(5)
+    o1, o2, t1, t2 = [torch.randn(256, 128, generator=g) for _ in range(4)]
+    want, (g1, g2) = _oracle_grad(lambda a, b, c, d: ts_oracle.byol_contrastive_loss(a, b, c, d), o1, o2,
+                                  others=(t1, t2))
+    d1, d2 = o1.to(device).requires_grad_(), o2.to(device).requires_grad_()
+    loss = ta.byol_contrastive_loss(d1, d2, t1.to(device), t2.to(device), None, None)
+    loss.backward()
+    assert rel_err(loss.item(), want) < 1e-5
+    assert max_rel_to_peak(d1.grad, g1) < 1e-5 and max_rel_to_peak(d2.grad, g2) < 1e-5
+    # gradient is orthogonal to the input row (normalize Jacobian)
+    assert (d1.grad * d1.detach()).sum(dim=1).abs().max().item() < 1e-7
+
+
+def test_byol_special_cases(device):
+    x = torch.tensor([[3.0, 4.0, 0.0], [0.0, 2.0, 0.0], [1.0, 0.0, 0.0]], device=device)
+    y = torch.stack([x[0] * 2.5, -x[1], torch.tensor([0.0, 0.0, 7.0], device=device)])
+    from tspipe_amd.losses import regression_loss_mean
+    assert abs(regression_loss_mean(x[:1], y[:1]).item() - 0.0) < 1e-6    # parallel
+    assert abs(regression_loss_mean(x[1:2], y[1:2]).item() - 4.0) < 1e-6  # opposite
+    assert abs(regression_loss_mean(x[2:], y[2:]).item() - 2.0) < 1e-6    # orthogonal
+    # odd width, single row, scale invariance
+    g = seeded(6)
+    a, b = torch.randn(3, 37, generator=g).to(device), torch.randn(3, 37, generator=g).to(device)
+    l1 = regression_loss_mean(a, b).item()
+    l2 = regression_loss_mean(a * 7.0, b * 0.25).item()
+    assert rel_err(l2, l1) < 1e-5
+    want = ts_oracle.byol_regression_loss(a.cpu().double(), b.cpu().double()).mean().item()
+    assert rel_err(l1, want) < 1e-5
+
+
+def _nce_inputs(n, c, seed, dtype):
+    g = seeded(seed)
+    q = torch.nn.functional.normalize(torch.randn(n, c, generator=g), dim=1).to(dtype)
+    k = torch.nn.functional.normalize(torch.randn(n, c, generator=g), dim=1).to(dtype)
+    return q, k
+
+
+@pytest.mark.parametrize("n,c", [(4096, 256), (1000, 256), (384, 128), (130, 64), (1, 64), (33, 256)])
+def test_infonce_bf16(device, n, c):
+    q, k = _nce_inputs(n, c, 3, torch.bfloat16)
+    want, (gw,) = _oracle_grad(lambda a, b: ts_oracle.infonce(a, b, 0.2), q, others=(k,))
+    qd = q.to(device).requires_grad_()
+    loss = ta.infonce_loss(qd, k.to(device), 0.2)
+    loss.backward()
+    assert rel_err(loss.item(), want) < 1e-3 or abs(loss.item() - want) < 1e-6
+    peak = gw.abs().max().item()
+    err = (qd.grad.cpu().double() - gw).abs()
+    assert (err <= 1e-3 * peak + gw.abs() * 2.0 ** -8).all() or peak < 1e-9
+
+
+def test_infonce_unnormalised_inputs_and_pair(device):
+    g = seeded(31)
+    o1, o2, t1, t2 = [(torch.randn(512, 256, generator=g) * (0.5 + i)).to(torch.bfloat16) for i in range(4)]
+    want, (g1, g2) = _oracle_grad(lambda a, b, c, d: ts_oracle.moco_contrastive_loss(a, b, c, d, 0.2), o1, o2,
+                                  others=(t1, t2))
+    d1, d2 = o1.to(device).requires_grad_(), o2.to(device).requires_grad_()
+    from argparse import Namespace
+    loss = ta.moco_contrastive_loss(d1, d2, t1.to(device), t2.to(device), None, Namespace(moco_t=0.2))
+    loss.backward()
+    assert rel_err(loss.item(), want) < 1e-3
+    for got, ref in ((d1.grad, g1), (d2.grad, g2)):
+        peak = ref.abs().max().item()
+        assert ((got.cpu().double() - ref).abs() <= 1e-3 * peak + ref.abs() * 2.0 ** -8).all()
+    # rows of dq are orthogonal to q (normalize Jacobian), up to bf16 storage of dq
+    dots = (d1.grad.float() * d1.detach().float()).sum(dim=1).abs().max().item()
+    assert dots < 2e-2 * d1.grad.float().abs().max().item() * d1.detach().float().norm(dim=1).max().item()
+
+
+def test_infonce_fp32_inputs_and_identities(device):
+    q, k = _nce_inputs(256, 128, 9, torch.float32)
+    want, (gw,) = _oracle_grad(lambda a, b: ts_oracle.infonce(a, b, 0.5), q, others=(k,))
+    qd = q.to(device).requires_grad_()
+    loss = ta.infonce_loss(qd, k.to(device), 0.5)
+    loss.backward()
+    # fp32 inputs are rounded to bf16 for the contraction: bf16-level tolerance
+    assert rel_err(loss.item(), want) < 2e-3
+    assert max_rel_to_peak(qd.grad, gw) < 1e-2
+    # N = 1: a single logit, loss 0
+    q1, k1 = _nce_inputs(1, 64, 10, torch.bfloat16)
+    assert abs(ta.infonce_loss(q1.to(device), k1.to(device), 0.2).item()) < 1e-6
+    # scale invariance in q and k
+    qb, kb = _nce_inputs(200, 64, 12, torch.bfloat16)
+    l1 = ta.infonce_loss(qb.to(device), kb.to(device), 0.2).item()
+    l2 = ta.infonce_loss((qb * 4).to(device), (kb * 0.5).to(device), 0.2).item()
+    assert rel_err(l2, l1) < 1e-4

@@ -1,0 +1,16 @@
+"""MI355X-native teacher-student step kernels behind TSPipe's plug-in API.
+
+Importing the package does not touch the GPU or the shared library; the
+library is loaded on the first kernel call (see ``_lib``).
+"""
+from .batch_ops import (Batch, ScatterGatherFn, batch_size, check, defaultScatterGatherFn, gather,
+                        generic_gather, generic_scatter, scatter, scatter_copy)
+from .batchnorm import DeferredBatchNorm
+from .ema import (calculate_target_network_parameters, calculate_updated_momentum_encoder,
+                  momentum_update, update_target_network_parameters_)
+from .losses import (SoftTarget, byol_contrastive_loss, byol_loss, distil_ce_loss, infonce_loss,
+                     kd_soft_target_loss, moco_contrastive_loss, moco_contrastive_loss_pair)
+from .model_wrapper import TSPipeModelOutput, TSPipeModelWrapper
+from .utils import generic_object_gather, generic_object_scatter, traverse_tensor_map
+
+__version__ = "0.1.0"

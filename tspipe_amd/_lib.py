@@ -1,0 +1,104 @@
+"""ctypes binding of libtspipe_amd.so (the C ABI declared in include/tspipe_amd.h).
+
+The library is loaded lazily, once per process, so that the adapters can be
+pickled into spawned worker processes the way TSPipe ships its plug-ins
+(tspipe/gpu_worker.py:596-600).  There is no fallback: if the library is
+missing, every operation raises.
+"""
+import ctypes
+import os
+import threading
+from ctypes import (POINTER, c_char_p, c_double, c_float, c_int, c_int64, c_size_t, c_uint8,
+                    c_void_p)
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libtspipe_amd.so")
+
+TS_F32, TS_BF16, TS_F16 = 0, 1, 2
+
+_lock = threading.Lock()
+_lib = None
+
+# name -> (restype, argtypes); one row per symbol of include/tspipe_amd.h
+SIGNATURES = {
+    "ts_version": (c_char_p, []),
+    "ts_error_string": (c_char_p, [c_int]),
+    "ts_last_hip_error": (c_int, []),
+    "ts_ema_auto_chunk": (c_int64, [c_int64]),
+    "ts_ema_plan": (c_int64, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_int64]),
+    "ts_ema_multi": (c_int, [c_void_p, c_int64, c_float, c_float, c_void_p]),
+    "ts_copy_auto_chunk": (c_int64, [c_int64]),
+    "ts_copy_plan": (c_int64, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_int64]),
+    "ts_copy_segments": (c_int, [c_void_p, c_int64, c_void_p]),
+    "ts_kd_workspace_bytes": (c_size_t, [c_int64]),
+    "ts_kd_fwd_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_float,
+                              c_float, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_void_p]),
+    "ts_scale_rows": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_int, c_void_p]),
+    "ts_byol_fwd_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_void_p,
+                                c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
+    "ts_infonce_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int]),
+    "ts_infonce_fwd_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_float,
+                                   c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
+    "ts_bn_stats": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_void_p,
+                            c_void_p, c_float, c_void_p]),
+    "ts_bn_commit": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_double,
+                             c_double, c_void_p]),
+    "ts_bn_apply": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64,
+                            c_int64, c_int, c_float, c_void_p]),
+    "ts_bn_backward": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                               c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p]),
+}
+
+
+class TSPipeAmdError(RuntimeError):
+    """A C-ABI call returned a negative status."""
+
+
+def lib() -> ctypes.CDLL:
+    """Returns the loaded library, loading it on first use."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is None:
+            if not os.path.exists(LIB_PATH):
+                raise ImportError(
+                    f"{LIB_PATH} is missing: build it with `python -m tspipe_amd.build` "
+                    "(hipcc, gfx950). There is no non-HIP fallback.")
+            # torch brings its own libamdhip64.so.7; importing it first makes
+            # this library bind to the same HIP runtime instance as torch's
+            # allocator and streams.
+            import torch  # noqa: F401
+            handle = ctypes.CDLL(LIB_PATH)
+            for name, (restype, argtypes) in SIGNATURES.items():
+                fn = getattr(handle, name)
+                fn.restype = restype
+                fn.argtypes = argtypes
+            _lib = handle
+    return _lib
+
+
+def check(status: int, what: str) -> int:
+    """Raises on a negative status; returns it otherwise (plans return counts)."""
+    if status < 0:
+        handle = lib()
+        msg = handle.ts_error_string(int(status)).decode()
+        hip = handle.ts_last_hip_error()
+        raise TSPipeAmdError(f"{what}: {msg} (status {status}, last HIP error {hip})")
+    return status
+
+
+def dtype_code(dtype) -> int:
+    import torch
+    if dtype == torch.float32:
+        return TS_F32
+    if dtype == torch.bfloat16:
+        return TS_BF16
+    if dtype == torch.float16:
+        return TS_F16
+    raise TypeError(f"unsupported dtype {dtype}: the kernels take float32, bfloat16 or float16")
+
+
+def current_stream_ptr(device) -> int:
+    import torch
+    return torch.cuda.current_stream(device).cuda_stream

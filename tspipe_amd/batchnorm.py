@@ -1,0 +1,205 @@
+"""DeferredBatchNorm on hand-written gfx950 kernels.
+
+Same module as tspipe/batchnorm.py (class 17-120, converter 122-154): a
+BatchNorm layer that normalises every micro-batch with that micro-batch's own
+statistics but updates ``running_mean`` / ``running_var`` once per mini-batch,
+from per-channel sums accumulated over ``chunks`` micro-batches.
+
+What runs where:
+
+* ``_track`` + the statistics pass of ``F.batch_norm(training=True)`` are one
+  kernel pass over the input (``ts_bn_stats``): it adds the micro-batch's
+  per-channel sum and sum of squares into the ``sum`` / ``sum_squares`` buffers
+  and leaves the micro-batch mean and inverse standard deviation for the
+  normalisation;
+* ``_commit`` is ``ts_bn_commit`` (biased variance, the reference's rounding
+  order, accumulators cleared on the device);
+* the normalisation and its backward are ``ts_bn_apply`` / ``ts_bn_backward``.
+
+State-dict keys, constructor arguments, the ``ValueError`` for inputs below 3-D
+and the converter's sharing of parameters and running buffers are unchanged.
+"""
+from typing import Optional, TypeVar, cast
+
+import torch
+from torch import Tensor, nn
+from torch.nn.modules.batchnorm import _BatchNorm
+
+from . import _lib
+
+__all__ = ["DeferredBatchNorm"]
+
+TModule = TypeVar("TModule", bound=nn.Module)
+
+
+def _ptr(t: Optional[Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _dims(x: Tensor):
+    n, c = int(x.shape[0]), int(x.shape[1])
+    hw = x.numel() // (n * c) if n * c else 0
+    return n, c, hw
+
+
+def _require_fp32_cuda(x: Tensor) -> None:
+    if not x.is_cuda:
+        raise TypeError("DeferredBatchNorm kernels need a device tensor (no host fallback)")
+    if x.dtype != torch.float32:
+        raise TypeError(f"DeferredBatchNorm kernels are fp32 (got {x.dtype})")
+
+
+class _NormalizeFn(torch.autograd.Function):
+    """y = (x - mean) * invstd * weight + bias with the given per-channel
+    statistics.  ``training``: the statistics are the micro-batch's own
+    (``spread`` holds inverse standard deviations, and backward accounts for
+    their dependence on x); otherwise they are the fixed running statistics
+    (``spread`` holds variances, ``eps`` is added on the fly)."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias, mean, spread, ws, training: bool, eps: float):
+        n, c, hw = _dims(x)
+        y = torch.empty_like(x)
+        with torch.cuda.device(x.device):
+            status = _lib.lib().ts_bn_apply(x.data_ptr(), y.data_ptr(), mean.data_ptr(), spread.data_ptr(),
+                                            _ptr(weight), _ptr(bias), n, c, hw, 0 if training else 1, eps,
+                                            _lib.current_stream_ptr(x.device))
+        _lib.check(status, "ts_bn_apply")
+        ctx.save_for_backward(x, weight, mean, spread)
+        ctx.ws = ws
+        ctx.training = training
+        ctx.eps = eps
+        ctx.has_bias = bias is not None
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, weight, mean, spread = ctx.saved_tensors
+        invstd = spread if ctx.training else torch.rsqrt(spread + ctx.eps)
+        n, c, hw = _dims(x)
+        dy = dy.contiguous()
+        dx = torch.empty_like(x)
+        dgamma = torch.empty(c, dtype=torch.float32, device=x.device)
+        dbeta = torch.empty(c, dtype=torch.float32, device=x.device)
+        with torch.cuda.device(x.device):
+            status = _lib.lib().ts_bn_backward(x.data_ptr(), dy.data_ptr(), mean.data_ptr(), invstd.data_ptr(),
+                                               _ptr(weight), dx.data_ptr(), dgamma.data_ptr(), dbeta.data_ptr(),
+                                               ctx.ws.data_ptr(), n, c, hw, 1 if ctx.training else 0,
+                                               _lib.current_stream_ptr(x.device))
+        _lib.check(status, "ts_bn_backward")
+        return (dx, dgamma if weight is not None else None, dbeta if ctx.has_bias else None,
+                None, None, None, None, None)
+
+
+class DeferredBatchNorm(_BatchNorm):
+    """A BatchNorm layer that tracks several micro-batches before it updates
+    its running statistics (tspipe/batchnorm.py:17-120)."""
+
+    sum: Tensor
+    sum_squares: Tensor
+
+    def __init__(self, num_features: int, eps: float = 1e-5, momentum: Optional[float] = 0.1,
+                 affine: bool = True, chunks: int = 1) -> None:
+        super().__init__(num_features, eps, momentum, affine, track_running_stats=True)
+        self.register_buffer("sum", torch.zeros_like(self.running_mean))
+        self.register_buffer("sum_squares", torch.zeros_like(self.running_var))
+        # reduction workspace of the kernels (zero between calls); not part of
+        # the state dict
+        self.register_buffer("_ws", torch.zeros(2 * num_features), persistent=False)
+        self.counter = 0
+        self.tracked = 0
+        self.chunks = chunks
+
+    def _check_input_dim(self, input: Tensor) -> None:
+        if input.dim() <= 2:
+            raise ValueError("expected at least 3D input (got %dD input)" % input.dim())
+
+    def _workspace(self, x: Tensor) -> Tensor:
+        if self._ws.device != x.device or self._ws.numel() != 2 * self.num_features:
+            self._ws = torch.zeros(2 * self.num_features, dtype=torch.float32, device=x.device)
+        return self._ws
+
+    def _stats(self, x: Tensor, accumulate: bool):
+        """One pass over x: micro-batch mean / invstd, optionally ``sum += ...``."""
+        n, c, hw = _dims(x)
+        mean = torch.empty(c, dtype=torch.float32, device=x.device)
+        invstd = torch.empty(c, dtype=torch.float32, device=x.device)
+        with torch.cuda.device(x.device):
+            status = _lib.lib().ts_bn_stats(
+                x.data_ptr(), n, c, hw, self._workspace(x).data_ptr(),
+                self.sum.data_ptr() if accumulate else None,
+                self.sum_squares.data_ptr() if accumulate else None,
+                mean.data_ptr(), invstd.data_ptr(), float(self.eps), _lib.current_stream_ptr(x.device))
+        _lib.check(status, "ts_bn_stats")
+        return mean, invstd
+
+    def _track(self, input: Tensor) -> bool:
+        """Adds a micro-batch to the accumulators (tspipe/batchnorm.py:45-59).
+        Returns True once ``chunks`` micro-batches have been seen."""
+        x = input.detach()
+        _require_fp32_cuda(x)
+        x = x if x.is_contiguous() else x.contiguous()
+        self._last_stats = self._stats(x, accumulate=True)
+        self.counter += input.size().numel() // input.size(1)
+        self.tracked += 1
+        return self.tracked == self.chunks
+
+    def _commit(self) -> None:
+        """Folds the accumulated sums into the running statistics
+        (tspipe/batchnorm.py:61-85)."""
+        dev = self.sum.device
+        with torch.cuda.device(dev):
+            status = _lib.lib().ts_bn_commit(
+                self.sum.data_ptr(), self.sum_squares.data_ptr(), self.running_mean.data_ptr(),
+                self.running_var.data_ptr(), self.num_batches_tracked.data_ptr(), self.num_features,
+                float(self.counter), -1.0 if self.momentum is None else float(self.momentum),
+                _lib.current_stream_ptr(dev))
+        _lib.check(status, "ts_bn_commit")
+        self.counter = 0
+        self.tracked = 0
+
+    def forward(self, input: Tensor) -> Tensor:  # type: ignore[override]
+        self._check_input_dim(input)
+        _require_fp32_cuda(input)
+        if input.size(1) != self.num_features:
+            raise ValueError(f"expected {self.num_features} channels, got {input.size(1)}")
+        x = input if input.is_contiguous() else input.contiguous()
+        weight = self.weight if self.affine else None
+        bias = self.bias if self.affine else None
+
+        if not self.training:
+            # fixed running statistics (tspipe/batchnorm.py:88-99)
+            return _NormalizeFn.apply(x, weight, bias, self.running_mean, self.running_var,
+                                      self._workspace(x), False, float(self.eps))
+
+        if self._track(x):
+            self._commit()
+        mean, invstd = self._last_stats
+        self._last_stats = None
+        return _NormalizeFn.apply(x, weight, bias, mean, invstd, self._workspace(x), True, float(self.eps))
+
+    @classmethod
+    def convert_deferred_batch_norm(cls, module: TModule, chunks: int = 1) -> TModule:
+        """Swaps every BatchNorm that tracks running statistics, at any depth,
+        for a DeferredBatchNorm sharing its parameters and running buffers
+        (tspipe/batchnorm.py:122-154)."""
+        if isinstance(module, DeferredBatchNorm) and module.chunks is chunks:
+            return cast(TModule, module)
+
+        converted: nn.Module = module
+        if isinstance(module, _BatchNorm) and module.track_running_stats:
+            converted = DeferredBatchNorm(module.num_features, module.eps, module.momentum, module.affine, chunks)
+            if module.affine:
+                converted.register_parameter("weight", module.weight)
+                converted.register_parameter("bias", module.bias)
+            for name in ("running_mean", "running_var", "num_batches_tracked"):
+                converted.register_buffer(name, getattr(module, name))
+            if module.running_mean is not None and module.running_mean.device != converted.sum.device:
+                dev = module.running_mean.device
+                converted.sum = converted.sum.to(dev)
+                converted.sum_squares = converted.sum_squares.to(dev)
+                converted._ws = converted._ws.to(dev)
+
+        for name, child in module.named_children():
+            converted.add_module(name, cls.convert_deferred_batch_norm(child, chunks))
+        return cast(TModule, converted)

@@ -1,0 +1,53 @@
+"""Builds libtspipe_amd.so (gfx950) from tspipe_amd/csrc with hipcc.
+
+Run as ``python -m tspipe_amd.build``.  The library is written next to this
+file so it travels with the source tree; nothing is installed.
+"""
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+OBJ_DIR = os.path.join(HERE, "build")
+LIB_PATH = os.path.join(HERE, "libtspipe_amd.so")
+SOURCES = ["misc.cpp", "plan.cpp", "ema_copy.hip", "losses.hip", "bn.hip", "infonce.hip"]
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+# -packed-fp32-ops off: the compiler's automatic v_pk_*_f32 forms are not
+# trusted on this hardware pool.
+DEVICE_FLAGS = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+COMMON_FLAGS = ["-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function", "-x", "hip"]
+
+
+def _compile(src: str) -> str:
+    obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")
+    cmd = [HIPCC, *COMMON_FLAGS, *DEVICE_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    noise = "is not a recognized feature for this target"
+    err = "\n".join(l for l in res.stderr.splitlines() if noise not in l)
+    if res.returncode != 0:
+        raise RuntimeError(f"hipcc failed on {src}:\n{err}")
+    if err.strip():
+        sys.stderr.write(err + "\n")
+    return obj
+
+
+def build(verbose: bool = True) -> str:
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as pool:
+        objs = list(pool.map(_compile, SOURCES))
+    tmp = LIB_PATH + ".tmp"
+    cmd = [HIPCC, "-shared", "-fPIC", "--offload-arch=gfx950", *objs, "-o", tmp]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"link failed:\n{res.stderr}")
+    os.replace(tmp, LIB_PATH)
+    if verbose:
+        print(f"built {LIB_PATH}")
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    build()

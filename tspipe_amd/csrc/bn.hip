@@ -1,0 +1,409 @@
+// DeferredBatchNorm kernels for fp32 [N, C, HW] activations.
+//
+// Work decomposition shared by every per-element kernel here: a workgroup
+// owns one channel c and a slab of consecutive samples n0..n1; inside a
+// sample the channel's HW values are contiguous, so the accesses are 16-byte
+// vectors over runs of HW floats.  gridDim = (slabs, C).
+//
+// Reductions are two-level: registers -> LDS tree inside the workgroup, then
+// one hardware fp32 atomic add per workgroup and quantity into a 2*C float
+// workspace.  The workspace is zero between calls: the small per-channel
+// kernel that consumes it also clears it.
+//
+// Sums are taken about a per-channel shift k_c = x[0, c, 0] (the channel's
+// first value): S' = sum(x - k), Q' = sum((x - k)^2).  The variance
+// Q'/n - (S'/n)^2 then cancels against (mean - k)^2, which is of the order
+// of the variance itself, instead of against mean^2; the raw sums the
+// reference accumulates follow exactly as  sum x = S' + n k  and
+// sum x^2 = Q' + 2 k S' + n k^2.
+#include "common.h"
+
+namespace ts {
+
+constexpr int kBnBlock = 256;
+constexpr int kBnUnroll = 4;
+
+struct PlaneSplit {
+  int64_t head, nvec, tail0;  // scalar head, 16-byte vectors, first tail element
+};
+
+__device__ __forceinline__ PlaneSplit split_plane(const float* p, int64_t HW) {
+  PlaneSplit s;
+  s.head = (int64_t)(((16u - (uint32_t)((uintptr_t)p & 15u)) & 15u) >> 2);
+  if (s.head > HW) s.head = HW;
+  s.nvec = (HW - s.head) >> 2;
+  s.tail0 = s.head + (s.nvec << 2);
+  return s;
+}
+
+// Accumulates (a, b) over the slab's elements of x (and optionally a second
+// tensor y with the same layout) through a functor: f(xv, yv, a, b).
+template <bool TWO, typename F>
+__device__ __forceinline__ void slab_reduce(const float* __restrict__ x, const float* __restrict__ y,
+                                            int64_t n0, int64_t n1, int64_t C, int64_t c, int64_t HW,
+                                            float& a, float& b, F f) {
+  const int tid = threadIdx.x;
+  for (int64_t n = n0; n < n1; ++n) {
+    const int64_t off = (n * C + c) * HW;
+    const float* px = x + off;
+    const float* py = TWO ? y + off : nullptr;
+    const PlaneSplit sp = split_plane(px, HW);
+    const bool yvec = !TWO || ((((uintptr_t)py) & 15u) == (((uintptr_t)px) & 15u));
+    if (tid < sp.head) f(px[tid], TWO ? py[tid] : 0.f, a, b);
+    const f32x4* px4 = reinterpret_cast<const f32x4*>(px + sp.head);
+    const f32x4* py4 = reinterpret_cast<const f32x4*>(py + sp.head);
+    for (int64_t base = 0; base < sp.nvec; base += kBnBlock * kBnUnroll) {
+      f32x4 vx[kBnUnroll], vy[kBnUnroll];
+#pragma unroll
+      for (int u = 0; u < kBnUnroll; ++u) {
+        const int64_t i = base + u * kBnBlock + tid;
+        if (i < sp.nvec) {
+          vx[u] = px4[i];
+          if (TWO) {
+            if (yvec) {
+              vy[u] = py4[i];
+            } else {
+              const float* q = py + sp.head + (i << 2);
+              vy[u] = f32x4{q[0], q[1], q[2], q[3]};
+            }
+          }
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < kBnUnroll; ++u) {
+        const int64_t i = base + u * kBnBlock + tid;
+        if (i < sp.nvec) {
+          f(vx[u].x, TWO ? vy[u].x : 0.f, a, b);
+          f(vx[u].y, TWO ? vy[u].y : 0.f, a, b);
+          f(vx[u].z, TWO ? vy[u].z : 0.f, a, b);
+          f(vx[u].w, TWO ? vy[u].w : 0.f, a, b);
+        }
+      }
+    }
+    const int64_t it = sp.tail0 + tid;
+    if (it < HW) f(px[it], TWO ? py[it] : 0.f, a, b);
+  }
+}
+
+__global__ __launch_bounds__(kBnBlock) void bn_stats_kernel(const float* __restrict__ x, int64_t N,
+                                                            int64_t C, int64_t HW, int64_t slab,
+                                                            float* __restrict__ ws) {
+  __shared__ float lds[kBnBlock / kWave];
+  const int64_t c = blockIdx.y;
+  const int64_t n0 = (int64_t)blockIdx.x * slab;
+  const int64_t n1 = (n0 + slab < N) ? n0 + slab : N;
+  const float k = x[c * HW];  // shift: first value of the channel
+  float S = 0.f, Q = 0.f;
+  slab_reduce<false>(x, nullptr, n0, n1, C, c, HW, S, Q, [k](float xv, float, float& a, float& b) {
+    const float d = xv - k;
+    a += d;
+    b += d * d;
+  });
+  S = block_sum<kBnBlock / kWave>(S, lds);
+  Q = block_sum<kBnBlock / kWave>(Q, lds);
+  if (threadIdx.x == 0) {
+    unsafeAtomicAdd(ws + c, S);
+    unsafeAtomicAdd(ws + C + c, Q);
+  }
+}
+
+// One thread per channel: consumes and clears the workspace.
+__global__ __launch_bounds__(256) void bn_stats_finalize_kernel(const float* __restrict__ x, int64_t C,
+                                                                int64_t HW, float cnt,
+                                                                float* __restrict__ ws, float* sum,
+                                                                float* sum_squares, float* ub_mean,
+                                                                float* ub_invstd, float eps) {
+  const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (c >= C) return;
+  const float S = ws[c], Q = ws[C + c];
+  ws[c] = 0.f;
+  ws[C + c] = 0.f;
+  const float k = x[c * HW];
+  if (sum) sum[c] += S + cnt * k;
+  if (sum_squares) sum_squares[c] += Q + 2.f * k * S + cnt * k * k;
+  const float dm = S / cnt;  // mean - k
+  if (ub_mean) ub_mean[c] = k + dm;
+  if (ub_invstd) ub_invstd[c] = 1.f / sqrtf(fmaxf(Q / cnt - dm * dm, 0.f) + eps);
+}
+
+// The reference's rounding order, one fp32 operation at a time:
+//   mean = sum / counter;  var = sum_squares / counter - mean**2
+//   running *= (1 - f);  running += stat * f
+__global__ __launch_bounds__(256) void bn_commit_kernel(float* __restrict__ sum, float* __restrict__ sum_squares,
+                                                        float* __restrict__ running_mean,
+                                                        float* __restrict__ running_var,
+                                                        int64_t* __restrict__ nbt, int64_t C, float counter,
+                                                        double momentum) {
+  const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  // every thread reads the counter before thread 0 of block 0 bumps it: the
+  // value used is "after the increment", computed locally
+  const int64_t tracked = nbt ? *nbt + 1 : 1;
+  const double f = (momentum < 0.0) ? 1.0 / (double)tracked : momentum;
+  const float f32 = (float)f, omf32 = (float)(1.0 - f);
+  if (c < C) {
+    const float mean = __fdiv_rn(sum[c], counter);
+    const float var = __fsub_rn(__fdiv_rn(sum_squares[c], counter), __fmul_rn(mean, mean));
+    running_mean[c] = __fadd_rn(__fmul_rn(running_mean[c], omf32), __fmul_rn(mean, f32));
+    running_var[c] = __fadd_rn(__fmul_rn(running_var[c], omf32), __fmul_rn(var, f32));
+    sum[c] = 0.f;
+    sum_squares[c] = 0.f;
+  }
+}
+
+__global__ void bn_bump_counter_kernel(int64_t* nbt) { *nbt += 1; }
+
+__global__ __launch_bounds__(kBnBlock) void bn_apply_kernel(const float* __restrict__ x, float* __restrict__ y,
+                                                            const float* __restrict__ mean,
+                                                            const float* __restrict__ invstd_or_var,
+                                                            const float* __restrict__ gamma,
+                                                            const float* __restrict__ beta, int64_t N,
+                                                            int64_t C, int64_t HW, int64_t slab, int is_var,
+                                                            float eps) {
+  const int64_t c = blockIdx.y;
+  const int64_t n0 = (int64_t)blockIdx.x * slab;
+  const int64_t n1 = (n0 + slab < N) ? n0 + slab : N;
+  const float mu = mean[c];
+  const float istd = is_var ? 1.f / sqrtf(invstd_or_var[c] + eps) : invstd_or_var[c];
+  const float a = gamma ? istd * gamma[c] : istd;
+  const float b = beta ? beta[c] : 0.f;
+  const int tid = threadIdx.x;
+  for (int64_t n = n0; n < n1; ++n) {
+    const int64_t off = (n * C + c) * HW;
+    const float* px = x + off;
+    float* py = y + off;
+    const PlaneSplit sp = split_plane(px, HW);
+    const bool yvec = (((uintptr_t)py) & 15u) == (((uintptr_t)px) & 15u);
+    if (tid < sp.head) py[tid] = (px[tid] - mu) * a + b;
+    const f32x4* px4 = reinterpret_cast<const f32x4*>(px + sp.head);
+    f32x4* py4 = reinterpret_cast<f32x4*>(py + sp.head);
+    for (int64_t base = 0; base < sp.nvec; base += kBnBlock * kBnUnroll) {
+      f32x4 v[kBnUnroll];
+#pragma unroll
+      for (int u = 0; u < kBnUnroll; ++u) {
+        const int64_t i = base + u * kBnBlock + tid;
+        if (i < sp.nvec) v[u] = px4[i];
+      }
+#pragma unroll
+      for (int u = 0; u < kBnUnroll; ++u) {
+        const int64_t i = base + u * kBnBlock + tid;
+        if (i < sp.nvec) {
+          f32x4 r;
+          r.x = (v[u].x - mu) * a + b;
+          r.y = (v[u].y - mu) * a + b;
+          r.z = (v[u].z - mu) * a + b;
+          r.w = (v[u].w - mu) * a + b;
+          if (yvec) {
+            __builtin_nontemporal_store(r, py4 + i);
+          } else {
+            float* q = py + sp.head + (i << 2);
+            q[0] = r.x;
+            q[1] = r.y;
+            q[2] = r.z;
+            q[3] = r.w;
+          }
+        }
+      }
+    }
+    const int64_t it = sp.tail0 + tid;
+    if (it < HW) py[it] = (px[it] - mu) * a + b;
+  }
+}
+
+// Backward, level 1: per-channel sum(dy) and sum(dy * xhat) into ws.
+__global__ __launch_bounds__(kBnBlock) void bn_bwd_reduce_kernel(const float* __restrict__ x,
+                                                                 const float* __restrict__ dy,
+                                                                 const float* __restrict__ mean,
+                                                                 const float* __restrict__ invstd, int64_t N,
+                                                                 int64_t C, int64_t HW, int64_t slab,
+                                                                 float* __restrict__ ws) {
+  __shared__ float lds[kBnBlock / kWave];
+  const int64_t c = blockIdx.y;
+  const int64_t n0 = (int64_t)blockIdx.x * slab;
+  const int64_t n1 = (n0 + slab < N) ? n0 + slab : N;
+  const float mu = mean[c], istd = invstd[c];
+  float sdy = 0.f, sdyx = 0.f;
+  slab_reduce<true>(x, dy, n0, n1, C, c, HW, sdy, sdyx, [mu, istd](float xv, float g, float& a, float& b) {
+    a += g;
+    b += g * ((xv - mu) * istd);
+  });
+  sdy = block_sum<kBnBlock / kWave>(sdy, lds);
+  sdyx = block_sum<kBnBlock / kWave>(sdyx, lds);
+  if (threadIdx.x == 0) {
+    unsafeAtomicAdd(ws + c, sdy);
+    unsafeAtomicAdd(ws + C + c, sdyx);
+  }
+}
+
+__global__ __launch_bounds__(256) void bn_bwd_finalize_kernel(int64_t C, float* __restrict__ ws,
+                                                              float* __restrict__ dgamma,
+                                                              float* __restrict__ dbeta) {
+  const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (c >= C) return;
+  dbeta[c] = ws[c];
+  dgamma[c] = ws[C + c];
+  ws[c] = 0.f;
+  ws[C + c] = 0.f;
+}
+
+// Backward, level 2: dx = gamma*invstd*(dy - dbeta/cnt - xhat*dgamma/cnt).
+__global__ __launch_bounds__(kBnBlock) void bn_bwd_dx_kernel(const float* __restrict__ x,
+                                                             const float* __restrict__ dy,
+                                                             const float* __restrict__ mean,
+                                                             const float* __restrict__ invstd,
+                                                             const float* __restrict__ gamma,
+                                                             const float* __restrict__ dgamma,
+                                                             const float* __restrict__ dbeta,
+                                                             float* __restrict__ dx, int64_t N, int64_t C,
+                                                             int64_t HW, int64_t slab, float inv_cnt /* 0: fixed statistics */) {
+  const int64_t c = blockIdx.y;
+  const int64_t n0 = (int64_t)blockIdx.x * slab;
+  const int64_t n1 = (n0 + slab < N) ? n0 + slab : N;
+  const float mu = mean[c], istd = invstd[c];
+  const float gi = (gamma ? gamma[c] : 1.f) * istd;
+  const float mb = dbeta[c] * inv_cnt, mg = dgamma[c] * inv_cnt;
+  const int tid = threadIdx.x;
+  auto one = [=](float xv, float g) { return gi * (g - mb - ((xv - mu) * istd) * mg); };
+  for (int64_t n = n0; n < n1; ++n) {
+    const int64_t off = (n * C + c) * HW;
+    const float* px = x + off;
+    const float* pg = dy + off;
+    float* pd = dx + off;
+    const PlaneSplit sp = split_plane(px, HW);
+    const bool vec = ((((uintptr_t)pg) & 15u) == (((uintptr_t)px) & 15u)) &&
+                     ((((uintptr_t)pd) & 15u) == (((uintptr_t)px) & 15u));
+    if (!vec) {
+      for (int64_t i = tid; i < HW; i += kBnBlock) pd[i] = one(px[i], pg[i]);
+      continue;
+    }
+    if (tid < sp.head) pd[tid] = one(px[tid], pg[tid]);
+    const f32x4* px4 = reinterpret_cast<const f32x4*>(px + sp.head);
+    const f32x4* pg4 = reinterpret_cast<const f32x4*>(pg + sp.head);
+    f32x4* pd4 = reinterpret_cast<f32x4*>(pd + sp.head);
+    for (int64_t base = 0; base < sp.nvec; base += kBnBlock * kBnUnroll) {
+      f32x4 vx[kBnUnroll], vg[kBnUnroll];
+#pragma unroll
+      for (int u = 0; u < kBnUnroll; ++u) {
+        const int64_t i = base + u * kBnBlock + tid;
+        if (i < sp.nvec) {
+          vx[u] = px4[i];
+          vg[u] = pg4[i];
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < kBnUnroll; ++u) {
+        const int64_t i = base + u * kBnBlock + tid;
+        if (i < sp.nvec) {
+          f32x4 r;
+          r.x = one(vx[u].x, vg[u].x);
+          r.y = one(vx[u].y, vg[u].y);
+          r.z = one(vx[u].z, vg[u].z);
+          r.w = one(vx[u].w, vg[u].w);
+          __builtin_nontemporal_store(r, pd4 + i);
+        }
+      }
+    }
+    const int64_t it = sp.tail0 + tid;
+    if (it < HW) pd[it] = one(px[it], pg[it]);
+  }
+}
+
+// Samples per workgroup: about 8K elements each, so small feature maps do
+// not degenerate into one workgroup per few hundred bytes.
+inline int64_t bn_slab(int64_t N, int64_t HW) {
+  int64_t s = (8192 + HW - 1) / HW;
+  if (s < 1) s = 1;
+  if (s > N) s = N;
+  return s;
+}
+
+inline int bn_check_dims(int64_t N, int64_t C, int64_t HW) {
+  if (N <= 0 || C <= 0 || HW <= 0) return TS_ERR_ARG;
+  if (C > 65535) return TS_ERR_RANGE;  // gridDim.y
+  if (N > 0x7fffffffLL) return TS_ERR_RANGE;
+  return TS_OK;
+}
+
+}  // namespace ts
+
+extern "C" {
+
+int ts_bn_stats(const float* x, int64_t N, int64_t C, int64_t HW, float* ws, float* sum,
+                float* sum_squares, float* ub_mean, float* ub_invstd, float eps, ts_stream_t stream) {
+  if (!x || !ws) return TS_ERR_ARG;
+  if ((ub_mean == nullptr) != (ub_invstd == nullptr)) return TS_ERR_ARG;
+  if ((sum == nullptr) != (sum_squares == nullptr)) return TS_ERR_ARG;
+  int rc = ts::bn_check_dims(N, C, HW);
+  if (rc) return rc;
+  if ((uintptr_t)x & 3u) return TS_ERR_ALIGN;
+  const int64_t slab = ts::bn_slab(N, HW);
+  dim3 grid((unsigned)((N + slab - 1) / slab), (unsigned)C);
+  hipStream_t st = (hipStream_t)stream;
+  hipLaunchKernelGGL(ts::bn_stats_kernel, grid, dim3(ts::kBnBlock), 0, st, x, N, C, HW, slab, ws);
+  rc = ts::check_launch();
+  if (rc) return rc;
+  hipLaunchKernelGGL(ts::bn_stats_finalize_kernel, dim3((unsigned)((C + 255) / 256)), dim3(256), 0, st,
+                     x, C, HW, (float)((double)N * (double)HW), ws, sum, sum_squares, ub_mean, ub_invstd,
+                     eps);
+  return ts::check_launch();
+}
+
+int ts_bn_commit(float* sum, float* sum_squares, float* running_mean, float* running_var,
+                 int64_t* num_batches_tracked, int64_t C, double counter, double momentum,
+                 ts_stream_t stream) {
+  if (!sum || !sum_squares || !running_mean || !running_var) return TS_ERR_ARG;
+  if (C <= 0) return TS_ERR_ARG;
+  if (momentum < 0.0 && !num_batches_tracked) return TS_ERR_ARG;
+  hipStream_t st = (hipStream_t)stream;
+  hipLaunchKernelGGL(ts::bn_commit_kernel, dim3((unsigned)((C + 255) / 256)), dim3(256), 0, st, sum,
+                     sum_squares, running_mean, running_var, num_batches_tracked, C, (float)counter,
+                     momentum);
+  int rc = ts::check_launch();
+  if (rc) return rc;
+  if (num_batches_tracked) {
+    // after the commit kernel on the same stream, so every workgroup of it
+    // saw the old value
+    hipLaunchKernelGGL(ts::bn_bump_counter_kernel, dim3(1), dim3(1), 0, st, num_batches_tracked);
+    rc = ts::check_launch();
+  }
+  return rc;
+}
+
+int ts_bn_apply(const float* x, float* y, const float* mean, const float* invstd_or_var,
+                const float* gamma, const float* beta, int64_t N, int64_t C, int64_t HW, int is_var,
+                float eps, ts_stream_t stream) {
+  if (!x || !y || !mean || !invstd_or_var) return TS_ERR_ARG;
+  int rc = ts::bn_check_dims(N, C, HW);
+  if (rc) return rc;
+  if (((uintptr_t)x | (uintptr_t)y) & 3u) return TS_ERR_ALIGN;
+  const int64_t slab = ts::bn_slab(N, HW);
+  dim3 grid((unsigned)((N + slab - 1) / slab), (unsigned)C);
+  hipLaunchKernelGGL(ts::bn_apply_kernel, grid, dim3(ts::kBnBlock), 0, (hipStream_t)stream, x, y, mean,
+                     invstd_or_var, gamma, beta, N, C, HW, slab, is_var, eps);
+  return ts::check_launch();
+}
+
+int ts_bn_backward(const float* x, const float* dy, const float* ub_mean, const float* ub_invstd,
+                   const float* gamma, float* dx, float* dgamma, float* dbeta, float* ws, int64_t N,
+                   int64_t C, int64_t HW, int training, ts_stream_t stream) {
+  if (!x || !dy || !ub_mean || !ub_invstd || !dx || !dgamma || !dbeta || !ws) return TS_ERR_ARG;
+  int rc = ts::bn_check_dims(N, C, HW);
+  if (rc) return rc;
+  if (((uintptr_t)x | (uintptr_t)dy | (uintptr_t)dx) & 3u) return TS_ERR_ALIGN;
+  const int64_t slab = ts::bn_slab(N, HW);
+  dim3 grid((unsigned)((N + slab - 1) / slab), (unsigned)C);
+  hipStream_t st = (hipStream_t)stream;
+  hipLaunchKernelGGL(ts::bn_bwd_reduce_kernel, grid, dim3(ts::kBnBlock), 0, st, x, dy, ub_mean, ub_invstd,
+                     N, C, HW, slab, ws);
+  rc = ts::check_launch();
+  if (rc) return rc;
+  hipLaunchKernelGGL(ts::bn_bwd_finalize_kernel, dim3((unsigned)((C + 255) / 256)), dim3(256), 0, st, C,
+                     ws, dgamma, dbeta);
+  rc = ts::check_launch();
+  if (rc) return rc;
+  hipLaunchKernelGGL(ts::bn_bwd_dx_kernel, grid, dim3(ts::kBnBlock), 0, st, x, dy, ub_mean, ub_invstd,
+                     gamma, dgamma, dbeta, dx, N, C, HW, slab,
+                     training ? (float)(1.0 / ((double)N * (double)HW)) : 0.f);
+  return ts::check_launch();
+}
+
+}  // extern "C"

@@ -1,0 +1,103 @@
+// Shared device helpers for the gfx950 kernels: 64-wide wavefront reductions,
+// 16-byte vector types, dtype conversion, launch-error bookkeeping.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/tspipe_amd.h"
+
+namespace ts {
+
+constexpr int kWave = 64;  // CDNA wavefront width
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint16_t u16x8 __attribute__((ext_vector_type(8)));
+
+// Records the HIP error of a failed launch for ts_last_hip_error().
+void set_last_hip_error(int code);
+
+inline int check_launch() {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    set_last_hip_error((int)e);
+    return TS_ERR_LAUNCH;
+  }
+  return TS_OK;
+}
+
+// ---- dtype conversion (storage type <-> fp32) ---------------------------
+
+struct bf16_t {
+  uint16_t bits;
+};
+struct f16_t {
+  _Float16 v;
+};
+
+__device__ __forceinline__ float to_f32(float x) { return x; }
+__device__ __forceinline__ float to_f32(bf16_t x) { return __uint_as_float((uint32_t)x.bits << 16); }
+__device__ __forceinline__ float to_f32(f16_t x) { return (float)x.v; }
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t bits) { return __uint_as_float(bits << 16); }
+
+// Round-to-nearest-even fp32 -> bf16, NaN kept quiet (what torch's cast does).
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+template <typename T>
+__device__ __forceinline__ T from_f32(float x);
+template <>
+__device__ __forceinline__ float from_f32<float>(float x) {
+  return x;
+}
+template <>
+__device__ __forceinline__ bf16_t from_f32<bf16_t>(float x) {
+  bf16_t r;
+  r.bits = f32_to_bf16_bits(x);
+  return r;
+}
+template <>
+__device__ __forceinline__ f16_t from_f32<f16_t>(float x) {
+  f16_t r;
+  r.v = (_Float16)x;
+  return r;
+}
+
+// ---- wavefront / block reductions -----------------------------------------
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+  return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int off = kWave / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
+  return v;
+}
+
+// Sum over a block of NWAVES wavefronts; every thread gets the result.
+// `lds` must hold NWAVES floats and may be reused after the call returns.
+template <int NWAVES>
+__device__ __forceinline__ float block_sum(float v, float* lds) {
+  v = wave_sum(v);
+  if (NWAVES == 1) return v;
+  const int lane = threadIdx.x & (kWave - 1), w = threadIdx.x / kWave;
+  __syncthreads();
+  if (lane == 0) lds[w] = v;
+  __syncthreads();
+  float r = 0.f;
+#pragma unroll
+  for (int i = 0; i < NWAVES; ++i) r += lds[i];
+  return r;
+}
+
+}  // namespace ts

@@ -1,0 +1,475 @@
+// MoCo-v3 InfoNCE loss, forward and backward fused, on bf16 MFMA.
+//
+//   qh = q/|q|, kh = k/|k|, logits = qh kh^T / tau,
+//   loss = 2 tau * mean_i( lse_i - logits_ii ),
+//   dqh_i = (2/N) (sum_j P_ij kh_j - kh_i),  P = softmax(logits) row-wise,
+//   dq_i  = (dqh_i - qh_i <qh_i, dqh_i>) / |q_i|.
+//
+// sum_j P_ij kh_j is an attention product with V = K, so the kernel is a
+// flash-attention forward: the N x N logits are never stored.  Two facts make
+// it simpler than the general case:
+//   * |logit| <= 1/tau because the rows are unit vectors, so the soft-max
+//     uses the fixed reference point x_max = log2(e)/tau instead of a running
+//     maximum: no rescaling of the accumulators, and partial results of
+//     different key ranges just add up;
+//   * the normalisation is applied as fp32 factors after the bf16 contraction
+//     (logit_ij = <q_i,k_j> * rq_i * rk_j / tau), so the raw bf16 inputs feed
+//     the MFMA and no rounded copy of qh / kh is ever made.
+//
+// Kernels:
+//   prep     per row: rq = 1/max(|q|,eps), rk, the diagonal logit, and K^T
+//            (bf16, [C][Npad]) so that the second contraction can read keys
+//            contiguously; fp32 inputs are also rounded to bf16 copies here.
+//   main     grid (q tile of 128 rows, key split, pair); 4 wavefronts, each
+//            owning 32 q rows; per 32-key tile: S^T = K Q^T (MFMA 32x32x16),
+//            P = 2^(S*scale - x_max), l += P, O^T += K^T (P*rk) (MFMA).
+//            Writes per-split partial l and O^T in register-native order.
+//   combine  per 32-row q tile: adds the splits, forms loss rows and dq.
+//
+// MFMA 32x32x16 operand layout used throughout (lane l, half h = l/32):
+//   A: row l%32, contraction slots 8h..8h+7;  B: column l%32, same slots;
+//   D[i]: row (i%4) + 4h + 8(i/4), column l%32.
+#include "common.h"
+
+namespace ts {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+constexpr float kNceLog2e = 1.4426950408889634f;
+constexpr float kNceLn2 = 0.6931471805599453f;
+constexpr float kNormEps = 1e-12f;  // F.normalize's eps
+constexpr int kQTile = 128;         // q rows per workgroup (32 per wavefront)
+constexpr int kKTile = 32;          // keys per inner iteration
+constexpr int kNceBlock = 256;
+
+// defined in losses.hip
+int launch_sum_scale(const float* v, int64_t n, float scale, float denom, float* out, hipStream_t stream);
+
+__host__ __device__ inline int64_t nce_round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
+
+// Workspace carve-up (all offsets multiples of 256 bytes): a head with the
+// loss rows of every pair, [pairs][npad] floats, then one region per pair.
+struct NceLayout {
+  int64_t npad;
+  int splits;
+  size_t head_bytes;
+  size_t off_rq, off_rk, off_diag, off_lpart, off_kt, off_qb, off_kb, off_opart, pair_bytes;
+};
+
+inline size_t nce_align(size_t x) { return (x + 255) & ~(size_t)255; }
+
+inline int nce_splits(int64_t npad, int n_pairs) {
+  const int64_t qtiles = npad / kQTile * n_pairs;
+  const int64_t ktiles = npad / kKTile;
+  int64_t s = (512 + qtiles - 1) / qtiles;  // aim for ~2 workgroups per CU
+  if (s > 16) s = 16;
+  if (s > ktiles) s = ktiles;
+  if (s < 1) s = 1;
+  return (int)s;
+}
+
+inline NceLayout nce_layout(int64_t n, int64_t c, int n_pairs, bool fp32_in) {
+  NceLayout L;
+  L.npad = nce_round_up(n > 0 ? n : 1, kQTile);
+  L.splits = nce_splits(L.npad, n_pairs);
+  L.head_bytes = nce_align((size_t)n_pairs * L.npad * 4);
+  size_t o = 0;
+  L.off_rq = o;       o += nce_align(L.npad * 4);
+  L.off_rk = o;       o += nce_align(L.npad * 4);
+  L.off_diag = o;     o += nce_align(L.npad * 4);
+  L.off_lpart = o;    o += nce_align((size_t)L.splits * L.npad * 4);
+  L.off_kt = o;       o += nce_align((size_t)c * L.npad * 2);
+  L.off_qb = o;       o += fp32_in ? nce_align((size_t)L.npad * c * 2) : 0;
+  L.off_kb = o;       o += fp32_in ? nce_align((size_t)L.npad * c * 2) : 0;
+  L.off_opart = o;    o += nce_align((size_t)L.splits * L.npad * c * 4);
+  L.pair_bytes = o;
+  return L;
+}
+
+// ---------------------------------------------------------------------------
+// prep: 64 rows per workgroup
+// ---------------------------------------------------------------------------
+template <typename T, int C>
+__global__ __launch_bounds__(kNceBlock) void nce_prep_kernel(const T* __restrict__ q, const T* __restrict__ k,
+                                                             int64_t n, int64_t npad, float scale2,
+                                                             float* __restrict__ rq, float* __restrict__ rk,
+                                                             float* __restrict__ diag, uint16_t* __restrict__ kt,
+                                                             uint16_t* __restrict__ qb, uint16_t* __restrict__ kb) {
+  constexpr int ROWS = 64;
+  constexpr int LD = C + 2;  // odd number of 4-byte words per row: column reads spread over banks
+  __shared__ uint16_t tile[ROWS * LD];
+  const int lane = threadIdx.x % kWave, w = threadIdx.x / kWave;
+  const int64_t row0 = (int64_t)blockIdx.x * ROWS;
+
+  for (int r = w; r < ROWS; r += kNceBlock / kWave) {
+    const int64_t row = row0 + r;
+    float sqq = 0.f, skk = 0.f, sqk = 0.f;
+    for (int f = lane; f < C; f += kWave) {
+      float qv = 0.f, kv = 0.f;
+      if (row < n) {
+        qv = to_f32(q[row * C + f]);
+        kv = to_f32(k[row * C + f]);
+      }
+      const uint16_t qbits = f32_to_bf16_bits(qv), kbits = f32_to_bf16_bits(kv);
+      sqq += qv * qv;
+      skk += kv * kv;
+      // the diagonal logit uses the values the MFMA will see
+      sqk += bf16_bits_to_f32(qbits) * bf16_bits_to_f32(kbits);
+      tile[r * LD + f] = kbits;
+      if (qb) {
+        qb[row * C + f] = qbits;
+        kb[row * C + f] = kbits;
+      }
+    }
+    sqq = wave_sum(sqq);
+    skk = wave_sum(skk);
+    sqk = wave_sum(sqk);
+    if (lane == 0) {
+      const bool live = row < n;
+      const float a = live ? 1.f / fmaxf(sqrtf(sqq), kNormEps) : 0.f;
+      const float b = live ? 1.f / fmaxf(sqrtf(skk), kNormEps) : 0.f;
+      rq[row] = a;
+      rk[row] = b;
+      diag[row] = sqk * a * b * scale2;
+    }
+  }
+  __syncthreads();
+  // transposed write: K^T[f][row0 + 8*chunk .. +7], 16 bytes per store
+  for (int id = threadIdx.x; id < C * (ROWS / 8); id += kNceBlock) {
+    const int f = id / (ROWS / 8), chunk = id % (ROWS / 8);
+    u16x8 v;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = tile[(chunk * 8 + e) * LD + f];
+    *reinterpret_cast<u16x8*>(kt + (int64_t)f * npad + row0 + chunk * 8) = v;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// main
+// ---------------------------------------------------------------------------
+template <int C>
+struct NceSmem {
+  static constexpr int KLD = C + 8;       // bf16 per K-tile row (16-byte pad: rows start on different banks)
+  static constexpr int TLD = kKTile + 8;  // bf16 per K^T-tile row (80 bytes, keeps 16-byte alignment)
+  uint16_t k[2][kKTile * KLD];
+  uint16_t kt[2][C * TLD];
+  float rk[2][kKTile];
+};
+
+template <int C>
+__global__ __launch_bounds__(kNceBlock) void nce_main_kernel(const uint16_t* __restrict__ qg,
+                                                             const uint16_t* __restrict__ kg,
+                                                             const uint16_t* __restrict__ ktg,
+                                                             const float* __restrict__ rq,
+                                                             const float* __restrict__ rk, int64_t n, int64_t npad,
+                                                             int splits, float scale2 /* log2(e)/tau */,
+                                                             float* __restrict__ lpart, float* __restrict__ opart) {
+  using Smem = NceSmem<C>;
+  __shared__ __attribute__((aligned(16))) Smem sm;
+  constexpr int KK = C / 16;  // contraction steps of S^T
+  constexpr int FB = C / 32;  // feature blocks of O^T
+  const int tid = threadIdx.x, lane = tid % kWave, w = tid / kWave;
+  const int col = lane % 32, h = lane / 32;
+  const int64_t qtile = blockIdx.x;
+  const int split = blockIdx.y;
+  const int64_t qrow = qtile * kQTile + w * 32 + col;  // the q row this lane is a column of
+
+  const int64_t ktiles = npad / kKTile;
+  const int64_t t0 = ktiles * split / splits, t1 = ktiles * (split + 1) / splits;
+
+  // Q fragments: B operand of S^T, resident for the whole kernel.
+  bf16x8 qf[KK];
+#pragma unroll
+  for (int kk = 0; kk < KK; ++kk) {
+    u32x4 raw = {0u, 0u, 0u, 0u};
+    if (qrow < n) raw = *reinterpret_cast<const u32x4*>(qg + qrow * C + kk * 16 + h * 8);
+    __builtin_memcpy(&qf[kk], &raw, 16);
+  }
+  const float rq_i = (qrow < n) ? rq[qrow] : 0.f;
+  const float sc_i = rq_i * scale2;
+
+  f32x16 oacc[FB];
+#pragma unroll
+  for (int fb = 0; fb < FB; ++fb)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) oacc[fb][i] = 0.f;
+  float lsum = 0.f;
+
+  // global -> register staging of one key tile (K rows, K^T rows, rk)
+  constexpr int KCH = kKTile * C / 8 / kNceBlock;  // 16-byte chunks per thread, K tile
+  constexpr int TCH = C * kKTile / 8 / kNceBlock;  // same, K^T tile
+  u32x4 stage_k[KCH], stage_t[TCH];
+  float stage_rk = 0.f;
+  auto load_tile = [&](int64_t t) {
+    const int64_t key0 = t * kKTile;
+#pragma unroll
+    for (int u = 0; u < KCH; ++u) {
+      const int id = tid + u * kNceBlock;
+      const int r = id / (C / 8), c8 = id % (C / 8);
+      u32x4 v = {0u, 0u, 0u, 0u};
+      if (key0 + r < n) v = *reinterpret_cast<const u32x4*>(kg + (key0 + r) * C + c8 * 8);
+      stage_k[u] = v;
+    }
+#pragma unroll
+    for (int u = 0; u < TCH; ++u) {
+      const int id = tid + u * kNceBlock;
+      const int f = id / (kKTile / 8), c8 = id % (kKTile / 8);
+      stage_t[u] = *reinterpret_cast<const u32x4*>(ktg + (int64_t)f * npad + key0 + c8 * 8);
+    }
+    if (tid < kKTile) stage_rk = rk[key0 + tid];  // zero for padded keys
+  };
+  auto store_tile = [&](int buf) {
+#pragma unroll
+    for (int u = 0; u < KCH; ++u) {
+      const int id = tid + u * kNceBlock;
+      const int r = id / (C / 8), c8 = id % (C / 8);
+      *reinterpret_cast<u32x4*>(&sm.k[buf][r * Smem::KLD + c8 * 8]) = stage_k[u];
+    }
+#pragma unroll
+    for (int u = 0; u < TCH; ++u) {
+      const int id = tid + u * kNceBlock;
+      const int f = id / (kKTile / 8), c8 = id % (kKTile / 8);
+      *reinterpret_cast<u32x4*>(&sm.kt[buf][f * Smem::TLD + c8 * 8]) = stage_t[u];
+    }
+    if (tid < kKTile) sm.rk[buf][tid] = stage_rk;
+  };
+
+  if (t0 < t1) {
+    load_tile(t0);
+    store_tile(0);
+  }
+  __syncthreads();
+
+  for (int64_t t = t0; t < t1; ++t) {
+    const int buf = (int)((t - t0) & 1);
+    const bool more = t + 1 < t1;
+    if (more) load_tile(t + 1);  // in flight while this tile is computed
+
+    // S^T[key][q] = sum_f K[key][f] Q[q][f]
+    f32x16 sacc;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) sacc[i] = 0.f;
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      bf16x8 a;
+      const u32x4 raw = *reinterpret_cast<const u32x4*>(&sm.k[buf][col * Smem::KLD + kk * 16 + h * 8]);
+      __builtin_memcpy(&a, &raw, 16);
+      sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[kk], sacc, 0, 0, 0);
+    }
+
+    // P = 2^(S * rq_i * rk_j * log2e/tau - x_max); keys this lane holds:
+    // key(i) = (i%4) + 4h + 8(i/4).  Padded keys have rk = 0 and are masked.
+    const int64_t key0 = t * kKTile;
+    bf16x8 pb[2];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const f32x4 rk4 = *reinterpret_cast<const f32x4*>(&sm.rk[buf][8 * g + 4 * h]);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int i = 4 * g + j;
+        const float rkj = rk4[j];
+        float p = exp2f(sacc[i] * (sc_i * rkj) - scale2);
+        if (key0 + 8 * g + 4 * h + j >= n) p = 0.f;
+        lsum += p;
+        pb[g / 2][(g % 2) * 4 + j] = (__bf16)(p * rkj);
+      }
+    }
+
+    // O^T[f][q] += sum_key K^T[f][key] * (P*rk)[key][q]; contraction slot
+    // 8h + 4gg + j of step tt is key 16tt + 8gg + 4h + j on both operands.
+#pragma unroll
+    for (int fb = 0; fb < FB; ++fb) {
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt) {
+        const uint16_t* base = &sm.kt[buf][(fb * 32 + col) * Smem::TLD + 16 * tt + 4 * h];
+        bf16x4 lo, hi;
+        __builtin_memcpy(&lo, base, 8);
+        __builtin_memcpy(&hi, base + 8, 8);
+        bf16x8 a = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        oacc[fb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb[tt], oacc[fb], 0, 0, 0);
+      }
+    }
+
+    if (more) store_tile(buf ^ 1);
+    __syncthreads();
+  }
+
+  // partial results, register-native order: [split][q tile of 32][fb][i][lane]
+  const float ltot = lsum + __shfl_xor(lsum, 32, kWave);
+  if (h == 0) lpart[(int64_t)split * npad + qtile * kQTile + w * 32 + col] = ltot;
+  const int64_t tile32 = qtile * (kQTile / 32) + w;
+  float* op = opart + (((int64_t)split * (npad / 32) + tile32) * FB) * 16 * kWave;
+#pragma unroll
+  for (int fb = 0; fb < FB; ++fb)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) op[(fb * 16 + i) * kWave + lane] = oacc[fb][i];
+}
+
+// ---------------------------------------------------------------------------
+// combine: one wavefront per 32 q rows
+// ---------------------------------------------------------------------------
+template <typename T, int C>
+__global__ __launch_bounds__(kNceBlock) void nce_combine_kernel(const T* __restrict__ q, const T* __restrict__ k,
+                                                                const float* __restrict__ rq,
+                                                                const float* __restrict__ rk,
+                                                                const float* __restrict__ diag,
+                                                                const float* __restrict__ lpart,
+                                                                const float* __restrict__ opart, int64_t n,
+                                                                int64_t npad, int splits, float scale2,
+                                                                float* __restrict__ row_loss, T* __restrict__ dq) {
+  constexpr int FB = C / 32;
+  const int lane = threadIdx.x % kWave, w = threadIdx.x / kWave;
+  const int col = lane % 32, h = lane / 32;
+  const int64_t tile32 = (int64_t)blockIdx.x * (kNceBlock / kWave) + w;
+  if (tile32 >= npad / 32) return;
+  const int64_t row = tile32 * 32 + col;
+  const bool live = row < n;
+
+  float l = 0.f;
+  for (int s = 0; s < splits; ++s) l += lpart[(int64_t)s * npad + row];
+  if (h == 0) row_loss[row] = live ? kNceLn2 * (scale2 + log2f(l) - diag[row]) : 0.f;
+  if (!dq) return;
+
+  const float inv_l = live ? 1.f / l : 0.f;
+  const float rq_i = rq[row], rk_i = rk[row];
+  const float gn = 2.f / (float)n;
+
+  // dqh and qh for the features this lane holds: f = 32 fb + 8 g + 4 h + j
+  float dqh[FB][16], qh[FB][16];
+  float dot = 0.f;
+#pragma unroll
+  for (int fb = 0; fb < FB; ++fb) {
+    float o[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) o[i] = 0.f;
+    for (int s = 0; s < splits; ++s) {
+      const float* op = opart + (((int64_t)s * (npad / 32) + tile32) * FB + fb) * 16 * kWave;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) o[i] += op[i * kWave + lane];
+    }
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int i = 4 * g + j;
+        const int f = 32 * fb + 8 * g + 4 * h + j;
+        const float kv = live ? to_f32(k[row * C + f]) : 0.f;
+        const float qv = live ? to_f32(q[row * C + f]) : 0.f;
+        dqh[fb][i] = gn * (o[i] * inv_l - kv * rk_i);
+        qh[fb][i] = qv * rq_i;
+        dot += qh[fb][i] * dqh[fb][i];
+      }
+    }
+  }
+  dot += __shfl_xor(dot, 32, kWave);
+  // below eps the norm is the constant eps and normalize() is linear
+  const bool clamped = rq_i >= 1.f / kNormEps;
+  if (clamped) dot = 0.f;
+  if (!live) return;
+#pragma unroll
+  for (int fb = 0; fb < FB; ++fb)
+#pragma unroll
+    for (int g = 0; g < 4; ++g)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int i = 4 * g + j;
+        const int f = 32 * fb + 8 * g + 4 * h + j;
+        dq[row * C + f] = from_f32<T>((dqh[fb][i] - qh[fb][i] * dot) * rq_i);
+      }
+}
+
+template <typename T, int C>
+int nce_run_pair(const void* q, const void* k, void* dq, int64_t n, float tau, char* ws, float* row_loss,
+                 const NceLayout& L, hipStream_t stream) {
+  constexpr bool kF32 = sizeof(T) == 4;
+  float* rq = (float*)(ws + L.off_rq);
+  float* rk = (float*)(ws + L.off_rk);
+  float* diag = (float*)(ws + L.off_diag);
+  float* lpart = (float*)(ws + L.off_lpart);
+  uint16_t* kt = (uint16_t*)(ws + L.off_kt);
+  uint16_t* qb = kF32 ? (uint16_t*)(ws + L.off_qb) : nullptr;
+  uint16_t* kb = kF32 ? (uint16_t*)(ws + L.off_kb) : nullptr;
+  float* opart = (float*)(ws + L.off_opart);
+  const float scale2 = kNceLog2e / tau;
+
+  hipLaunchKernelGGL((nce_prep_kernel<T, C>), dim3((unsigned)(L.npad / 64)), dim3(kNceBlock), 0, stream,
+                     (const T*)q, (const T*)k, n, L.npad, scale2, rq, rk, diag, kt, qb, kb);
+  int rc = check_launch();
+  if (rc) return rc;
+  const uint16_t* qsrc = kF32 ? qb : (const uint16_t*)q;
+  const uint16_t* ksrc = kF32 ? kb : (const uint16_t*)k;
+  // with bf16 copies the rows beyond n exist (zero); the kernel guards by n either way
+  hipLaunchKernelGGL((nce_main_kernel<C>), dim3((unsigned)(L.npad / kQTile), (unsigned)L.splits),
+                     dim3(kNceBlock), 0, stream, qsrc, ksrc, kt, rq, rk, n, L.npad, L.splits, scale2, lpart,
+                     opart);
+  rc = check_launch();
+  if (rc) return rc;
+  const int64_t tiles32 = L.npad / 32;
+  hipLaunchKernelGGL((nce_combine_kernel<T, C>), dim3((unsigned)((tiles32 + 3) / 4)), dim3(kNceBlock), 0, stream,
+                     (const T*)q, (const T*)k, rq, rk, diag, lpart, opart, n, L.npad, L.splits, scale2, row_loss,
+                     (T*)dq);
+  return check_launch();
+}
+
+template <typename T>
+int nce_dispatch_c(const void* q, const void* k, void* dq, int64_t n, int64_t c, float tau, char* ws,
+                   float* row_loss, const NceLayout& L, hipStream_t stream) {
+  switch (c) {
+    case 64: return nce_run_pair<T, 64>(q, k, dq, n, tau, ws, row_loss, L, stream);
+    case 128: return nce_run_pair<T, 128>(q, k, dq, n, tau, ws, row_loss, L, stream);
+    case 256: return nce_run_pair<T, 256>(q, k, dq, n, tau, ws, row_loss, L, stream);
+    default: return TS_ERR_ARG;
+  }
+}
+
+}  // namespace ts
+
+extern "C" {
+
+size_t ts_infonce_workspace_bytes(int64_t n, int64_t c, int n_pairs) {
+  if (n < 0 || c <= 0 || n_pairs < 1 || n_pairs > 2) return 0;
+  // sized for fp32 inputs (the larger layout) so one query serves both dtypes
+  const ts::NceLayout L = ts::nce_layout(n, c, n_pairs, true);
+  return L.head_bytes + L.pair_bytes * (size_t)n_pairs;
+}
+
+int ts_infonce_fwd_bwd(const void* q1, const void* k1, const void* q2, const void* k2, int64_t n, int64_t c,
+                       float tau, void* workspace, float* loss_out, void* dq1, void* dq2, int dtype,
+                       ts_stream_t stream) {
+  if (!q1 || !k1 || !workspace || !loss_out) return TS_ERR_ARG;
+  if ((q2 == nullptr) != (k2 == nullptr)) return TS_ERR_ARG;
+  if (n < 0 || !(tau > 0.f)) return TS_ERR_ARG;
+  if (c != 64 && c != 128 && c != 256) return TS_ERR_ARG;
+  if (dtype != TS_F32 && dtype != TS_BF16) return TS_ERR_ARG;
+  // fixed soft-max reference point: 2^(-2 log2(e)/tau) must stay a normal fp32
+  if (tau < 0.03f) return TS_ERR_RANGE;
+  if (n > (1 << 24)) return TS_ERR_RANGE;
+  if ((uintptr_t)workspace & 255u) return TS_ERR_ALIGN;
+  // rows are read as 16-byte vectors
+  if (((uintptr_t)q1 | (uintptr_t)k1 | (uintptr_t)q2 | (uintptr_t)k2) & 15u) return TS_ERR_ALIGN;
+  hipStream_t st = (hipStream_t)stream;
+  const int pairs = q2 ? 2 : 1;
+  if (n == 0) {
+    // cross entropy over zero rows: mean of nothing = NaN, as torch gives
+    return ts::launch_sum_scale((const float*)workspace, 0, 1.f, 0.f, loss_out, st);
+  }
+  const ts::NceLayout L = ts::nce_layout(n, c, pairs, true);
+  char* ws = (char*)workspace;
+  float* row_loss = (float*)ws;
+  for (int p = 0; p < pairs; ++p) {
+    const void* q = p ? q2 : q1;
+    const void* k = p ? k2 : k1;
+    void* dq = p ? dq2 : dq1;
+    char* wsp = ws + L.head_bytes + (size_t)p * L.pair_bytes;
+    float* rl = row_loss + (size_t)p * L.npad;
+    int rc = (dtype == TS_F32) ? ts::nce_dispatch_c<float>(q, k, dq, n, c, tau, wsp, rl, L, st)
+                               : ts::nce_dispatch_c<ts::bf16_t>(q, k, dq, n, c, tau, wsp, rl, L, st);
+    if (rc) return rc;
+  }
+  // loss = 2 tau / n * sum over all pairs' rows (padding rows hold zero)
+  return ts::launch_sum_scale(row_loss, (int64_t)pairs * L.npad, 2.f * tau, (float)n, loss_out, st);
+}
+
+}  // extern "C"

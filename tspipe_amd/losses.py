@@ -1,0 +1,259 @@
+"""Teacher-student losses with fused forward+backward HIP kernels, behind the
+``loss_fn`` plug-in signatures TSPipe calls (tspipe/gpu_task.py:178-179 for
+distillation, 202-203 for self-supervised momentum training).
+
+Each loss is a ``torch.autograd.Function`` whose forward launches one fused
+kernel that produces the scalar loss *and* the gradient with respect to the
+student input; backward hands that gradient out (rescaled on the device by the
+incoming gradient, which is exactly 1 when the pipeline calls
+``torch.autograd.backward(loss)``, tspipe/gpu_task.py:207-212).  Teacher inputs
+receive no gradient: the pipeline detaches them (tspipe/gpu_task.py:109).
+
+The scalar loss is returned in fp32 whatever the input dtype, since the
+kernels accumulate in fp32.
+"""
+from argparse import Namespace
+from typing import Optional
+
+import torch
+from torch import Tensor, nn
+
+from . import _lib
+
+
+def _require_cuda(*tensors: Tensor) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise TypeError("tspipe_amd losses run on device tensors only (no host fallback)")
+
+
+def _once(ctx) -> None:
+    if ctx.backward_done:
+        raise RuntimeError("the fused loss keeps one gradient buffer: backward can run once per forward")
+    ctx.backward_done = True
+
+
+def _scale_saved_grad(grad: Tensor, grad_output: Tensor, rows: int, cols: int) -> Tensor:
+    """grad *= grad_output on the device, without a host sync; the kernel
+    returns immediately when grad_output is 1."""
+    g = grad_output.detach().to(torch.float32).reshape(1)
+    with torch.cuda.device(grad.device):
+        status = _lib.lib().ts_scale_rows(grad.data_ptr(), rows, cols, cols, g.data_ptr(),
+                                          _lib.dtype_code(grad.dtype), _lib.current_stream_ptr(grad.device))
+    _lib.check(status, "ts_scale_rows")
+    return grad
+
+
+# ---------------------------------------------------------------------------
+# KD soft-target loss
+# ---------------------------------------------------------------------------
+
+class _KDSoftTargetFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, out_s: Tensor, out_t: Tensor, row_mask: Optional[Tensor], T: float, weight: float):
+        _require_cuda(out_s, out_t, row_mask)
+        if out_s.shape != out_t.shape:
+            raise ValueError(f"student/teacher logits differ in shape: {tuple(out_s.shape)} vs {tuple(out_t.shape)}")
+        if out_s.dtype != out_t.dtype:
+            raise TypeError(f"student/teacher logits differ in dtype: {out_s.dtype} vs {out_t.dtype}")
+        V = int(out_s.shape[-1])
+        s = out_s.detach().reshape(-1, V)
+        t = out_t.detach().reshape(-1, V)
+        s = s if s.is_contiguous() else s.contiguous()
+        t = t if t.is_contiguous() else t.contiguous()
+        rows = int(s.shape[0])
+        mask_ptr = None
+        if row_mask is not None:
+            m = row_mask.detach().reshape(-1)
+            if m.numel() != rows:
+                raise ValueError(f"row mask has {m.numel()} entries for {rows} rows")
+            if m.dtype != torch.bool:
+                m = m != 0
+            m = m.contiguous().view(torch.uint8)
+            mask_ptr = m.data_ptr()
+        need_grad = ctx.needs_input_grad[0]
+        lib = _lib.lib()
+        dev = s.device
+        ws = torch.empty(lib.ts_kd_workspace_bytes(rows), dtype=torch.uint8, device=dev)
+        loss = torch.empty((), dtype=torch.float32, device=dev)
+        grad = torch.empty_like(s) if need_grad else None
+        with torch.cuda.device(dev):
+            status = lib.ts_kd_fwd_bwd(s.data_ptr(), t.data_ptr(), mask_ptr, rows, V, V, V, 1.0 / T,
+                                       T * T * weight, ws.data_ptr(), loss.data_ptr(),
+                                       None if grad is None else grad.data_ptr(), V,
+                                       _lib.dtype_code(s.dtype), _lib.current_stream_ptr(dev))
+        _lib.check(status, "ts_kd_fwd_bwd")
+        ctx.grad = grad
+        ctx.shape = out_s.shape
+        ctx.dims = (rows, V)
+        ctx.backward_done = False
+        return loss
+
+    @staticmethod
+    def backward(ctx, grad_output: Tensor):
+        if ctx.grad is None:
+            return None, None, None, None, None
+        _once(ctx)
+        grad = _scale_saved_grad(ctx.grad, grad_output, *ctx.dims)
+        return grad.view(ctx.shape), None, None, None, None
+
+
+def kd_soft_target_loss(out_s: Tensor, out_t: Tensor, T: float, weight: float = 1.0,
+                        row_mask: Optional[Tensor] = None) -> Tensor:
+    """``weight * T^2 * KL(softmax(out_t/T) || softmax(out_s/T))`` averaged over
+    the rows (last dimension = classes) selected by ``row_mask`` (all rows when
+    ``None``); the formula of benchmarks/soft_target/kd_losses/st.py:18-23 and,
+    with a mask, of benchmarks/distilbert/distiller.py:719-740."""
+    return _KDSoftTargetFn.apply(out_s, out_t, row_mask, float(T), float(weight))
+
+
+class SoftTarget(nn.Module):
+    """Drop-in for benchmarks/soft_target/kd_losses/st.py:9-23."""
+
+    def __init__(self, T: float):
+        super().__init__()
+        self.T = T
+
+    def forward(self, out_s: Tensor, out_t: Tensor) -> Tensor:
+        if out_s.dim() != 2:
+            raise ValueError("SoftTarget expects [batch, classes] logits")
+        return kd_soft_target_loss(out_s, out_t, self.T)
+
+
+def distil_ce_loss(s_logits: Tensor, t_logits: Tensor, row_mask: Tensor, temperature: float,
+                   alpha_ce: float = 1.0) -> Tensor:
+    """The distillation term of DistilBERT's loss
+    (benchmarks/distilbert/distiller.py:719-740): rows of ``[bs, seq, vocab]``
+    logits where ``row_mask`` (``[bs, seq]``) is set, KL with batchmean over the
+    selected rows, times ``temperature**2`` and ``alpha_ce``.  No row is copied:
+    the kernel reads the mask and writes a dense gradient with zeros elsewhere."""
+    return _KDSoftTargetFn.apply(s_logits, t_logits, row_mask, float(temperature), float(alpha_ce))
+
+
+# ---------------------------------------------------------------------------
+# BYOL normalised MSE
+# ---------------------------------------------------------------------------
+
+class _BYOLFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x1: Tensor, y1: Tensor, x2: Optional[Tensor], y2: Optional[Tensor]):
+        _require_cuda(x1, y1, x2, y2)
+        tensors = [x1, y1] + ([x2, y2] if x2 is not None else [])
+        if any(t.dim() != 2 for t in tensors):
+            raise ValueError("BYOL loss expects [batch, features] projections")
+        if any(t.shape != x1.shape or t.dtype != x1.dtype for t in tensors):
+            raise ValueError("BYOL loss inputs must agree in shape and dtype")
+        n, c = int(x1.shape[0]), int(x1.shape[1])
+        prep = [t.detach() if t.is_contiguous() else t.detach().contiguous() for t in tensors]
+        dev = x1.device
+        ws = torch.empty(2 * max(n, 1), dtype=torch.float32, device=dev)
+        loss = torch.empty((), dtype=torch.float32, device=dev)
+        g1 = torch.empty_like(prep[0]) if ctx.needs_input_grad[0] else None
+        g2 = torch.empty_like(prep[2]) if (x2 is not None and ctx.needs_input_grad[2]) else None
+        with torch.cuda.device(dev):
+            status = _lib.lib().ts_byol_fwd_bwd(
+                prep[0].data_ptr(), prep[1].data_ptr(),
+                prep[2].data_ptr() if x2 is not None else None,
+                prep[3].data_ptr() if x2 is not None else None, n, c, ws.data_ptr(), loss.data_ptr(),
+                None if g1 is None else g1.data_ptr(), None if g2 is None else g2.data_ptr(),
+                _lib.dtype_code(x1.dtype), _lib.current_stream_ptr(dev))
+        _lib.check(status, "ts_byol_fwd_bwd")
+        ctx.g1, ctx.g2, ctx.dims = g1, g2, (n, c)
+        ctx.backward_done = False
+        return loss
+
+    @staticmethod
+    def backward(ctx, grad_output: Tensor):
+        _once(ctx)
+        out1 = out2 = None
+        if ctx.g1 is not None:
+            out1 = _scale_saved_grad(ctx.g1, grad_output, *ctx.dims)
+        if ctx.g2 is not None:
+            out2 = _scale_saved_grad(ctx.g2, grad_output, *ctx.dims)
+        return out1, None, out2, None
+
+
+def byol_loss(online_view_1: Tensor, online_view_2: Tensor, target_view_1: Tensor,
+              target_view_2: Tensor) -> Tensor:
+    """``mean(rl(o1, t2) + rl(o2, t1))`` with ``rl(x, y) = 2 - 2 <x^, y^>``
+    (benchmarks/byol/trainer.py:51-55, 192-196)."""
+    return _BYOLFn.apply(online_view_1, target_view_2, online_view_2, target_view_1)
+
+
+def regression_loss_mean(x: Tensor, y: Tensor) -> Tensor:
+    """``regression_loss(x, y).mean()`` for a single pair (benchmarks/byol/trainer.py:51-55)."""
+    return _BYOLFn.apply(x, y, None, None)
+
+
+# ---------------------------------------------------------------------------
+# MoCo-v3 InfoNCE
+# ---------------------------------------------------------------------------
+
+class _InfoNCEFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q1: Tensor, k1: Tensor, q2: Optional[Tensor], k2: Optional[Tensor], tau: float):
+        _require_cuda(q1, k1, q2, k2)
+        tensors = [q1, k1] + ([q2, k2] if q2 is not None else [])
+        if any(t.dim() != 2 for t in tensors):
+            raise ValueError("InfoNCE expects [batch, features] embeddings")
+        if any(t.shape != q1.shape or t.dtype != q1.dtype for t in tensors):
+            raise ValueError("InfoNCE inputs must agree in shape and dtype")
+        n, c = int(q1.shape[0]), int(q1.shape[1])
+        prep = [t.detach() if t.is_contiguous() else t.detach().contiguous() for t in tensors]
+        dev = q1.device
+        lib = _lib.lib()
+        pairs = 2 if q2 is not None else 1
+        ws = torch.empty(lib.ts_infonce_workspace_bytes(n, c, pairs), dtype=torch.uint8, device=dev)
+        loss = torch.empty((), dtype=torch.float32, device=dev)
+        g1 = torch.empty_like(prep[0]) if ctx.needs_input_grad[0] else None
+        g2 = torch.empty_like(prep[2]) if (q2 is not None and ctx.needs_input_grad[2]) else None
+        with torch.cuda.device(dev):
+            status = lib.ts_infonce_fwd_bwd(
+                prep[0].data_ptr(), prep[1].data_ptr(),
+                prep[2].data_ptr() if q2 is not None else None,
+                prep[3].data_ptr() if q2 is not None else None, n, c, tau, ws.data_ptr(), loss.data_ptr(),
+                None if g1 is None else g1.data_ptr(), None if g2 is None else g2.data_ptr(),
+                _lib.dtype_code(q1.dtype), _lib.current_stream_ptr(dev))
+        _lib.check(status, "ts_infonce_fwd_bwd")
+        ctx.g1, ctx.g2, ctx.dims = g1, g2, (n, c)
+        ctx.backward_done = False
+        return loss
+
+    @staticmethod
+    def backward(ctx, grad_output: Tensor):
+        _once(ctx)
+        out1 = out2 = None
+        if ctx.g1 is not None:
+            out1 = _scale_saved_grad(ctx.g1, grad_output, *ctx.dims)
+        if ctx.g2 is not None:
+            out2 = _scale_saved_grad(ctx.g2, grad_output, *ctx.dims)
+        return out1, None, out2, None, None
+
+
+def infonce_loss(q: Tensor, k: Tensor, tau: float) -> Tensor:
+    """One direction of MoCo-v3's loss: ``CE(q^ k^T / tau, arange(N)) * 2 tau``
+    (benchmarks/moco-v3/main.py:149-160)."""
+    return _InfoNCEFn.apply(q, k, None, None, float(tau))
+
+
+def moco_contrastive_loss_pair(online_view_1: Tensor, online_view_2: Tensor, target_view_1: Tensor,
+                               target_view_2: Tensor, tau: float) -> Tensor:
+    """``loss(o1, t2) + loss(o2, t1)`` in one launch (benchmarks/moco-v3/main.py:162)."""
+    return _InfoNCEFn.apply(online_view_1, target_view_2, online_view_2, target_view_1, float(tau))
+
+
+# ---------------------------------------------------------------------------
+# loss_fn plug-ins with the reference's signatures
+# ---------------------------------------------------------------------------
+
+def byol_contrastive_loss(online_view_1, online_view_2, target_view_1, target_view_2,
+                          args: Namespace = None, extra_args: Namespace = None) -> Tensor:
+    """``TSPipeBYOLTrainer.contrastive_loss`` (benchmarks/byol/trainer.py:192-196)."""
+    return byol_loss(online_view_1, online_view_2, target_view_1, target_view_2)
+
+
+def moco_contrastive_loss(online_view_1, online_view_2, target_view_1, target_view_2, args, extra_args) -> Tensor:
+    """``contrastive_loss`` of benchmarks/moco-v3/main.py:147-162; the
+    temperature comes from ``extra_args.moco_t``."""
+    return moco_contrastive_loss_pair(online_view_1, online_view_2, target_view_1, target_view_2,
+                                      float(extra_args.moco_t))
