@@ -1,0 +1,315 @@
+#!/usr/bin/env python3
+"""Benchmark of the teacher-student step kernels on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-kernels]
+
+One "step" is the MoCo-v3 ViT-Base teacher-student step of the kernel path:
+the momentum EMA over the ViT-B/16 parameter list (152 fp32 tensors,
+86,567,656 elements, m = 0.99) on one HIP stream, and the InfoNCE loss forward
++ backward on bf16 q, k of 4096 x 256 (tau = 0.2) on a second stream, joined at
+the end of the step.  All inputs are resident in HBM before the timed region.
+
+Prints ONE JSON line.  `value` is steps per second over exactly K timed steps;
+`roofline` is for the dominant kernel (the multi-tensor EMA): algorithmic bytes
+per launch (12 B per parameter) over its average duration, measured with HIP
+events recorded on the kernel's own stream inside the timed region;
+`cpu_baseline` is the oracle's eager PyTorch restatement of the same step on
+the host cores (bounded sample); `kernels` holds stand-alone timings of every
+kernel at the other configurations (informational).
+"""
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+HBM_PEAK_GBS = 8000.0       # MI355X published HBM3E bandwidth
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+
+
+def _shapes():
+    from shapes import numel, resnet18_shapes, vit_base_shapes
+    return numel, resnet18_shapes(), vit_base_shapes()
+
+
+def _event_ms(pairs):
+    return [a.elapsed_time(b) for a, b in pairs]
+
+
+def _time_gpu(fn, iters, warmup=5):
+    """Median / mean milliseconds of fn() over `iters` runs, HIP events on the current stream."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    pairs = []
+    for _ in range(iters):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        fn()
+        b.record()
+        pairs.append((a, b))
+    torch.cuda.synchronize()
+    ms = _event_ms(pairs)
+    return statistics.median(ms), sum(ms) / len(ms), min(ms)
+
+
+def run_step_benchmark(steps, warmup, dev):
+    import torch
+    import tspipe_amd as ta
+    from tspipe_amd import ema as ema_mod
+    numel, _, vit = _shapes()
+
+    g = torch.Generator().manual_seed(3)
+    teacher = [(torch.randn(s, generator=g) * 0.02).to(dev) for s in vit]
+    student = [(torch.randn(s, generator=g) * 0.02).to(dev) for s in vit]
+    q = torch.nn.functional.normalize(torch.randn(4096, 256, generator=g), dim=1).to(torch.bfloat16).to(dev)
+    k = torch.nn.functional.normalize(torch.randn(4096, 256, generator=g), dim=1).to(torch.bfloat16).to(dev)
+    q.requires_grad_()
+    n_params = sum(numel(s) for s in vit)
+
+    s_ema, s_loss = torch.cuda.Stream(dev), torch.cuda.Stream(dev)
+    state = {"teacher": teacher, "loss": None}
+
+    def step():
+        main = torch.cuda.current_stream(dev)
+        s_ema.wait_stream(main)
+        s_loss.wait_stream(main)
+        with torch.cuda.stream(s_ema):
+            state["teacher"] = ta.calculate_updated_momentum_encoder(0.99, student, state["teacher"])
+        with torch.cuda.stream(s_loss):
+            q.grad = None
+            loss = ta.infonce_loss(q, k, 0.2)
+            loss.backward()
+            state["loss"] = loss
+        main.wait_stream(s_ema)
+        main.wait_stream(s_loss)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    ema_mod.kernel_events = []  # (start, end) HIP events around every EMA kernel launch
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    events = ema_mod.kernel_events
+    ema_mod.kernel_events = None
+    ema_ms = _event_ms(events)
+    assert len(ema_ms) == steps
+    avg_ema_ms = sum(ema_ms) / len(ema_ms)
+    algo_bytes = 12 * n_params
+    achieved = algo_bytes / (avg_ema_ms * 1e-3) / 1e9
+    return {
+        "elapsed": elapsed, "n_params": n_params, "loss": float(state["loss"].item()),
+        "roofline": {"bound": "hbm", "kernel": "ema_multi_kernel", "achieved": round(achieved, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": None, "algorithmic_bytes_per_launch": algo_bytes,
+                     "avg_kernel_ms": round(avg_ema_ms, 4), "launches_timed": len(ema_ms)},
+    }
+
+
+def run_kernel_table(dev):
+    """Stand-alone timings of each kernel at the other configurations."""
+    import torch
+    import tspipe_amd as ta
+    from tspipe_amd import _lib
+    numel, r18, vit = _shapes()
+    out = {}
+    g = torch.Generator().manual_seed(0)
+
+    def gbs(nbytes, ms):
+        return round(nbytes / (ms * 1e-3) / 1e9, 1)
+
+    def entry(nbytes, t, note=None):
+        med, mean, best = t
+        e = {"ms_median": round(med, 4), "ms_min": round(best, 4), "GB/s": gbs(nbytes, med),
+             "frac_hbm_peak": round(gbs(nbytes, med) / HBM_PEAK_GBS, 4), "algorithmic_bytes": nbytes}
+        if note:
+            e["note"] = note
+        return e
+
+    # EMA, stand-alone (no concurrent loss), both parameter lists
+    for name, shapes, m in (("ema_vit_base", vit, 0.99), ("ema_resnet18", r18, 0.996)):
+        teacher = [(torch.randn(s, generator=g) * 0.02).to(dev) for s in shapes]
+        student = [(torch.randn(s, generator=g) * 0.02).to(dev) for s in shapes]
+        st = {"t": teacher}
+
+        def f():
+            st["t"] = ta.calculate_target_network_parameters(m, student, st["t"])
+        from tspipe_amd import ema as ema_mod
+        for _ in range(5):
+            f()
+        torch.cuda.synchronize()
+        ema_mod.kernel_events = []
+        for _ in range(30):
+            f()
+        torch.cuda.synchronize()
+        ms = _event_ms(ema_mod.kernel_events)
+        ema_mod.kernel_events = None
+        nbytes = 12 * sum(numel(s) for s in shapes)
+        note = "working set below the 256 MB Infinity Cache: not an HBM figure" if name == "ema_resnet18" else None
+        out[name] = entry(nbytes, (statistics.median(ms), sum(ms) / len(ms), min(ms)), note)
+        del teacher, student, st
+
+    # KD small (cfg2) and a scaled shape for a bandwidth figure
+    for name, rows in (("kd_256x100_f32", 256), ("kd_65536x100_f32", 65536)):
+        s = (torch.randn(rows, 100, generator=g) * 3).to(dev).requires_grad_()
+        t = (torch.randn(rows, 100, generator=g) * 3).to(dev)
+
+        def f():
+            s.grad = None
+            ta.kd_soft_target_loss(s, t, 4.0).backward()
+        out[name] = entry(3 * rows * 100 * 4, _time_gpu(f, 50), "latency-bound" if rows == 256 else None)
+
+    # DistilBERT-shaped masked KD (cfg3) after a gather of 4 micro-batches
+    pieces_s = [(torch.randn(8, 128, 30522, generator=g) * 2).to(torch.bfloat16).to(dev) for _ in range(4)]
+    pieces_t = [(torch.randn(8, 128, 30522, generator=g) * 2).to(torch.bfloat16).to(dev) for _ in range(4)]
+    mask = (torch.rand(32, 128, generator=g) < 0.15).to(dev)
+    n_sel = int(mask.sum().item())
+    batches = [ta.Batch(p) for p in pieces_s]
+    out["gather_4x62.5MB_bf16"] = entry(2 * 250036224, _time_gpu(lambda: ta.gather(batches), 20))
+    s_full = ta.gather(batches).requires_grad_()
+    t_full = ta.gather([ta.Batch(p) for p in pieces_t])
+    del pieces_s, pieces_t, batches
+
+    def f():
+        s_full.grad = None
+        ta.distil_ce_loss(s_full, t_full, mask, 2.0).backward()
+    row_b = 30522 * 2
+    out["kd_masked_32x128x30522_bf16"] = entry(3 * n_sel * row_b + (4096 - n_sel) * row_b, _time_gpu(f, 20),
+                                               f"n_sel={n_sel}; bytes = 3 rows r/r/w for selected + zero-fill of the rest")
+    del s_full, t_full
+
+    # InfoNCE (cfg4), single pair
+    q = torch.nn.functional.normalize(torch.randn(4096, 256, generator=g), dim=1).to(torch.bfloat16).to(dev).requires_grad_()
+    k = torch.nn.functional.normalize(torch.randn(4096, 256, generator=g), dim=1).to(torch.bfloat16).to(dev)
+
+    def f():
+        q.grad = None
+        ta.infonce_loss(q, k, 0.2).backward()
+    med, mean, best = _time_gpu(f, 50)
+    flops = 2 * 2 * 4096 * 4096 * 256
+    out["infonce_4096x256_bf16"] = {"ms_median": round(med, 4), "ms_min": round(best, 4),
+                                    "TFLOP/s": round(flops / (med * 1e-3) / 1e12, 1),
+                                    "frac_mfma_bf16_peak": round(flops / (med * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+                                    "algorithmic_flop": flops}
+
+    # BYOL loss (latency only)
+    o = [torch.randn(256, 128, generator=g).to(dev) for _ in range(4)]
+    o[0].requires_grad_()
+    o[1].requires_grad_()
+
+    def f():
+        o[0].grad = o[1].grad = None
+        ta.byol_loss(o[0], o[1], o[2], o[3]).backward()
+    med, mean, best = _time_gpu(f, 50)
+    out["byol_256x128_f32"] = {"ms_median": round(med, 4), "ms_min": round(best, 4), "note": "latency-bound"}
+
+    # DeferredBatchNorm (cfg5): statistics only, and statistics + normalise
+    x = (torch.randn(32, 256, 56, 56, generator=g) * 1.5 + 0.5).to(dev)
+    bn = ta.DeferredBatchNorm(256, chunks=8).to(dev)
+    lib = _lib.lib()
+    mean_b = torch.empty(256, device=dev)
+    inv_b = torch.empty(256, device=dev)
+
+    def stats_only():
+        _lib.check(lib.ts_bn_stats(x.data_ptr(), 32, 256, 3136, bn._ws.data_ptr(), bn.sum.data_ptr(),
+                                   bn.sum_squares.data_ptr(), mean_b.data_ptr(), inv_b.data_ptr(), 1e-5,
+                                   _lib.current_stream_ptr(dev)), "ts_bn_stats")
+    out["bn_stats_32x256x56x56_f32"] = entry(x.numel() * 4, _time_gpu(stats_only, 30))
+    with torch.no_grad():
+        out["bn_track_normalise_32x256x56x56_f32"] = entry(x.numel() * 12, _time_gpu(lambda: bn(x), 30))
+    return out
+
+
+def run_cpu_baseline(budget_s=12.0):
+    """The oracle's eager-PyTorch step (reference arithmetic) on the host cores."""
+    import torch
+    from oracle import ts_oracle
+    numel, _, vit = _shapes()
+    cores = os.cpu_count() or 1
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    torch.set_num_threads(cores)
+    g = torch.Generator().manual_seed(3)
+    teacher = [torch.randn(s, generator=g) * 0.02 for s in vit]
+    student = [torch.randn(s, generator=g) * 0.02 for s in vit]
+    q = torch.nn.functional.normalize(torch.randn(4096, 256, generator=g), dim=1).to(torch.bfloat16).requires_grad_()
+    k = torch.nn.functional.normalize(torch.randn(4096, 256, generator=g), dim=1).to(torch.bfloat16)
+
+    def step(t):
+        t = ts_oracle.ema_update(0.99, student, t, skip_none=True)
+        q.grad = None
+        ts_oracle.infonce(q, k, 0.2).backward()
+        return t
+
+    teacher = step(teacher)  # warm-up
+    n, t0 = 0, time.perf_counter()
+    while True:
+        teacher = step(teacher)
+        n += 1
+        el = time.perf_counter() - t0
+        if el > budget_s or n >= 50:
+            break
+    return {"value": round(n / el, 4), "unit": "steps/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"{n} full steps (EMA over 152 tensors / 86.6M params per-tensor loop + InfoNCE 4096x256 bf16 "
+                      f"fwd+bwd, eager PyTorch on CPU) in {el:.1f} s"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel table")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py: this build measures one GPU only; the kernel path has no cross-GPU exchange "
+                 "(each pipeline partition runs it on its own parameters). Run with --gpus 1.")
+
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    from tspipe_amd import _lib
+    _lib.lib()  # fail loudly if the HIP library is missing
+
+    res = run_step_benchmark(args.steps, args.warmup, dev)
+    line = {
+        "metric": "TS-steps/sec at ViT-B momentum (EMA over 86.6M fp32 params || InfoNCE 4096x256 bf16 fwd+bwd)",
+        "value": round(args.steps / res["elapsed"], 2),
+        "unit": "steps/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(res["elapsed"] / args.steps * 1e3, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "MoCo-v3 ViT-Base step: fp32 EMA over ViT-B/16 shapes (152 tensors, 86,567,656 params, "
+                               "m=0.99) + InfoNCE fwd+bwd on bf16 q,k 4096x256, tau=0.2, two HIP streams",
+                   "ema_tensors": 152, "ema_params": res["n_params"], "infonce_n": 4096, "infonce_c": 256},
+        "roofline": res["roofline"],
+        "loss": res["loss"],
+    }
+    if not args.no_kernels:
+        line["kernels"] = run_kernel_table(dev)
+    if not args.no_cpu:
+        line["cpu_baseline"] = run_cpu_baseline()
+    else:
+        line["cpu_baseline"] = None
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

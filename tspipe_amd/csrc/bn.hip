@@ -141,10 +141,14 @@ __global__ __launch_bounds__(256) void bn_commit_kernel(float* __restrict__ sum,
   const double f = (momentum < 0.0) ? 1.0 / (double)tracked : momentum;
   const float f32 = (float)f, omf32 = (float)(1.0 - f);
   if (c < C) {
-    const float mean = __fdiv_rn(sum[c], counter);
-    const float var = __fsub_rn(__fdiv_rn(sum_squares[c], counter), __fmul_rn(mean, mean));
-    running_mean[c] = __fadd_rn(__fmul_rn(running_mean[c], omf32), __fmul_rn(mean, f32));
-    running_var[c] = __fadd_rn(__fmul_rn(running_var[c], omf32), __fmul_rn(var, f32));
+#pragma clang fp contract(off)
+    const float mean = sum[c] / counter;
+    const float msq = mean * mean;
+    const float var = sum_squares[c] / counter - msq;
+    const float rm = running_mean[c] * omf32, dm = mean * f32;
+    const float rv = running_var[c] * omf32, dv = var * f32;
+    running_mean[c] = rm + dm;
+    running_var[c] = rv + dv;
     sum[c] = 0.f;
     sum_squares[c] = 0.f;
   }

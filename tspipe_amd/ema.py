@@ -16,6 +16,10 @@ import torch
 
 from . import _lib, _tables
 
+# When set to a list, every EMA launch appends a (start, end) pair of HIP
+# events recorded on the launch stream around the kernel alone (profiling aid).
+kernel_events = None
+
 
 def _prepare(online: Iterable[Optional[torch.Tensor]], target: Iterable[torch.Tensor], skip_none: bool):
     students, teachers = [], []
@@ -47,9 +51,16 @@ def _launch(m: float, students: Sequence[torch.Tensor], teachers: Sequence[torch
                                   _tables.ptr_array(outs), numels, device)
         # the reference multiplies by the Python doubles m and (1. - m); torch
         # rounds each to fp32 before the fp32 multiply
+        timed = kernel_events is not None
+        if timed:
+            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record(torch.cuda.current_stream(device))
         status = _lib.lib().ts_ema_multi(table.dev_ptr, table.n_chunks, float(m), 1.0 - float(m),
                                         _lib.current_stream_ptr(device))
         _lib.check(status, "ts_ema_multi")
+        if timed:
+            end.record(torch.cuda.current_stream(device))
+            kernel_events.append((start, end))
         table.done()
 
 
