@@ -72,16 +72,19 @@ typedef struct ts_ema_chunk {
 int64_t ts_ema_auto_chunk(int64_t total_elems);
 
 /* Host: split n_tensors (t[i], s[i], out[i], numel[i]) into chunks.
- * chunk_elems: elements per chunk, a positive multiple of 1024, or 0 = auto.
+ * chunk_elems: elements per chunk, a positive multiple of 1024, or 0 = the
+ * value of ts_ema_auto_chunk(sum of numel).
  * table == NULL: only count.  Returns the chunk count (>= 0) or TS_ERR_*.
  * Tensors with numel 0 produce no chunk.  Pointers must be 4-byte aligned. */
 int64_t ts_ema_plan(const void* const* t, const void* const* s, void* const* out,
                     const int64_t* numel, int64_t n_tensors, int64_t chunk_elems,
                     ts_ema_chunk* table, int64_t capacity);
 
-/* Device: run the EMA over a table that lives in device memory. */
-int ts_ema_multi(const ts_ema_chunk* table_dev, int64_t n_chunks, float m32, float c32,
-                 ts_stream_t stream);
+/* Device: run the EMA over a table that lives in device memory.  chunk_elems
+ * is the chunk size the table was planned with (the kernel cuts every chunk
+ * into workgroup-sized pieces of 1024 elements). */
+int ts_ema_multi(const ts_ema_chunk* table_dev, int64_t n_chunks, int64_t chunk_elems, float m32,
+                 float c32, ts_stream_t stream);
 
 /* ------------------------------------------------------------------------ */
 /* Multi-segment copy: micro-batch gather (torch.cat on dim 0,      */
@@ -101,13 +104,15 @@ typedef struct ts_copy_chunk {
 int64_t ts_copy_auto_chunk(int64_t total_bytes);
 
 /* Host: split n_segments (src[i], dst[i], bytes[i]) into chunks of at most
- * chunk_bytes (positive multiple of 4096, or 0 = auto).  Same return rule as
+ * chunk_bytes (positive multiple of 4096, or 0 = ts_copy_auto_chunk(sum)).  Same return rule as
  * ts_ema_plan.  Source and destination ranges must not overlap. */
 int64_t ts_copy_plan(const void* const* src, void* const* dst, const int64_t* bytes,
                      int64_t n_segments, int64_t chunk_bytes, ts_copy_chunk* table,
                      int64_t capacity);
 
-int ts_copy_segments(const ts_copy_chunk* table_dev, int64_t n_chunks, ts_stream_t stream);
+/* chunk_bytes: the chunk size the table was planned with. */
+int ts_copy_segments(const ts_copy_chunk* table_dev, int64_t n_chunks, int64_t chunk_bytes,
+                     ts_stream_t stream);
 
 /* ------------------------------------------------------------------------ */
 /* KD soft-target loss, forward and backward in one pass over rows.   */

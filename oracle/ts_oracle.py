@@ -160,9 +160,13 @@ def gather(pieces: list):
     return tuple(torch.cat(group) for group in zip(*pieces))
 
 
-def generic_object_scatter(obj: Any, chunks: int) -> Any:
-    """tspipe/utils.py:225-254 (TSPipeModelOutput handling left to the caller).
-    dict is matched before OrderedDict, as in the reference."""
+def generic_object_scatter(obj: Any, chunks: int, output_cls=None) -> Any:
+    """tspipe/utils.py:225-254.  dict is matched before OrderedDict, as in the
+    reference.  output_cls: the TSPipeModelOutput-like dataclass to unwrap and
+    re-wrap at the top level (utils.py:246-250), if any."""
+    if output_cls is not None and isinstance(obj, output_cls):
+        return [output_cls(data=x, lst_require_grad_tensor_path=obj.lst_require_grad_tensor_path)
+                for x in generic_object_scatter(obj.data, chunks)]
     if isinstance(obj, list):
         return [list(x) for x in zip(*[generic_object_scatter(x, chunks) for x in obj])]
     if isinstance(obj, tuple):
@@ -176,8 +180,14 @@ def generic_object_scatter(obj: Any, chunks: int) -> Any:
     return [obj for _ in range(chunks)]
 
 
-def generic_object_gather(*objs: Any) -> Any:
-    """tspipe/utils.py:256-286."""
+def generic_object_gather(*objs: Any, output_cls=None) -> Any:
+    """tspipe/utils.py:256-292.  With output_cls, a call whose arguments are all
+    of that class gathers their .data and keeps the first one's path list; as in
+    the reference, that test is vacuously true for an empty call, which then
+    fails on objs[0]."""
+    if output_cls is not None and all(isinstance(o, output_cls) for o in objs):
+        return output_cls(data=generic_object_gather(*[o.data for o in objs]),
+                          lst_require_grad_tensor_path=objs[0].lst_require_grad_tensor_path)
     if len(objs) == 0:
         return tuple()
     first = objs[0]

@@ -70,10 +70,10 @@ def ptr_array(tensors: Sequence[torch.Tensor]) -> np.ndarray:
 
 class StagedTable:
     """A planned table resident on the device; call done() after the launch."""
-    __slots__ = ("slot", "n_chunks", "device")
+    __slots__ = ("slot", "n_chunks", "chunk", "device")
 
-    def __init__(self, slot: _Slot, n_chunks: int, device: torch.device):
-        self.slot, self.n_chunks, self.device = slot, n_chunks, device
+    def __init__(self, slot: _Slot, n_chunks: int, chunk: int, device: torch.device):
+        self.slot, self.n_chunks, self.chunk, self.device = slot, n_chunks, chunk, device
 
     @property
     def dev_ptr(self) -> int:
@@ -89,6 +89,8 @@ def stage_ema(t_ptrs: np.ndarray, s_ptrs: np.ndarray, o_ptrs: np.ndarray, numels
               device: torch.device, chunk_elems: int = 0) -> StagedTable:
     lib = _lib.lib()
     n = len(numels)
+    if chunk_elems == 0:
+        chunk_elems = lib.ts_ema_auto_chunk(int(numels.sum()))
     args = (t_ptrs.ctypes.data, s_ptrs.ctypes.data, o_ptrs.ctypes.data, numels.ctypes.data, n, chunk_elems)
     count = _lib.check(lib.ts_ema_plan(*args, None, 0), "ts_ema_plan(count)")
     slot = _ring(device).acquire(count)
@@ -96,13 +98,15 @@ def stage_ema(t_ptrs: np.ndarray, s_ptrs: np.ndarray, o_ptrs: np.ndarray, numels
     if count:
         nbytes = count * ENTRY_BYTES
         slot.dev[:nbytes].copy_(slot.pinned[:nbytes], non_blocking=True)
-    return StagedTable(slot, count, device)
+    return StagedTable(slot, count, chunk_elems, device)
 
 
 def stage_copy(src_ptrs: np.ndarray, dst_ptrs: np.ndarray, nbytes_arr: np.ndarray,
                device: torch.device, chunk_bytes: int = 0) -> StagedTable:
     lib = _lib.lib()
     n = len(nbytes_arr)
+    if chunk_bytes == 0:
+        chunk_bytes = lib.ts_copy_auto_chunk(int(nbytes_arr.sum()))
     args = (src_ptrs.ctypes.data, dst_ptrs.ctypes.data, nbytes_arr.ctypes.data, n, chunk_bytes)
     count = _lib.check(lib.ts_copy_plan(*args, None, 0), "ts_copy_plan(count)")
     slot = _ring(device).acquire(count)
@@ -110,7 +114,7 @@ def stage_copy(src_ptrs: np.ndarray, dst_ptrs: np.ndarray, nbytes_arr: np.ndarra
     if count:
         nbytes = count * ENTRY_BYTES
         slot.dev[:nbytes].copy_(slot.pinned[:nbytes], non_blocking=True)
-    return StagedTable(slot, count, device)
+    return StagedTable(slot, count, chunk_bytes, device)
 
 
 def copy_segments(srcs: Sequence[torch.Tensor], dsts: Sequence[torch.Tensor]) -> None:
@@ -120,6 +124,7 @@ def copy_segments(srcs: Sequence[torch.Tensor], dsts: Sequence[torch.Tensor]) ->
     device = dsts[0].device
     nbytes = np.fromiter((s.numel() * s.element_size() for s in srcs), dtype=np.int64, count=len(srcs))
     table = stage_copy(ptr_array(srcs), ptr_array(dsts), nbytes, device)
-    _lib.check(_lib.lib().ts_copy_segments(table.dev_ptr, table.n_chunks, _lib.current_stream_ptr(device)),
+    _lib.check(_lib.lib().ts_copy_segments(table.dev_ptr, table.n_chunks, table.chunk,
+                                           _lib.current_stream_ptr(device)),
                "ts_copy_segments")
     table.done()

@@ -55,7 +55,7 @@ struct NceLayout {
   int64_t npad;
   int splits;
   size_t head_bytes;
-  size_t off_rq, off_rk, off_diag, off_lpart, off_kt, off_qb, off_kb, off_opart, pair_bytes;
+  size_t off_rq, off_rk, off_diag, off_lpart, off_apart, off_kt, off_qb, off_kb, off_opart, pair_bytes;
 };
 
 inline size_t nce_align(size_t x) { return (x + 255) & ~(size_t)255; }
@@ -63,7 +63,7 @@ inline size_t nce_align(size_t x) { return (x + 255) & ~(size_t)255; }
 inline int nce_splits(int64_t npad, int n_pairs) {
   const int64_t qtiles = npad / kQTile * n_pairs;
   const int64_t ktiles = npad / kKTile;
-  int64_t s = (512 + qtiles - 1) / qtiles;  // aim for ~2 workgroups per CU
+  int64_t s = (256 + qtiles - 1) / qtiles;  // one workgroup per CU: the kernel's registers allow no more
   if (s > 16) s = 16;
   if (s > ktiles) s = ktiles;
   if (s < 1) s = 1;
@@ -80,6 +80,7 @@ inline NceLayout nce_layout(int64_t n, int64_t c, int n_pairs, bool fp32_in) {
   L.off_rk = o;       o += nce_align(L.npad * 4);
   L.off_diag = o;     o += nce_align(L.npad * 4);
   L.off_lpart = o;    o += nce_align((size_t)L.splits * L.npad * 4);
+  L.off_apart = o;    o += nce_align((size_t)L.splits * L.npad * 4);
   L.off_kt = o;       o += nce_align((size_t)c * L.npad * 2);
   L.off_qb = o;       o += fp32_in ? nce_align((size_t)L.npad * c * 2) : 0;
   L.off_kb = o;       o += fp32_in ? nce_align((size_t)L.npad * c * 2) : 0;
@@ -89,45 +90,76 @@ inline NceLayout nce_layout(int64_t n, int64_t c, int n_pairs, bool fp32_in) {
 }
 
 // ---------------------------------------------------------------------------
-// prep: 64 rows per workgroup
+// prep: 16-byte row loads, a group of C/VEC lanes per row; the K rows of the
+// workgroup pass through LDS to come out transposed
 // ---------------------------------------------------------------------------
+template <typename T, int C>
+struct NcePrep {
+  static constexpr int VEC = 16 / sizeof(T);               // elements per 16-byte load
+  static constexpr int LPR = C / VEC;                      // lanes per row (8 .. 64)
+  static constexpr int RPP = kWave / LPR;                  // rows per wavefront pass
+  static constexpr int ROWS = (4 * RPP > 16) ? 4 * RPP : 16;  // rows per workgroup
+  static constexpr int LD = C + 8;                         // bf16 per LDS row (16-byte aligned rows)
+};
+
 template <typename T, int C>
 __global__ __launch_bounds__(kNceBlock) void nce_prep_kernel(const T* __restrict__ q, const T* __restrict__ k,
                                                              int64_t n, int64_t npad, float scale2,
                                                              float* __restrict__ rq, float* __restrict__ rk,
                                                              float* __restrict__ diag, uint16_t* __restrict__ kt,
                                                              uint16_t* __restrict__ qb, uint16_t* __restrict__ kb) {
-  constexpr int ROWS = 64;
-  constexpr int LD = C + 2;  // odd number of 4-byte words per row: column reads spread over banks
-  __shared__ uint16_t tile[ROWS * LD];
+  using P = NcePrep<T, C>;
+  __shared__ __attribute__((aligned(16))) uint16_t tile[P::ROWS * P::LD];
   const int lane = threadIdx.x % kWave, w = threadIdx.x / kWave;
-  const int64_t row0 = (int64_t)blockIdx.x * ROWS;
+  const int sub = lane / P::LPR, li = lane % P::LPR;  // row within the pass, lane within the row
+  const int64_t row0 = (int64_t)blockIdx.x * P::ROWS;
 
-  for (int r = w; r < ROWS; r += kNceBlock / kWave) {
+  for (int r = w * P::RPP + sub; r < P::ROWS; r += 4 * P::RPP) {
     const int64_t row = row0 + r;
-    float sqq = 0.f, skk = 0.f, sqk = 0.f;
-    for (int f = lane; f < C; f += kWave) {
-      float qv = 0.f, kv = 0.f;
-      if (row < n) {
-        qv = to_f32(q[row * C + f]);
-        kv = to_f32(k[row * C + f]);
+    const bool live = row < n;
+    float qv[P::VEC], kv[P::VEC];
+    if (live) {
+      u32x4 rawq = *reinterpret_cast<const u32x4*>(q + row * C + li * P::VEC);
+      u32x4 rawk = *reinterpret_cast<const u32x4*>(k + row * C + li * P::VEC);
+      T tq[P::VEC], tk[P::VEC];
+      __builtin_memcpy(tq, &rawq, 16);
+      __builtin_memcpy(tk, &rawk, 16);
+#pragma unroll
+      for (int e = 0; e < P::VEC; ++e) {
+        qv[e] = to_f32(tq[e]);
+        kv[e] = to_f32(tk[e]);
       }
-      const uint16_t qbits = f32_to_bf16_bits(qv), kbits = f32_to_bf16_bits(kv);
-      sqq += qv * qv;
-      skk += kv * kv;
+    } else {
+#pragma unroll
+      for (int e = 0; e < P::VEC; ++e) qv[e] = kv[e] = 0.f;
+    }
+    float sqq = 0.f, skk = 0.f, sqk = 0.f;
+    uint16_t qbits[P::VEC], kbits[P::VEC];
+#pragma unroll
+    for (int e = 0; e < P::VEC; ++e) {
+      qbits[e] = f32_to_bf16_bits(qv[e]);
+      kbits[e] = f32_to_bf16_bits(kv[e]);
+      sqq += qv[e] * qv[e];
+      skk += kv[e] * kv[e];
       // the diagonal logit uses the values the MFMA will see
-      sqk += bf16_bits_to_f32(qbits) * bf16_bits_to_f32(kbits);
-      tile[r * LD + f] = kbits;
-      if (qb) {
-        qb[row * C + f] = qbits;
-        kb[row * C + f] = kbits;
+      sqk += bf16_bits_to_f32(qbits[e]) * bf16_bits_to_f32(kbits[e]);
+    }
+#pragma unroll
+    for (int e = 0; e < P::VEC; ++e) tile[r * P::LD + li * P::VEC + e] = kbits[e];
+    if (qb) {
+#pragma unroll
+      for (int e = 0; e < P::VEC; ++e) {
+        qb[row * C + li * P::VEC + e] = qbits[e];
+        kb[row * C + li * P::VEC + e] = kbits[e];
       }
     }
-    sqq = wave_sum(sqq);
-    skk = wave_sum(skk);
-    sqk = wave_sum(sqk);
-    if (lane == 0) {
-      const bool live = row < n;
+#pragma unroll
+    for (int off = P::LPR / 2; off > 0; off >>= 1) {
+      sqq += __shfl_xor(sqq, off, kWave);
+      skk += __shfl_xor(skk, off, kWave);
+      sqk += __shfl_xor(sqk, off, kWave);
+    }
+    if (li == 0) {
       const float a = live ? 1.f / fmaxf(sqrtf(sqq), kNormEps) : 0.f;
       const float b = live ? 1.f / fmaxf(sqrtf(skk), kNormEps) : 0.f;
       rq[row] = a;
@@ -137,11 +169,11 @@ __global__ __launch_bounds__(kNceBlock) void nce_prep_kernel(const T* __restrict
   }
   __syncthreads();
   // transposed write: K^T[f][row0 + 8*chunk .. +7], 16 bytes per store
-  for (int id = threadIdx.x; id < C * (ROWS / 8); id += kNceBlock) {
-    const int f = id / (ROWS / 8), chunk = id % (ROWS / 8);
+  for (int id = threadIdx.x; id < C * (P::ROWS / 8); id += kNceBlock) {
+    const int f = id / (P::ROWS / 8), chunk = id % (P::ROWS / 8);
     u16x8 v;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) v[e] = tile[(chunk * 8 + e) * LD + f];
+    for (int e = 0; e < 8; ++e) v[e] = tile[(chunk * 8 + e) * P::LD + f];
     *reinterpret_cast<u16x8*>(kt + (int64_t)f * npad + row0 + chunk * 8) = v;
   }
 }
@@ -165,7 +197,8 @@ __global__ __launch_bounds__(kNceBlock) void nce_main_kernel(const uint16_t* __r
                                                              const float* __restrict__ rq,
                                                              const float* __restrict__ rk, int64_t n, int64_t npad,
                                                              int splits, float scale2 /* log2(e)/tau */,
-                                                             float* __restrict__ lpart, float* __restrict__ opart) {
+                                                             float* __restrict__ lpart, float* __restrict__ apart,
+                                                             float* __restrict__ opart) {
   using Smem = NceSmem<C>;
   __shared__ __attribute__((aligned(16))) Smem sm;
   constexpr int KK = C / 16;  // contraction steps of S^T
@@ -195,7 +228,8 @@ __global__ __launch_bounds__(kNceBlock) void nce_main_kernel(const uint16_t* __r
   for (int fb = 0; fb < FB; ++fb)
 #pragma unroll
     for (int i = 0; i < 16; ++i) oacc[fb][i] = 0.f;
-  float lsum = 0.f;
+  float lsum = 0.f;  // sum_j P_ij
+  float asum = 0.f;  // sum_j P_ij x_ij (x: logit in the log2 domain) = <qh_i, sum_j P_ij kh_j> * log2e/tau
 
   // global -> register staging of one key tile (K rows, K^T rows, rk)
   constexpr int KCH = kKTile * C / 8 / kNceBlock;  // 16-byte chunks per thread, K tile
@@ -270,9 +304,11 @@ __global__ __launch_bounds__(kNceBlock) void nce_main_kernel(const uint16_t* __r
       for (int j = 0; j < 4; ++j) {
         const int i = 4 * g + j;
         const float rkj = rk4[j];
-        float p = exp2f(sacc[i] * (sc_i * rkj) - scale2);
+        const float x = sacc[i] * (sc_i * rkj);
+        float p = exp2f(x - scale2);
         if (key0 + 8 * g + 4 * h + j >= n) p = 0.f;
         lsum += p;
+        asum += p * x;
         pb[g / 2][(g % 2) * 4 + j] = (__bf16)(p * rkj);
       }
     }
@@ -298,7 +334,11 @@ __global__ __launch_bounds__(kNceBlock) void nce_main_kernel(const uint16_t* __r
 
   // partial results, register-native order: [split][q tile of 32][fb][i][lane]
   const float ltot = lsum + __shfl_xor(lsum, 32, kWave);
-  if (h == 0) lpart[(int64_t)split * npad + qtile * kQTile + w * 32 + col] = ltot;
+  const float atot = asum + __shfl_xor(asum, 32, kWave);
+  if (h == 0) {
+    lpart[(int64_t)split * npad + qtile * kQTile + w * 32 + col] = ltot;
+    apart[(int64_t)split * npad + qtile * kQTile + w * 32 + col] = atot;
+  }
   const int64_t tile32 = qtile * (kQTile / 32) + w;
   float* op = opart + (((int64_t)split * (npad / 32) + tile32) * FB) * 16 * kWave;
 #pragma unroll
@@ -308,7 +348,9 @@ __global__ __launch_bounds__(kNceBlock) void nce_main_kernel(const uint16_t* __r
 }
 
 // ---------------------------------------------------------------------------
-// combine: one wavefront per 32 q rows
+// combine: one wavefront per (32 q rows, 32-feature block); purely
+// element-wise, because <qh_i, dqh_i> follows from the row sums:
+//   <qh_i, sum_j P_ij kh_j> = (tau/log2e) A_i / l_i,  <qh_i, kh_i> = (tau/log2e) diag_i
 // ---------------------------------------------------------------------------
 template <typename T, int C>
 __global__ __launch_bounds__(kNceBlock) void nce_combine_kernel(const T* __restrict__ q, const T* __restrict__ k,
@@ -316,68 +358,57 @@ __global__ __launch_bounds__(kNceBlock) void nce_combine_kernel(const T* __restr
                                                                 const float* __restrict__ rk,
                                                                 const float* __restrict__ diag,
                                                                 const float* __restrict__ lpart,
+                                                                const float* __restrict__ apart,
                                                                 const float* __restrict__ opart, int64_t n,
                                                                 int64_t npad, int splits, float scale2,
                                                                 float* __restrict__ row_loss, T* __restrict__ dq) {
   constexpr int FB = C / 32;
   const int lane = threadIdx.x % kWave, w = threadIdx.x / kWave;
   const int col = lane % 32, h = lane / 32;
-  const int64_t tile32 = (int64_t)blockIdx.x * (kNceBlock / kWave) + w;
+  const int64_t item = (int64_t)blockIdx.x * (kNceBlock / kWave) + w;
+  const int64_t tile32 = item / FB;
+  const int fb = (int)(item % FB);
   if (tile32 >= npad / 32) return;
   const int64_t row = tile32 * 32 + col;
   const bool live = row < n;
 
-  float l = 0.f;
-  for (int s = 0; s < splits; ++s) l += lpart[(int64_t)s * npad + row];
-  if (h == 0) row_loss[row] = live ? kNceLn2 * (scale2 + log2f(l) - diag[row]) : 0.f;
+  float l = 0.f, A = 0.f;
+  for (int s = 0; s < splits; ++s) {
+    l += lpart[(int64_t)s * npad + row];
+    A += apart[(int64_t)s * npad + row];
+  }
+  const float d = diag[row];
+  if (fb == 0 && h == 0) row_loss[row] = live ? kNceLn2 * (scale2 + log2f(l) - d) : 0.f;
   if (!dq) return;
 
-  const float inv_l = live ? 1.f / l : 0.f;
+  float o[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) o[i] = 0.f;
+  for (int s = 0; s < splits; ++s) {
+    const float* op = opart + (((int64_t)s * (npad / 32) + tile32) * FB + fb) * 16 * kWave;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) o[i] += op[i * kWave + lane];
+  }
+  if (!live) return;
+  const float inv_l = 1.f / l;
   const float rq_i = rq[row], rk_i = rk[row];
   const float gn = 2.f / (float)n;
-
-  // dqh and qh for the features this lane holds: f = 32 fb + 8 g + 4 h + j
-  float dqh[FB][16], qh[FB][16];
-  float dot = 0.f;
-#pragma unroll
-  for (int fb = 0; fb < FB; ++fb) {
-    float o[16];
-#pragma unroll
-    for (int i = 0; i < 16; ++i) o[i] = 0.f;
-    for (int s = 0; s < splits; ++s) {
-      const float* op = opart + (((int64_t)s * (npad / 32) + tile32) * FB + fb) * 16 * kWave;
-#pragma unroll
-      for (int i = 0; i < 16; ++i) o[i] += op[i * kWave + lane];
-    }
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int i = 4 * g + j;
-        const int f = 32 * fb + 8 * g + 4 * h + j;
-        const float kv = live ? to_f32(k[row * C + f]) : 0.f;
-        const float qv = live ? to_f32(q[row * C + f]) : 0.f;
-        dqh[fb][i] = gn * (o[i] * inv_l - kv * rk_i);
-        qh[fb][i] = qv * rq_i;
-        dot += qh[fb][i] * dqh[fb][i];
-      }
-    }
-  }
-  dot += __shfl_xor(dot, 32, kWave);
-  // below eps the norm is the constant eps and normalize() is linear
+  // below eps the norm is the constant eps and normalize() is linear: no projection
   const bool clamped = rq_i >= 1.f / kNormEps;
-  if (clamped) dot = 0.f;
-  if (!live) return;
+  const float dot = clamped ? 0.f : gn * (A * inv_l - d) / scale2;
 #pragma unroll
-  for (int fb = 0; fb < FB; ++fb)
+  for (int g = 0; g < 4; ++g) {
+    const int f0 = 32 * fb + 8 * g + 4 * h;  // this lane holds features f0 .. f0+3 of its row
+    T kv[4], qv[4], out[4];
+    __builtin_memcpy(kv, k + row * C + f0, sizeof(kv));
+    __builtin_memcpy(qv, q + row * C + f0, sizeof(qv));
 #pragma unroll
-    for (int g = 0; g < 4; ++g)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int i = 4 * g + j;
-        const int f = 32 * fb + 8 * g + 4 * h + j;
-        dq[row * C + f] = from_f32<T>((dqh[fb][i] - qh[fb][i] * dot) * rq_i);
-      }
+    for (int j = 0; j < 4; ++j) {
+      const float dqh = gn * (o[4 * g + j] * inv_l - to_f32(kv[j]) * rk_i);
+      out[j] = from_f32<T>((dqh - to_f32(qv[j]) * rq_i * dot) * rq_i);
+    }
+    __builtin_memcpy(dq + row * C + f0, out, sizeof(out));
+  }
 }
 
 template <typename T, int C>
@@ -388,14 +419,15 @@ int nce_run_pair(const void* q, const void* k, void* dq, int64_t n, float tau, c
   float* rk = (float*)(ws + L.off_rk);
   float* diag = (float*)(ws + L.off_diag);
   float* lpart = (float*)(ws + L.off_lpart);
+  float* apart = (float*)(ws + L.off_apart);
   uint16_t* kt = (uint16_t*)(ws + L.off_kt);
   uint16_t* qb = kF32 ? (uint16_t*)(ws + L.off_qb) : nullptr;
   uint16_t* kb = kF32 ? (uint16_t*)(ws + L.off_kb) : nullptr;
   float* opart = (float*)(ws + L.off_opart);
   const float scale2 = kNceLog2e / tau;
 
-  hipLaunchKernelGGL((nce_prep_kernel<T, C>), dim3((unsigned)(L.npad / 64)), dim3(kNceBlock), 0, stream,
-                     (const T*)q, (const T*)k, n, L.npad, scale2, rq, rk, diag, kt, qb, kb);
+  hipLaunchKernelGGL((nce_prep_kernel<T, C>), dim3((unsigned)(L.npad / NcePrep<T, C>::ROWS)), dim3(kNceBlock), 0,
+                     stream, (const T*)q, (const T*)k, n, L.npad, scale2, rq, rk, diag, kt, qb, kb);
   int rc = check_launch();
   if (rc) return rc;
   const uint16_t* qsrc = kF32 ? qb : (const uint16_t*)q;
@@ -403,13 +435,13 @@ int nce_run_pair(const void* q, const void* k, void* dq, int64_t n, float tau, c
   // with bf16 copies the rows beyond n exist (zero); the kernel guards by n either way
   hipLaunchKernelGGL((nce_main_kernel<C>), dim3((unsigned)(L.npad / kQTile), (unsigned)L.splits),
                      dim3(kNceBlock), 0, stream, qsrc, ksrc, kt, rq, rk, n, L.npad, L.splits, scale2, lpart,
-                     opart);
+                     apart, opart);
   rc = check_launch();
   if (rc) return rc;
-  const int64_t tiles32 = L.npad / 32;
-  hipLaunchKernelGGL((nce_combine_kernel<T, C>), dim3((unsigned)((tiles32 + 3) / 4)), dim3(kNceBlock), 0, stream,
-                     (const T*)q, (const T*)k, rq, rk, diag, lpart, opart, n, L.npad, L.splits, scale2, row_loss,
-                     (T*)dq);
+  const int64_t items = L.npad / 32 * (C / 32);  // a multiple of 4: npad is a multiple of 128
+  hipLaunchKernelGGL((nce_combine_kernel<T, C>), dim3((unsigned)(items / 4)), dim3(kNceBlock), 0, stream,
+                     (const T*)q, (const T*)k, rq, rk, diag, lpart, apart, opart, n, L.npad, L.splits, scale2,
+                     row_loss, (T*)dq);
   return check_launch();
 }
 

@@ -22,8 +22,7 @@ extern "C" {
 
 int64_t ts_ema_auto_chunk(int64_t total_elems) {
   if (total_elems <= 0) return 4096;
-  int64_t c = round_up((total_elems + kTargetChunks - 1) / kTargetChunks, 1024);
-  if (c < 4096) c = 4096;
+  int64_t c = round_up((total_elems + kTargetChunks - 1) / kTargetChunks, 4096);
   if (c > (int64_t)1 << 30) c = (int64_t)1 << 30;
   return c;
 }
@@ -70,8 +69,7 @@ int64_t ts_ema_plan(const void* const* t, const void* const* s, void* const* out
 
 int64_t ts_copy_auto_chunk(int64_t total_bytes) {
   if (total_bytes <= 0) return 16384;
-  int64_t c = round_up((total_bytes + kTargetChunks - 1) / kTargetChunks, 4096);
-  if (c < 16384) c = 16384;
+  int64_t c = round_up((total_bytes + kTargetChunks - 1) / kTargetChunks, 16384);
   if (c > (int64_t)1 << 31) c = (int64_t)1 << 31;
   return c;
 }
