@@ -132,11 +132,11 @@ int ts_copy_segments(const ts_copy_chunk* table_dev, int64_t n_chunks, int64_t c
 /* s, t, grad: [n_rows, V] row-major with leading dimensions ld_* in         */
 /* elements; dtype TS_F32 / TS_BF16 / TS_F16 (same for all three);           */
 /* accumulation is fp32.  grad may be NULL (loss only).                      */
-/* workspace: ts_kd_workspace_bytes(n_rows) bytes, 16-byte aligned, contents */
-/* irrelevant on entry.  loss_out: one float.                                */
+/* workspace: ts_kd_workspace_bytes(n_rows, V, dtype) bytes, 32-byte aligned,  */
+/* contents irrelevant on entry.  loss_out: one float.                       */
 /* ------------------------------------------------------------------------ */
 
-size_t ts_kd_workspace_bytes(int64_t n_rows);
+size_t ts_kd_workspace_bytes(int64_t n_rows, int64_t V, int dtype);
 
 int ts_kd_fwd_bwd(const void* s, const void* t, const uint8_t* row_mask, int64_t n_rows,
                   int64_t V, int64_t ld_s, int64_t ld_t, float inv_T, float loss_scale,

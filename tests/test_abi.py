@@ -160,6 +160,7 @@ def test_device_entry_points_validate_before_launching():
     assert lib.ts_bn_apply(p, None, p, p, None, None, 2, 3, 4, 0, 1e-5, None) == -1
     assert lib.ts_bn_backward(p, p, p, p, None, p, p, None, p, 2, 3, 4, 1, None) == -1
     assert lib.ts_scale_rows(p, 4, 10, 9, p, 0, None) == -1
-    assert lib.ts_kd_workspace_bytes(0) == 16 and lib.ts_kd_workspace_bytes(5) == 48
+    assert lib.ts_kd_workspace_bytes(0, 100, 0) == 32 and lib.ts_kd_workspace_bytes(5, 100, 0) == 96
+    assert lib.ts_kd_workspace_bytes(4096, 30522, 1) == 32 + 2 * 4096 * 4 + 4096 * 4 * 32  # 4 parts per wide row
     assert lib.ts_infonce_workspace_bytes(4096, 256, 1) > 4096 * 256 * 4
     assert lib.ts_infonce_workspace_bytes(4096, 256, 3) == 0

@@ -30,7 +30,7 @@ SIGNATURES = {
     "ts_copy_auto_chunk": (c_int64, [c_int64]),
     "ts_copy_plan": (c_int64, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_int64]),
     "ts_copy_segments": (c_int, [c_void_p, c_int64, c_int64, c_void_p]),
-    "ts_kd_workspace_bytes": (c_size_t, [c_int64]),
+    "ts_kd_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int]),
     "ts_kd_fwd_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_float,
                               c_float, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_void_p]),
     "ts_scale_rows": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_int, c_void_p]),

@@ -43,12 +43,13 @@ __device__ __forceinline__ float to_f32(f16_t x) { return (float)x.v; }
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t bits) { return __uint_as_float(bits << 16); }
 
-// Round-to-nearest-even fp32 -> bf16, NaN kept quiet (what torch's cast does).
+// Round-to-nearest-even fp32 -> bf16 (what torch's cast does); the compiler
+// emits gfx950's v_cvt_pk_bf16_f32 for this conversion.
 __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (uint16_t)(u >> 16);
+  const __bf16 b = (__bf16)f;
+  uint16_t u;
+  __builtin_memcpy(&u, &b, 2);
+  return u;
 }
 
 template <typename T>
@@ -69,6 +70,12 @@ __device__ __forceinline__ f16_t from_f32<f16_t>(float x) {
   r.v = (_Float16)x;
   return r;
 }
+
+// 2^x on the hardware transcendental unit (v_exp_f32, 1 ulp).  Results below
+// the normal range flush to zero, which is what a soft-max term that small
+// contributes anyway; the library exp2f spends several extra instructions on
+// rescaling them.
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 // ---- wavefront / block reductions -----------------------------------------
 

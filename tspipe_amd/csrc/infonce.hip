@@ -305,7 +305,7 @@ __global__ __launch_bounds__(kNceBlock) void nce_main_kernel(const uint16_t* __r
         const int i = 4 * g + j;
         const float rkj = rk4[j];
         const float x = sacc[i] * (sc_i * rkj);
-        float p = exp2f(x - scale2);
+        float p = fast_exp2(x - scale2);
         if (key0 + 8 * g + 4 * h + j >= n) p = 0.f;
         lsum += p;
         asum += p * x;

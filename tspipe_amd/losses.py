@@ -74,7 +74,7 @@ class _KDSoftTargetFn(torch.autograd.Function):
         need_grad = ctx.needs_input_grad[0]
         lib = _lib.lib()
         dev = s.device
-        ws = torch.empty(lib.ts_kd_workspace_bytes(rows), dtype=torch.uint8, device=dev)
+        ws = torch.empty(lib.ts_kd_workspace_bytes(rows, V, _lib.dtype_code(s.dtype)), dtype=torch.uint8, device=dev)
         loss = torch.empty((), dtype=torch.float32, device=dev)
         grad = torch.empty_like(s) if need_grad else None
         with torch.cuda.device(dev):
