@@ -156,3 +156,28 @@ def test_gather_large_cfg3_shape(device):
 def test_gather_rejects_host_tensors():
     with pytest.raises(TypeError):
         ta.gather([ta.Batch(torch.zeros(2, 2)), ta.Batch(torch.zeros(2, 2))])
+
+
+def test_ema_output_arenas_are_recycled_only_when_unreferenced(device):
+    from tspipe_amd import ema as ema_mod
+    ema_mod.release_pool()
+    teacher, student = param_lists([(64, 8), (16,), (32, 4)], 9)
+    t_dev = [t.to(device) for t in teacher]
+    s_dev = [s.to(device) for s in student]
+    a = ta.momentum_update(0.9, s_dev, t_dev)
+    a_ptr = a[0].data_ptr()
+    b = ta.momentum_update(0.8, s_dev, t_dev)          # `a` is still held: must not be overwritten
+    assert b[0].data_ptr() != a_ptr
+    want_a = ts_oracle.ema_update(0.9, student, teacher)
+    assert all(bits_equal(x, w) for x, w in zip(a, want_a))
+    alias = a[1].view(-1)                               # an alias survives the list
+    del a
+    c = ta.momentum_update(0.7, s_dev, t_dev)
+    assert c[0].data_ptr() != a_ptr                     # storage still aliased: no reuse
+    assert bits_equal(alias, want_a[1].view(-1))
+    del alias, c
+    d = ta.momentum_update(0.6, s_dev, t_dev)
+    assert d[0].data_ptr() in (a_ptr, b[0].data_ptr()) or True  # reuse is allowed now, never required
+    assert all(bits_equal(x, w) for x, w in zip(d, ts_oracle.ema_update(0.6, student, teacher)))
+    assert all(bits_equal(x, w) for x, w in zip(b, ts_oracle.ema_update(0.8, student, teacher)))
+    ema_mod.release_pool()

@@ -9,6 +9,9 @@ implementations of that plug-in are
 (benchmarks/moco-v3/main.py:133-144): per tensor,
 ``t.clone() * m + s * (1. - m)``, returned as a new list.
 """
+import operator
+import sys
+import threading
 from typing import Iterable, List, Optional, Sequence
 
 import numpy as np
@@ -22,47 +25,57 @@ kernel_events = None
 
 
 _F32 = torch.float32
+_shape_of = operator.attrgetter("shape")
+_dtype_of = operator.attrgetter("dtype")
+_device_of = operator.attrgetter("device")
+_use_count = getattr(torch._C, "_storage_Use_Count", None)
 
 
 def _prepare(online: Iterable[Optional[torch.Tensor]], target: Iterable[torch.Tensor], skip_none: bool):
     """Pairs the lists up as ``zip`` does, validates them and makes them dense.
+    Returns (students, teachers, shapes).
 
-    Written as a few flat comprehensions: at 150+ tensors per call the Python
-    work here costs more than the kernel, so every per-tensor call counts."""
+    At 150+ tensors per call the Python work here costs more than the kernel,
+    so the checks run as C-level ``map`` calls over the lists rather than as a
+    Python loop per tensor."""
     pairs = list(zip(online, target))
     if any(s is None for s, _ in pairs):
         if not skip_none:
             raise TypeError("online parameter is None (use calculate_updated_momentum_encoder to skip those)")
         pairs = [p for p in pairs if p[0] is not None]  # benchmarks/moco-v3/main.py:139-140
     if not pairs:
-        return [], []
-    students = [s for s, _ in pairs]
-    teachers = [t for _, t in pairs]
-    dev = teachers[0].device
-    if dev.type != "cuda":
-        raise TypeError("EMA kernel needs device tensors (the pipeline asserts the same, tspipe/gpu_task.py:407)")
-    if not all(t.dtype is _F32 and s.dtype is _F32 for s, t in pairs):
-        bad = next((s.dtype, t.dtype) for s, t in pairs if not (t.dtype is _F32 and s.dtype is _F32))
-        raise TypeError(f"EMA kernel is fp32 (got student {bad[0]}, teacher {bad[1]})")
-    if not all(t.device == dev and s.device == dev for s, t in pairs):
-        if any(not t.is_cuda or not s.is_cuda for s, t in pairs):
+        return [], [], ()
+    students = [p[0] for p in pairs]
+    teachers = [p[1] for p in pairs]
+    devices = set(map(_device_of, teachers)) | set(map(_device_of, students))
+    if len(devices) != 1:
+        if any(d.type != "cuda" for d in devices):
             raise TypeError("EMA kernel needs device tensors (the pipeline asserts the same, tspipe/gpu_task.py:407)")
         raise ValueError("teacher and student parameters live on different devices")
-    if [t.shape for t in teachers] != [s.shape for s in students]:
+    if next(iter(devices)).type != "cuda":
+        raise TypeError("EMA kernel needs device tensors (the pipeline asserts the same, tspipe/gpu_task.py:407)")
+    dtypes = set(map(_dtype_of, teachers)) | set(map(_dtype_of, students))
+    if dtypes != {_F32}:
+        raise TypeError(f"EMA kernel is fp32 (got {sorted(map(str, dtypes))})")
+    shapes = tuple(map(_shape_of, teachers))
+    if shapes != tuple(map(_shape_of, students)):
         bad = next((tuple(t.shape), tuple(s.shape)) for s, t in pairs if t.shape != s.shape)
         raise ValueError(f"teacher/student shapes differ: {bad[0]} vs {bad[1]}")
-    if not all(t.is_contiguous() and s.is_contiguous() for s, t in pairs):
+    if not (all(map(torch.Tensor.is_contiguous, teachers)) and all(map(torch.Tensor.is_contiguous, students))):
         students = [s if s.is_contiguous() else s.detach().contiguous() for s in students]
         teachers = [t if t.is_contiguous() else t.detach().contiguous() for t in teachers]
-    return students, teachers
+    return students, teachers, shapes
+
+
+def _ptrs(tensors: Sequence[torch.Tensor]) -> np.ndarray:
+    return np.array(list(map(torch.Tensor.data_ptr, tensors)), dtype=np.uint64)
 
 
 def _launch(m: float, students: Sequence[torch.Tensor], teachers: Sequence[torch.Tensor],
-            outs: Sequence[torch.Tensor], numels: np.ndarray) -> None:
+            out_ptrs: np.ndarray, numels: np.ndarray) -> None:
     device = teachers[0].device
     with torch.cuda.device(device):
-        table = _tables.stage_ema(_tables.ptr_array(teachers), _tables.ptr_array(students),
-                                  _tables.ptr_array(outs), numels, device)
+        table = _tables.stage_ema(_ptrs(teachers), _ptrs(students), out_ptrs, numels, device)
         timed = kernel_events is not None
         if timed:
             start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -78,32 +91,85 @@ def _launch(m: float, students: Sequence[torch.Tensor], teachers: Sequence[torch
         table.done()
 
 
-def _new_outputs(teachers: Sequence[torch.Tensor], numels: np.ndarray) -> List[torch.Tensor]:
-    """One flat allocation carved into views shaped like the teachers, each
-    starting on a 16-byte boundary."""
+class _Arena:
+    """One flat output allocation and its views, shaped like a parameter list."""
+    __slots__ = ("flat", "views", "ptrs", "numels", "stream")
+
+    def __init__(self, teachers: Sequence[torch.Tensor]):
+        device = teachers[0].device
+        # like a block of torch's caching allocator, the arena belongs to the
+        # stream it was made on and is only handed out again on that stream
+        self.stream = torch.cuda.current_stream(device).cuda_stream
+        numels = np.array(list(map(torch.Tensor.numel, teachers)), dtype=np.int64)
+        if not (numels & 3).any():
+            # every size is a multiple of 4 elements: pieces sit back to back,
+            # each on a 16-byte boundary, and torch's C++ unflatten makes the views
+            self.flat = torch.empty(int(numels.sum()), dtype=_F32, device=device)
+            self.views = list(torch._C._nn.unflatten_dense_tensors(self.flat, teachers))
+        else:
+            padded = ((numels + 3) & ~3).tolist()
+            self.flat = torch.empty(sum(padded), dtype=_F32, device=device)
+            pieces = self.flat.split(padded)
+            self.views = [p[:t.numel()].view(t.shape) for p, t in zip(pieces, teachers)]
+        self.ptrs = _ptrs(self.views)
+        self.numels = numels
+
+    def is_free(self) -> bool:
+        """True when nothing outside this arena can reach its memory: no view
+        object is referenced elsewhere and the storage has no further alias."""
+        storage = self.flat.untyped_storage()
+        if _use_count(storage._cdata) != len(self.views) + 2:  # flat + views + the wrapper just made
+            return False
+        return all(c == 2 for c in map(sys.getrefcount, self.views))
+
+
+# Output arenas whose tensors the caller has dropped are handed out again
+# (same tensor objects, same memory): making 150+ view tensors costs more host
+# time than the kernel takes.  Keyed by (device, stream, shapes); a handful per key,
+# matching the few parameter versions a pipeline keeps alive.
+_POOL_LIMIT = 6
+_pool = {}
+_pool_lock = threading.Lock()
+
+
+def release_pool() -> None:
+    """Drops every cached output arena (memory returns to torch's allocator
+    once the caller's own references are gone)."""
+    with _pool_lock:
+        _pool.clear()
+
+
+def _acquire_arena(teachers: Sequence[torch.Tensor], shapes) -> _Arena:
+    if _use_count is None:
+        return _Arena(teachers)
     device = teachers[0].device
-    if not (numels & 3).any():
-        # every size is a multiple of 4 elements: pieces are back to back and
-        # torch's C++ unflatten makes all the views in one call
-        flat = torch.empty(int(numels.sum()), dtype=_F32, device=device)
-        return list(torch._C._nn.unflatten_dense_tensors(flat, teachers))
-    padded = ((numels + 3) & ~3).tolist()
-    flat = torch.empty(sum(padded), dtype=_F32, device=device)
-    pieces = flat.split(padded)
-    return [p[:t.numel()].view(t.shape) for p, t in zip(pieces, teachers)]
+    key = (device, torch.cuda.current_stream(device).cuda_stream, shapes)
+    with _pool_lock:
+        arenas = _pool.setdefault(key, [])
+        for arena in arenas:
+            if arena.is_free():
+                return arena
+        arena = _Arena(teachers)
+        arenas.append(arena)
+        if len(arenas) > _POOL_LIMIT:
+            arenas.pop(0)  # stays alive for as long as its user holds it
+        return arena
 
 
 @torch.no_grad()
 def momentum_update(m: float, online_new_param: Iterable[Optional[torch.Tensor]],
                     target_param: Iterable[torch.Tensor], skip_none: bool = False) -> List[torch.Tensor]:
-    """Returns new tensors ``t*m + s*(1-m)``; the inputs are left untouched."""
-    students, teachers = _prepare(online_new_param, target_param, skip_none)
+    """Returns new tensors ``t*m + s*(1-m)``; the inputs are left untouched.
+
+    The results are views of one flat allocation.  "New" means not aliased by
+    anything the caller still holds: tensors of an earlier result may be handed
+    out again once the caller has dropped every reference to them."""
+    students, teachers, shapes = _prepare(online_new_param, target_param, skip_none)
     if not teachers:
         return []
-    numels = np.fromiter((t.numel() for t in teachers), dtype=np.int64, count=len(teachers))
-    outs = _new_outputs(teachers, numels)
-    _launch(m, students, teachers, outs, numels)
-    return outs
+    arena = _acquire_arena(teachers, shapes)
+    _launch(m, students, teachers, arena.ptrs, arena.numels)
+    return list(arena.views)
 
 
 def calculate_target_network_parameters(m, online_new_param, target_param=None):
@@ -123,11 +189,11 @@ def update_target_network_parameters_(online_params: Iterable[torch.Tensor],
     ``param_k.data = param_k.data * m + param_q.data * (1. - m)``
     (benchmarks/byol/trainer.py:43-49, benchmarks/moco-v3/moco/builder.py:57-61)."""
     target_params = list(target_params)
-    students, teachers = _prepare(online_params, target_params, skip_none=False)
+    students, teachers, _ = _prepare(online_params, target_params, skip_none=False)
     if not teachers:
         return
-    numels = np.fromiter((t.numel() for t in teachers), dtype=np.int64, count=len(teachers))
-    _launch(m, students, teachers, teachers, numels)
+    numels = np.array(list(map(torch.Tensor.numel, teachers)), dtype=np.int64)
+    _launch(m, students, teachers, _ptrs(teachers), numels)
     for live, work in zip(target_params, teachers):
         if work.data_ptr() != live.data_ptr():  # a non-contiguous parameter was densified
             live.detach().copy_(work)
