@@ -119,27 +119,48 @@ def run_step_benchmark(steps, warmup, dev):
     }
 
 
+def _time_stream(fn, iters, warmup=5):
+    """Average milliseconds per call of fn() over `iters` back-to-back calls,
+    one pair of HIP events around the whole batch on the current stream.  The
+    calls go straight to the C ABI with preallocated buffers (about 10 us of
+    host time each), so for kernels longer than that the figure is device time."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(iters):
+        fn()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / iters
+
+
 def run_kernel_table(dev):
-    """Stand-alone timings of each kernel at the other configurations."""
+    """Stand-alone device timings of each kernel at the other configurations,
+    called through the C ABI with preallocated outputs and workspaces."""
     import torch
     import tspipe_amd as ta
-    from tspipe_amd import _lib
+    from tspipe_amd import _lib, _tables
+    from tspipe_amd import ema as ema_mod
     numel, r18, vit = _shapes()
+    lib = _lib.lib()
     out = {}
     g = torch.Generator().manual_seed(0)
+    stream = _lib.current_stream_ptr(dev)
 
-    def gbs(nbytes, ms):
-        return round(nbytes / (ms * 1e-3) / 1e9, 1)
-
-    def entry(nbytes, t, note=None):
-        med, mean, best = t
-        e = {"ms_median": round(med, 4), "ms_min": round(best, 4), "GB/s": gbs(nbytes, med),
-             "frac_hbm_peak": round(gbs(nbytes, med) / HBM_PEAK_GBS, 4), "algorithmic_bytes": nbytes}
+    def entry(nbytes, ms, note=None, launches=None):
+        gbs = nbytes / (ms * 1e-3) / 1e9
+        e = {"ms": round(ms, 4), "GB/s": round(gbs, 1), "frac_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
+             "algorithmic_bytes": nbytes}
+        if launches:
+            e["kernel_launches"] = launches
         if note:
             e["note"] = note
         return e
 
-    # EMA, stand-alone (no concurrent loss), both parameter lists
+    # EMA, stand-alone (no concurrent loss), both parameter lists; kernel-only events
     for name, shapes, m in (("ema_vit_base", vit, 0.99), ("ema_resnet18", r18, 0.996)):
         teacher = [(torch.randn(s, generator=g) * 0.02).to(dev) for s in shapes]
         student = [(torch.randn(s, generator=g) * 0.02).to(dev) for s in shapes]
@@ -147,7 +168,6 @@ def run_kernel_table(dev):
 
         def f():
             st["t"] = ta.calculate_target_network_parameters(m, student, st["t"])
-        from tspipe_amd import ema as ema_mod
         for _ in range(5):
             f()
         torch.cuda.synchronize()
@@ -159,77 +179,110 @@ def run_kernel_table(dev):
         ema_mod.kernel_events = None
         nbytes = 12 * sum(numel(s) for s in shapes)
         note = "working set below the 256 MB Infinity Cache: not an HBM figure" if name == "ema_resnet18" else None
-        out[name] = entry(nbytes, (statistics.median(ms), sum(ms) / len(ms), min(ms)), note)
+        out[name] = entry(nbytes, statistics.median(ms), note, 1)
         del teacher, student, st
+    ema_mod.release_pool()
+
+    def kd_call(s, t, mask, T, grad):
+        rows, V = s.shape[0] * (s.shape[1] if s.dim() == 3 else 1), s.shape[-1]
+        code = _lib.dtype_code(s.dtype)
+        ws = torch.empty(lib.ts_kd_workspace_bytes(rows, V, code), dtype=torch.uint8, device=dev)
+        loss = torch.empty((), device=dev)
+        mptr = None if mask is None else mask.view(torch.uint8).data_ptr()
+
+        def f():
+            _lib.check(lib.ts_kd_fwd_bwd(s.data_ptr(), t.data_ptr(), mptr, rows, V, V, V, 1.0 / T, T * T, ws.data_ptr(),
+                                         loss.data_ptr(), grad.data_ptr(), V, code, stream), "ts_kd_fwd_bwd")
+        f.keep = (ws, loss)
+        return f
 
     # KD small (cfg2) and a scaled shape for a bandwidth figure
     for name, rows in (("kd_256x100_f32", 256), ("kd_65536x100_f32", 65536)):
-        s = (torch.randn(rows, 100, generator=g) * 3).to(dev).requires_grad_()
+        s = (torch.randn(rows, 100, generator=g) * 3).to(dev)
         t = (torch.randn(rows, 100, generator=g) * 3).to(dev)
-
-        def f():
-            s.grad = None
-            ta.kd_soft_target_loss(s, t, 4.0).backward()
-        out[name] = entry(3 * rows * 100 * 4, _time_gpu(f, 50), "latency-bound" if rows == 256 else None)
+        f = kd_call(s, t, None, 4.0, torch.empty_like(s))
+        out[name] = entry(3 * rows * 100 * 4, _time_stream(f, 50),
+                          "latency-bound: 2 launches of a few us each" if rows == 256 else None, 2)
 
     # DistilBERT-shaped masked KD (cfg3) after a gather of 4 micro-batches
     pieces_s = [(torch.randn(8, 128, 30522, generator=g) * 2).to(torch.bfloat16).to(dev) for _ in range(4)]
     pieces_t = [(torch.randn(8, 128, 30522, generator=g) * 2).to(torch.bfloat16).to(dev) for _ in range(4)]
     mask = (torch.rand(32, 128, generator=g) < 0.15).to(dev)
     n_sel = int(mask.sum().item())
-    batches = [ta.Batch(p) for p in pieces_s]
-    out["gather_4x62.5MB_bf16"] = entry(2 * 250036224, _time_gpu(lambda: ta.gather(batches), 20))
-    s_full = ta.gather(batches).requires_grad_()
+    s_full = torch.empty(32, 128, 30522, dtype=torch.bfloat16, device=dev)
+    dsts = list(s_full.chunk(4))
+    for i in range(25):
+        if i == 5:
+            torch.cuda.synchronize()
+            _tables.kernel_events = []
+        _tables.copy_segments(pieces_s, dsts)
+    torch.cuda.synchronize()
+    ms = _event_ms(_tables.kernel_events)
+    _tables.kernel_events = None
+    out["gather_4x62.5MB_bf16"] = entry(2 * 250036224, statistics.median(ms), "kernel-only events", 1)
     t_full = ta.gather([ta.Batch(p) for p in pieces_t])
-    del pieces_s, pieces_t, batches
-
-    def f():
-        s_full.grad = None
-        ta.distil_ce_loss(s_full, t_full, mask, 2.0).backward()
+    del pieces_s, pieces_t
     row_b = 30522 * 2
-    out["kd_masked_32x128x30522_bf16"] = entry(3 * n_sel * row_b + (4096 - n_sel) * row_b, _time_gpu(f, 20),
-                                               f"n_sel={n_sel}; bytes = 3 rows r/r/w for selected + zero-fill of the rest")
-    del s_full, t_full
+    f = kd_call(s_full, t_full, mask, 2.0, torch.empty_like(s_full))
+    out["kd_masked_32x128x30522_bf16"] = entry(3 * n_sel * row_b + (4096 - n_sel) * row_b, _time_stream(f, 30),
+                                               f"n_sel={n_sel}; bytes = read s,t + write grad for selected rows, "
+                                               f"zero-fill of the other rows", 4)
+    del s_full, t_full, f
 
     # InfoNCE (cfg4), single pair
-    q = torch.nn.functional.normalize(torch.randn(4096, 256, generator=g), dim=1).to(torch.bfloat16).to(dev).requires_grad_()
+    q = torch.nn.functional.normalize(torch.randn(4096, 256, generator=g), dim=1).to(torch.bfloat16).to(dev)
     k = torch.nn.functional.normalize(torch.randn(4096, 256, generator=g), dim=1).to(torch.bfloat16).to(dev)
+    ws = torch.empty(lib.ts_infonce_workspace_bytes(4096, 256, 1), dtype=torch.uint8, device=dev)
+    loss, dq = torch.empty((), device=dev), torch.empty_like(q)
 
     def f():
-        q.grad = None
-        ta.infonce_loss(q, k, 0.2).backward()
-    med, mean, best = _time_gpu(f, 50)
+        _lib.check(lib.ts_infonce_fwd_bwd(q.data_ptr(), k.data_ptr(), None, None, 4096, 256, 0.2, ws.data_ptr(),
+                                          loss.data_ptr(), dq.data_ptr(), None, _lib.TS_BF16, stream), "ts_infonce_fwd_bwd")
+    ms = _time_stream(f, 50)
     flops = 2 * 2 * 4096 * 4096 * 256
-    out["infonce_4096x256_bf16"] = {"ms_median": round(med, 4), "ms_min": round(best, 4),
-                                    "TFLOP/s": round(flops / (med * 1e-3) / 1e12, 1),
-                                    "frac_mfma_bf16_peak": round(flops / (med * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
-                                    "algorithmic_flop": flops}
+    out["infonce_4096x256_bf16"] = {"ms": round(ms, 4), "TFLOP/s": round(flops / (ms * 1e-3) / 1e12, 1),
+                                    "frac_mfma_bf16_peak": round(flops / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+                                    "algorithmic_flop": flops, "kernel_launches": 4}
 
     # BYOL loss (latency only)
     o = [torch.randn(256, 128, generator=g).to(dev) for _ in range(4)]
-    o[0].requires_grad_()
-    o[1].requires_grad_()
+    g1, g2 = torch.empty_like(o[0]), torch.empty_like(o[1])
+    wsb = torch.empty(512, device=dev)
 
     def f():
-        o[0].grad = o[1].grad = None
-        ta.byol_loss(o[0], o[1], o[2], o[3]).backward()
-    med, mean, best = _time_gpu(f, 50)
-    out["byol_256x128_f32"] = {"ms_median": round(med, 4), "ms_min": round(best, 4), "note": "latency-bound"}
+        _lib.check(lib.ts_byol_fwd_bwd(o[0].data_ptr(), o[3].data_ptr(), o[1].data_ptr(), o[2].data_ptr(), 256, 128,
+                                       wsb.data_ptr(), loss.data_ptr(), g1.data_ptr(), g2.data_ptr(), _lib.TS_F32,
+                                       stream), "ts_byol_fwd_bwd")
+    out["byol_256x128_f32"] = {"ms": round(_time_stream(f, 50), 4), "note": "latency-bound", "kernel_launches": 2}
 
-    # DeferredBatchNorm (cfg5): statistics only, and statistics + normalise
+    # DeferredBatchNorm (cfg5): statistics only, statistics + normalise, backward
     x = (torch.randn(32, 256, 56, 56, generator=g) * 1.5 + 0.5).to(dev)
-    bn = ta.DeferredBatchNorm(256, chunks=8).to(dev)
-    lib = _lib.lib()
-    mean_b = torch.empty(256, device=dev)
-    inv_b = torch.empty(256, device=dev)
+    y = torch.empty_like(x)
+    z = lambda n: torch.zeros(n, device=dev)  # noqa: E731
+    wsn, acc_s, acc_q, mean_b, inv_b = z(512), z(256), z(256), z(256), z(256)
+    gamma, beta = torch.rand(256, generator=g).to(dev) + 0.5, (torch.randn(256, generator=g) * 0.1).to(dev)
 
-    def stats_only():
-        _lib.check(lib.ts_bn_stats(x.data_ptr(), 32, 256, 3136, bn._ws.data_ptr(), bn.sum.data_ptr(),
-                                   bn.sum_squares.data_ptr(), mean_b.data_ptr(), inv_b.data_ptr(), 1e-5,
-                                   _lib.current_stream_ptr(dev)), "ts_bn_stats")
-    out["bn_stats_32x256x56x56_f32"] = entry(x.numel() * 4, _time_gpu(stats_only, 30))
-    with torch.no_grad():
-        out["bn_track_normalise_32x256x56x56_f32"] = entry(x.numel() * 12, _time_gpu(lambda: bn(x), 30))
+    def stats():
+        _lib.check(lib.ts_bn_stats(x.data_ptr(), 32, 256, 3136, wsn.data_ptr(), acc_s.data_ptr(), acc_q.data_ptr(),
+                                   mean_b.data_ptr(), inv_b.data_ptr(), 1e-5, stream), "ts_bn_stats")
+
+    def apply():
+        _lib.check(lib.ts_bn_apply(x.data_ptr(), y.data_ptr(), mean_b.data_ptr(), inv_b.data_ptr(), gamma.data_ptr(),
+                                   beta.data_ptr(), 32, 256, 3136, 0, 1e-5, stream), "ts_bn_apply")
+
+    def both():
+        stats()
+        apply()
+    out["bn_stats_32x256x56x56_f32"] = entry(x.numel() * 4, _time_stream(stats, 50), None, 2)
+    out["bn_stats_normalise_32x256x56x56_f32"] = entry(x.numel() * 12, _time_stream(both, 50), None, 3)
+    dy, dx, dgam, dbet = torch.randn_like(x), torch.empty_like(x), z(256), z(256)
+
+    def bwd():
+        _lib.check(lib.ts_bn_backward(x.data_ptr(), dy.data_ptr(), mean_b.data_ptr(), inv_b.data_ptr(), gamma.data_ptr(),
+                                      dx.data_ptr(), dgam.data_ptr(), dbet.data_ptr(), wsn.data_ptr(), 32, 256, 3136, 1,
+                                      stream), "ts_bn_backward")
+    out["bn_backward_32x256x56x56_f32"] = entry(x.numel() * 20, _time_stream(bwd, 30),
+                                                "bytes = read x,dy twice + write dx", 3)
     return out
 
 

@@ -17,6 +17,9 @@ from . import _lib
 
 ENTRY_BYTES = 32
 _RING = 4
+# When set to a list, every multi-segment copy appends a (start, end) pair of
+# HIP events recorded on the launch stream around the kernel alone (profiling aid).
+kernel_events = None
 _tls = threading.local()
 
 
@@ -124,7 +127,14 @@ def copy_segments(srcs: Sequence[torch.Tensor], dsts: Sequence[torch.Tensor]) ->
     device = dsts[0].device
     nbytes = np.fromiter((s.numel() * s.element_size() for s in srcs), dtype=np.int64, count=len(srcs))
     table = stage_copy(ptr_array(srcs), ptr_array(dsts), nbytes, device)
+    timed = kernel_events is not None
+    if timed:
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record(torch.cuda.current_stream(device))
     _lib.check(_lib.lib().ts_copy_segments(table.dev_ptr, table.n_chunks, table.chunk,
                                            _lib.current_stream_ptr(device)),
                "ts_copy_segments")
+    if timed:
+        end.record(torch.cuda.current_stream(device))
+        kernel_events.append((start, end))
     table.done()
