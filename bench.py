@@ -31,6 +31,10 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBS = 8000.0       # MI355X published HBM3E bandwidth
 MFMA_BF16_PEAK_TFLOPS = 2500.0
+# HBM bytes one ViT-B EMA launch moves, from two rocprofv3 --pmc runs (FETCH_SIZE,
+# WRITE_SIZE) scaled by the same counters on the copy kernel of known size;
+# summary in profiles/hbm_traffic_pmc_all_kernels.md.  Not measured by this script.
+EMA_VITB_TRAFFIC_BYTES = 1035.3e6
 
 
 def _shapes():
@@ -114,7 +118,7 @@ def run_step_benchmark(steps, warmup, dev):
         "elapsed": elapsed, "n_params": n_params, "loss": float(state["loss"].item()),
         "roofline": {"bound": "hbm", "kernel": "ema_multi_kernel", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": None, "algorithmic_bytes_per_launch": algo_bytes,
+                     "traffic": EMA_VITB_TRAFFIC_BYTES, "algorithmic_bytes_per_launch": algo_bytes,
                      "avg_kernel_ms": round(avg_ema_ms, 4), "launches_timed": len(ema_ms)},
     }
 
