@@ -79,21 +79,27 @@ def run_step_benchmark(steps, warmup, dev):
     n_params = sum(numel(s) for s in vit)
 
     s_ema, s_loss = torch.cuda.Stream(dev), torch.cuda.Stream(dev)
+    fork, join_ema, join_loss = torch.cuda.Event(), torch.cuda.Event(), torch.cuda.Event()
     state = {"teacher": teacher, "loss": None}
 
     def step():
+        # fork: both side streams wait for what the main stream has queued
         main = torch.cuda.current_stream(dev)
-        s_ema.wait_stream(main)
-        s_loss.wait_stream(main)
+        fork.record(main)
+        s_ema.wait_event(fork)
+        s_loss.wait_event(fork)
         with torch.cuda.stream(s_ema):
             state["teacher"] = ta.calculate_updated_momentum_encoder(0.99, student, state["teacher"])
+            join_ema.record(s_ema)
         with torch.cuda.stream(s_loss):
             q.grad = None
             loss = ta.infonce_loss(q, k, 0.2)
             loss.backward()
             state["loss"] = loss
-        main.wait_stream(s_ema)
-        main.wait_stream(s_loss)
+            join_loss.record(s_loss)
+        # join: the step is over when both streams are
+        main.wait_event(join_ema)
+        main.wait_event(join_loss)
 
     for _ in range(warmup):
         step()

@@ -181,3 +181,26 @@ def test_ema_output_arenas_are_recycled_only_when_unreferenced(device):
     assert all(bits_equal(x, w) for x, w in zip(d, ts_oracle.ema_update(0.6, student, teacher)))
     assert all(bits_equal(x, w) for x, w in zip(b, ts_oracle.ema_update(0.8, student, teacher)))
     ema_mod.release_pool()
+
+
+def test_clone_and_copy_in_of_a_parameter_list(device):
+    # the two whole-list copies around the EMA in the optimizer step
+    g = seeded(31)
+    params = [torch.nn.Parameter(torch.randn(s, generator=g).to(device)) for s in [(64, 3, 7, 7), (64,), (5, 3), (1,)]]
+    params.append(torch.nn.Parameter(torch.randint(0, 100, (7,), generator=g).to(device), requires_grad=False))
+    clones = ta.clone_params(params)
+    assert len(clones) == len(params)
+    for c, p in zip(clones, params):
+        assert c.shape == p.shape and c.dtype == p.dtype and not c.requires_grad
+        assert c.data_ptr() != p.data_ptr() and bits_equal(c, p)
+        assert c.data_ptr() % 16 == 0
+    live = [torch.nn.Parameter(torch.zeros_like(p), requires_grad=p.is_floating_point()) for p in params]
+    ptrs = [p.data_ptr() for p in live]
+    ta.copy_params_(live, clones)
+    for l, c, ptr in zip(live, clones, ptrs):
+        assert bits_equal(l, c) and l.data_ptr() == ptr
+    assert ta.clone_params([]) == []
+    with pytest.raises(ValueError):
+        ta.copy_params_(live[:2], clones[:1])
+    with pytest.raises(ValueError):
+        ta.copy_params_([live[0]], [clones[1]])

@@ -78,6 +78,31 @@ def lib() -> ctypes.CDLL:
     return _lib
 
 
+HOST_LIB_PATH = os.path.join(_HERE, "_ts_hostlist.so")
+_host = None
+_host_tried = False
+
+
+def host_helper():
+    """The optional C++ list helper (tspipe_amd/csrc_host), or None when it has
+    not been built.  It only walks Python lists of tensors faster; all GPU work
+    goes through lib()."""
+    global _host, _host_tried
+    if _host_tried:
+        return _host
+    with _lock:
+        if not _host_tried:
+            if os.path.exists(HOST_LIB_PATH):
+                import importlib.util
+                import torch  # noqa: F401  (the module links against torch)
+                spec = importlib.util.spec_from_file_location("_ts_hostlist", HOST_LIB_PATH)
+                mod = importlib.util.module_from_spec(spec)
+                spec.loader.exec_module(mod)
+                _host = mod
+            _host_tried = True
+    return _host
+
+
 def check(status: int, what: str) -> int:
     """Raises on a negative status; returns it otherwise (plans return counts)."""
     if status < 0:

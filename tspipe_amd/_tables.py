@@ -24,10 +24,11 @@ _tls = threading.local()
 
 
 class _Slot:
-    __slots__ = ("pinned", "dev", "event", "capacity")
+    __slots__ = ("pinned", "dev", "event", "spare", "capacity")
 
     def __init__(self, device: torch.device, capacity: int):
         self.capacity = capacity
+        self.spare = None  # the event object of the previous use, recycled
         self.pinned = torch.empty(capacity * ENTRY_BYTES, dtype=torch.uint8, pin_memory=True)
         self.dev = torch.empty(capacity * ENTRY_BYTES, dtype=torch.uint8, device=device)
         self.event = None
@@ -41,7 +42,7 @@ class _Ring:
 
     def acquire(self, n_entries: int) -> _Slot:
         if len(self.slots) < _RING:
-            slot = _Slot(self.device, max(n_entries, 1024))
+            slot = _Slot(self.device, max(n_entries, 4608))
             self.slots.append(slot)
             return slot
         idx = self.next
@@ -49,11 +50,16 @@ class _Ring:
         slot = self.slots[idx]
         if slot.event is not None:
             slot.event.synchronize()  # the launch that read this table is done
-            slot.event = None
+            slot.spare, slot.event = slot.event, None
         if slot.capacity < n_entries:
-            slot = _Slot(self.device, max(n_entries, 2 * slot.capacity))
-            self.slots[idx] = slot
+            slot = self.grow(slot, n_entries)
         return slot
+
+    def grow(self, slot: _Slot, n_entries: int) -> _Slot:
+        """Replaces an idle slot by a larger one."""
+        bigger = _Slot(self.device, max(n_entries, 2 * slot.capacity))
+        self.slots[self.slots.index(slot)] = bigger
+        return bigger
 
 
 def _ring(device: torch.device) -> _Ring:
@@ -83,7 +89,7 @@ class StagedTable:
         return self.slot.dev.data_ptr()
 
     def done(self) -> None:
-        ev = torch.cuda.Event()
+        ev = self.slot.spare or torch.cuda.Event()
         ev.record(torch.cuda.current_stream(self.device))
         self.slot.event = ev
 
@@ -95,9 +101,14 @@ def stage_ema(t_ptrs: np.ndarray, s_ptrs: np.ndarray, o_ptrs: np.ndarray, numels
     if chunk_elems == 0:
         chunk_elems = lib.ts_ema_auto_chunk(int(numels.sum()))
     args = (t_ptrs.ctypes.data, s_ptrs.ctypes.data, o_ptrs.ctypes.data, numels.ctypes.data, n, chunk_elems)
-    count = _lib.check(lib.ts_ema_plan(*args, None, 0), "ts_ema_plan(count)")
-    slot = _ring(device).acquire(count)
-    _lib.check(lib.ts_ema_plan(*args, slot.pinned.data_ptr(), slot.capacity), "ts_ema_plan")
+    ring = _ring(device)
+    slot = ring.acquire(0)
+    count = lib.ts_ema_plan(*args, slot.pinned.data_ptr(), slot.capacity)
+    if count == -2:  # TS_ERR_CAPACITY: count, grow the slot, plan again
+        count = _lib.check(lib.ts_ema_plan(*args, None, 0), "ts_ema_plan(count)")
+        slot = ring.grow(slot, count)
+        count = lib.ts_ema_plan(*args, slot.pinned.data_ptr(), slot.capacity)
+    _lib.check(count, "ts_ema_plan")
     if count:
         nbytes = count * ENTRY_BYTES
         slot.dev[:nbytes].copy_(slot.pinned[:nbytes], non_blocking=True)
@@ -111,9 +122,14 @@ def stage_copy(src_ptrs: np.ndarray, dst_ptrs: np.ndarray, nbytes_arr: np.ndarra
     if chunk_bytes == 0:
         chunk_bytes = lib.ts_copy_auto_chunk(int(nbytes_arr.sum()))
     args = (src_ptrs.ctypes.data, dst_ptrs.ctypes.data, nbytes_arr.ctypes.data, n, chunk_bytes)
-    count = _lib.check(lib.ts_copy_plan(*args, None, 0), "ts_copy_plan(count)")
-    slot = _ring(device).acquire(count)
-    _lib.check(lib.ts_copy_plan(*args, slot.pinned.data_ptr(), slot.capacity), "ts_copy_plan")
+    ring = _ring(device)
+    slot = ring.acquire(0)
+    count = lib.ts_copy_plan(*args, slot.pinned.data_ptr(), slot.capacity)
+    if count == -2:  # TS_ERR_CAPACITY: count, grow the slot, plan again
+        count = _lib.check(lib.ts_copy_plan(*args, None, 0), "ts_copy_plan(count)")
+        slot = ring.grow(slot, count)
+        count = lib.ts_copy_plan(*args, slot.pinned.data_ptr(), slot.capacity)
+    _lib.check(count, "ts_copy_plan")
     if count:
         nbytes = count * ENTRY_BYTES
         slot.dev[:nbytes].copy_(slot.pinned[:nbytes], non_blocking=True)

@@ -49,5 +49,26 @@ def build(verbose: bool = True) -> str:
     return LIB_PATH
 
 
+HOST_DIR = os.path.join(HERE, "csrc_host")
+HOST_NAME = "_ts_hostlist"
+
+
+def build_host(verbose: bool = False) -> str:
+    """Builds the optional host-side list helper (plain C++ against torch's
+    headers, no GPU code) into tspipe_amd/csrc_host/.  The adapters work
+    without it, only with more Python overhead per call."""
+    from torch.utils import cpp_extension
+    os.makedirs(os.path.join(HOST_DIR, "build"), exist_ok=True)
+    cpp_extension.load(name=HOST_NAME, sources=[os.path.join(HOST_DIR, "hostlist.cpp")],
+                       build_directory=os.path.join(HOST_DIR, "build"), extra_cflags=["-O2"], verbose=verbose)
+    built = os.path.join(HOST_DIR, "build", HOST_NAME + ".so")
+    final = os.path.join(HERE, HOST_NAME + ".so")
+    import shutil
+    shutil.copyfile(built, final + ".tmp")
+    os.replace(final + ".tmp", final)
+    return final
+
+
 if __name__ == "__main__":
     build()
+    build_host()

@@ -91,6 +91,55 @@ def _launch(m: float, students: Sequence[torch.Tensor], teachers: Sequence[torch
         table.done()
 
 
+_tls = threading.local()
+
+
+def _scratch(n: int):
+    """Per-thread pointer / size arrays the C++ helper fills."""
+    buf = getattr(_tls, "buf", None)
+    if buf is None or buf[0].size < n:
+        cap = max(256, 2 * n)
+        buf = _tls.buf = (np.empty(cap, np.uint64), np.empty(cap, np.uint64), np.empty(cap, np.int64))
+    return buf
+
+
+def _fast_update(m: float, online, target) -> Optional[List[torch.Tensor]]:
+    """The common case -- two lists of dense fp32 tensors on one GPU -- with the
+    per-tensor work done by the C++ helper.  Returns None whenever anything is
+    unusual (no helper, not lists, None entries, strided tensors, errors): the
+    Python path then handles it or raises the proper exception."""
+    host = _lib.host_helper()
+    if host is None or type(online) is not list or type(target) is not list or _use_count is None:
+        return None
+    n = min(len(online), len(target))
+    if n == 0:
+        return None
+    sp, tp, nn = _scratch(n)
+    status, n, dev_index, shape_hash, total = host.pair_info(online, target, sp.ctypes.data, tp.ctypes.data,
+                                                             nn.ctypes.data, sp.size)
+    if status != 0:
+        return None
+    teachers = target if len(target) == n else target[:n]
+    arena = _acquire_arena(teachers, (n, total, shape_hash))
+    if arena.numels.size != n or not np.array_equal(arena.numels, nn[:n]):
+        return None  # hash collision between different lists: take the exact path
+    device = teachers[0].device
+    with torch.cuda.device(device):
+        table = _tables.stage_ema(tp[:n], sp[:n], arena.ptrs, arena.numels, device)
+        timed = kernel_events is not None
+        if timed:
+            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record(torch.cuda.current_stream(device))
+        status = _lib.lib().ts_ema_multi(table.dev_ptr, table.n_chunks, table.chunk, float(m), 1.0 - float(m),
+                                        _lib.current_stream_ptr(device))
+        _lib.check(status, "ts_ema_multi")
+        if timed:
+            end.record(torch.cuda.current_stream(device))
+            kernel_events.append((start, end))
+        table.done()
+    return list(arena.views)
+
+
 class _Arena:
     """One flat output allocation and its views, shaped like a parameter list."""
     __slots__ = ("flat", "views", "ptrs", "numels", "stream")
@@ -120,6 +169,9 @@ class _Arena:
         storage = self.flat.untyped_storage()
         if _use_count(storage._cdata) != len(self.views) + 2:  # flat + views + the wrapper just made
             return False
+        host = _lib.host_helper()
+        if host is not None:
+            return host.all_refcounts_equal(self.views, 1)  # only self.views holds them
         return all(c == 2 for c in map(sys.getrefcount, self.views))
 
 
@@ -140,6 +192,8 @@ def release_pool() -> None:
 
 
 def _acquire_arena(teachers: Sequence[torch.Tensor], shapes) -> _Arena:
+    """shapes: anything hashable that identifies the list's shapes (the tuple of
+    shapes, or the helper's (count, total, 64-bit shape hash) triple)."""
     if _use_count is None:
         return _Arena(teachers)
     device = teachers[0].device
@@ -164,6 +218,9 @@ def momentum_update(m: float, online_new_param: Iterable[Optional[torch.Tensor]]
     The results are views of one flat allocation.  "New" means not aliased by
     anything the caller still holds: tensors of an earlier result may be handed
     out again once the caller has dropped every reference to them."""
+    fast = _fast_update(m, online_new_param, target_param)
+    if fast is not None:
+        return fast
     students, teachers, shapes = _prepare(online_new_param, target_param, skip_none)
     if not teachers:
         return []
@@ -197,3 +254,62 @@ def update_target_network_parameters_(online_params: Iterable[torch.Tensor],
     for live, work in zip(target_params, teachers):
         if work.data_ptr() != live.data_ptr():  # a non-contiguous parameter was densified
             live.detach().copy_(work)
+
+
+# ---------------------------------------------------------------------------
+# The EMA's neighbours in the optimizer step: whole-list clone and copy-in
+# ---------------------------------------------------------------------------
+
+def _check_copy_lists(srcs: Sequence[torch.Tensor], dsts: Sequence[torch.Tensor]) -> None:
+    if len(srcs) != len(dsts):
+        raise ValueError(f"list lengths differ: {len(srcs)} vs {len(dsts)}")
+    for s, d in zip(srcs, dsts):
+        if s.shape != d.shape or s.dtype != d.dtype:
+            raise ValueError(f"copy needs matching shape and dtype: {tuple(s.shape)} {s.dtype} vs {tuple(d.shape)} {d.dtype}")
+        if not (s.is_cuda and d.is_cuda) or s.device != d.device:
+            raise TypeError("whole-list copies run on tensors of one GPU (no host fallback)")
+        if not d.is_contiguous():
+            raise ValueError("destination tensors must be contiguous")
+
+
+@torch.no_grad()
+def clone_params(params: Iterable[torch.Tensor]) -> List[torch.Tensor]:
+    """``[p.detach().clone() for p in params]`` as one kernel launch: the copy
+    of the student parameters the pipeline takes after every optimizer step
+    (tspipe/gpu_task.py:398).  The clones are views of one flat allocation."""
+    srcs = [p.detach() for p in params]
+    if not srcs:
+        return []
+    if any(not s.is_cuda for s in srcs):
+        raise TypeError("whole-list copies run on device tensors (no host fallback)")
+    dense = [s if s.is_contiguous() else s.contiguous() for s in srcs]
+    by_dtype = {}
+    for i, s in enumerate(dense):
+        by_dtype.setdefault(s.dtype, []).append(i)
+    outs: List[Optional[torch.Tensor]] = [None] * len(dense)
+    for dtype, idx in by_dtype.items():
+        esize = dense[idx[0]].element_size()
+        per16 = 16 // esize  # elements per 16 bytes: every clone starts on a 16-byte boundary
+        padded = [(dense[i].numel() + per16 - 1) // per16 * per16 for i in idx]
+        flat = torch.empty(sum(padded), dtype=dtype, device=dense[idx[0]].device)
+        for i, piece in zip(idx, flat.split(padded)):
+            outs[i] = piece[:dense[i].numel()].view(dense[i].shape)
+    live = [(s, o) for s, o in zip(dense, outs) if s.numel()]
+    with torch.cuda.device(dense[0].device):
+        _tables.copy_segments([s for s, _ in live], [o for _, o in live])
+    return outs  # type: ignore[return-value]
+
+
+@torch.no_grad()
+def copy_params_(dst_params: Iterable[torch.Tensor], src_params: Iterable[torch.Tensor]) -> None:
+    """``for p, new in zip(dst, src): p.copy_(new)`` as one kernel launch: how a
+    stored parameter version reaches the live module (tspipe/gpu_task.py:706-724)."""
+    dsts = [d.detach() for d in dst_params]
+    srcs = [s.detach() for s in src_params]
+    _check_copy_lists(srcs, dsts)
+    srcs = [s if s.is_contiguous() else s.contiguous() for s in srcs]
+    live = [(s, d) for s, d in zip(srcs, dsts) if s.numel()]
+    if not live:
+        return
+    with torch.cuda.device(dsts[0].device):
+        _tables.copy_segments([s for s, _ in live], [d for _, d in live])
