@@ -184,7 +184,8 @@ __global__ __launch_bounds__(kNceBlock) void nce_prep_kernel(const T* __restrict
 template <int C>
 struct NceSmem {
   static constexpr int KLD = C + 8;       // bf16 per K-tile row (16-byte pad: rows start on different banks)
-  static constexpr int TLD = kKTile + 8;  // bf16 per K^T-tile row (80 bytes, keeps 16-byte alignment)
+  static constexpr int TLD = kKTile + 4;  // bf16 per K^T-tile row: 72 bytes, so 16 consecutive rows start on
+                                          // 16 different bank pairs and the 8-byte operand reads do not collide
   uint16_t k[2][kKTile * KLD];
   uint16_t kt[2][C * TLD];
   float rk[2][kKTile];
@@ -205,8 +206,11 @@ __global__ __launch_bounds__(kNceBlock) void nce_main_kernel(const uint16_t* __r
   constexpr int FB = C / 32;  // feature blocks of O^T
   const int tid = threadIdx.x, lane = tid % kWave, w = tid / kWave;
   const int col = lane % 32, h = lane / 32;
-  const int64_t qtile = blockIdx.x;
-  const int split = blockIdx.y;
+  // Workgroup ids are dealt round-robin to the 8 XCDs.  With the key split as
+  // the fastest index (and 8 splits), every XCD keeps seeing the same eighth
+  // of K and K^T, which then stays in that XCD's own L2.
+  const int split = blockIdx.x;
+  const int64_t qtile = blockIdx.y;
   const int64_t qrow = qtile * kQTile + w * 32 + col;  // the q row this lane is a column of
 
   const int64_t ktiles = npad / kKTile;
@@ -265,7 +269,10 @@ __global__ __launch_bounds__(kNceBlock) void nce_main_kernel(const uint16_t* __r
     for (int u = 0; u < TCH; ++u) {
       const int id = tid + u * kNceBlock;
       const int f = id / (kKTile / 8), c8 = id % (kKTile / 8);
-      *reinterpret_cast<u32x4*>(&sm.kt[buf][f * Smem::TLD + c8 * 8]) = stage_t[u];
+      // rows are only 8-byte aligned: two 8-byte stores
+      uint2 lo = {stage_t[u].x, stage_t[u].y}, hi = {stage_t[u].z, stage_t[u].w};
+      *reinterpret_cast<uint2*>(&sm.kt[buf][f * Smem::TLD + c8 * 8]) = lo;
+      *reinterpret_cast<uint2*>(&sm.kt[buf][f * Smem::TLD + c8 * 8 + 4]) = hi;
     }
     if (tid < kKTile) sm.rk[buf][tid] = stage_rk;
   };
@@ -281,52 +288,74 @@ __global__ __launch_bounds__(kNceBlock) void nce_main_kernel(const uint16_t* __r
     const bool more = t + 1 < t1;
     if (more) load_tile(t + 1);  // in flight while this tile is computed
 
+    // All operand fragments of a phase are read from LDS into their own
+    // registers before the phase's MFMAs start: with one wavefront per SIMD
+    // nothing else hides the LDS latency, and a read-wait-multiply chain per
+    // MFMA would pay it 48 times per tile.
+    bf16x8 ka[KK];
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      const u32x4 raw = *reinterpret_cast<const u32x4*>(&sm.k[buf][col * Smem::KLD + kk * 16 + h * 8]);
+      __builtin_memcpy(&ka[kk], &raw, 16);
+    }
+    __builtin_amdgcn_sched_barrier(0);  // keep the reads above from being sunk next to their MFMAs
+    const f32x4 rk0 = *reinterpret_cast<const f32x4*>(&sm.rk[buf][4 * h]);
+    const f32x4 rk1 = *reinterpret_cast<const f32x4*>(&sm.rk[buf][8 + 4 * h]);
+    const f32x4 rk2 = *reinterpret_cast<const f32x4*>(&sm.rk[buf][16 + 4 * h]);
+    const f32x4 rk3 = *reinterpret_cast<const f32x4*>(&sm.rk[buf][24 + 4 * h]);
+
     // S^T[key][q] = sum_f K[key][f] Q[q][f]
     f32x16 sacc;
 #pragma unroll
     for (int i = 0; i < 16; ++i) sacc[i] = 0.f;
 #pragma unroll
-    for (int kk = 0; kk < KK; ++kk) {
-      bf16x8 a;
-      const u32x4 raw = *reinterpret_cast<const u32x4*>(&sm.k[buf][col * Smem::KLD + kk * 16 + h * 8]);
-      __builtin_memcpy(&a, &raw, 16);
-      sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[kk], sacc, 0, 0, 0);
+    for (int kk = 0; kk < KK; ++kk) sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[kk], qf[kk], sacc, 0, 0, 0);
+
+    // K^T fragments for the second product: issued now, they land while the
+    // soft-max arithmetic below runs.  Contraction slot 8h + 4gg + j of step
+    // tt is key 16tt + 8gg + 4h + j on both operands.
+    bf16x8 ta[FB][2];
+#pragma unroll
+    for (int fb = 0; fb < FB; ++fb) {
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt) {
+        const uint2* base =
+            reinterpret_cast<const uint2*>(&sm.kt[buf][(fb * 32 + col) * Smem::TLD + 16 * tt + 4 * h]);
+        const uint2 lo = base[0], hi = base[2];
+        const u32x4 raw = {lo.x, lo.y, hi.x, hi.y};
+        __builtin_memcpy(&ta[fb][tt], &raw, 16);
+      }
     }
+
+    __builtin_amdgcn_sched_barrier(0);
 
     // P = 2^(S * rq_i * rk_j * log2e/tau - x_max); keys this lane holds:
     // key(i) = (i%4) + 4h + 8(i/4).  Padded keys have rk = 0 and are masked.
     const int64_t key0 = t * kKTile;
+    const bool ragged = key0 + kKTile > n;  // only the last tile can hold padded keys
     bf16x8 pb[2];
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
-      const f32x4 rk4 = *reinterpret_cast<const f32x4*>(&sm.rk[buf][8 * g + 4 * h]);
+      const f32x4 rk4 = (g == 0) ? rk0 : (g == 1) ? rk1 : (g == 2) ? rk2 : rk3;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int i = 4 * g + j;
         const float rkj = rk4[j];
         const float x = sacc[i] * (sc_i * rkj);
         float p = fast_exp2(x - scale2);
-        if (key0 + 8 * g + 4 * h + j >= n) p = 0.f;
+        if (ragged && key0 + 8 * g + 4 * h + j >= n) p = 0.f;
         lsum += p;
         asum += p * x;
         pb[g / 2][(g % 2) * 4 + j] = (__bf16)(p * rkj);
       }
     }
 
-    // O^T[f][q] += sum_key K^T[f][key] * (P*rk)[key][q]; contraction slot
-    // 8h + 4gg + j of step tt is key 16tt + 8gg + 4h + j on both operands.
+    // O^T[f][q] += sum_key K^T[f][key] * (P*rk)[key][q]
 #pragma unroll
-    for (int fb = 0; fb < FB; ++fb) {
+    for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
-      for (int tt = 0; tt < 2; ++tt) {
-        const uint16_t* base = &sm.kt[buf][(fb * 32 + col) * Smem::TLD + 16 * tt + 4 * h];
-        bf16x4 lo, hi;
-        __builtin_memcpy(&lo, base, 8);
-        __builtin_memcpy(&hi, base + 8, 8);
-        bf16x8 a = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-        oacc[fb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb[tt], oacc[fb], 0, 0, 0);
-      }
-    }
+      for (int fb = 0; fb < FB; ++fb)
+        oacc[fb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ta[fb][tt], pb[tt], oacc[fb], 0, 0, 0);
 
     if (more) store_tile(buf ^ 1);
     __syncthreads();
@@ -433,7 +462,7 @@ int nce_run_pair(const void* q, const void* k, void* dq, int64_t n, float tau, c
   const uint16_t* qsrc = kF32 ? qb : (const uint16_t*)q;
   const uint16_t* ksrc = kF32 ? kb : (const uint16_t*)k;
   // with bf16 copies the rows beyond n exist (zero); the kernel guards by n either way
-  hipLaunchKernelGGL((nce_main_kernel<C>), dim3((unsigned)(L.npad / kQTile), (unsigned)L.splits),
+  hipLaunchKernelGGL((nce_main_kernel<C>), dim3((unsigned)L.splits, (unsigned)(L.npad / kQTile)),
                      dim3(kNceBlock), 0, stream, qsrc, ksrc, kt, rq, rk, n, L.npad, L.splits, scale2, lpart,
                      apart, opart);
   rc = check_launch();
