@@ -143,6 +143,25 @@ int ts_kd_fwd_bwd(const void* s, const void* t, const uint8_t* row_mask, int64_t
                   void* workspace, float* loss_out, void* grad, int64_t ld_g, int dtype,
                   ts_stream_t stream);
 
+/* The same pass with the hard-label cross entropy added, the combination the
+ * reference's distillation plug-ins compute on the student logits:
+ *   benchmarks/soft_target/train_kd.py:439-453
+ *       CrossEntropyLoss()(model_out, label) + SoftTarget(T)(model_out, ema_out) * lambda_kd
+ *   benchmarks/distilbert/distiller.py:719-744
+ *       alpha_ce * KLDiv(masked rows) * T^2 + alpha_mlm * CrossEntropyLoss(ignore_index=-100)(all rows, lm_labels)
+ *
+ *   loss = kd_scale / B_kd * sum_{rows with row_mask} KL(...)
+ *        + ce_weight / B_ce * sum_{rows with a valid label} (logsumexp(s_row) - s_row[label])
+ * B_kd as in ts_kd_fwd_bwd; B_ce = rows whose label differs from ignore_index
+ * (labels outside [0, V) are treated as ignored).  The two row sets are
+ * independent; rows in neither get a zero gradient.  labels: int64 per row, or
+ * NULL for no CE term (then identical to ts_kd_fwd_bwd with loss_scale =
+ * kd_scale).  Same workspace as ts_kd_fwd_bwd. */
+int ts_kdce_fwd_bwd(const void* s, const void* t, const uint8_t* row_mask, const int64_t* labels,
+                    int64_t ignore_index, int64_t n_rows, int64_t V, int64_t ld_s, int64_t ld_t,
+                    float inv_T, float kd_scale, float ce_weight, void* workspace, float* loss_out,
+                    void* grad, int64_t ld_g, int dtype, ts_stream_t stream);
+
 /* grad *= *g for the rows the loss touched; returns at once on the device
  * when *g == 1 (the only value TSPipe's torch.autograd.backward(loss) feeds,
  * tspipe/gpu_task.py:207-212).  g_dev: one float in device memory. */
@@ -163,6 +182,20 @@ int ts_scale_rows(void* grad, int64_t n_rows, int64_t V, int64_t ld_g, const flo
 int ts_byol_fwd_bwd(const void* x1, const void* y1, const void* x2, const void* y2, int64_t n,
                     int64_t c, float* workspace, float* loss_out, void* gx1, void* gx2,
                     int dtype, ts_stream_t stream);
+
+/* Cosine embedding loss with target +1, forward and backward: the hidden-state
+ * term of DistilBERT's loss (benchmarks/distilbert/distiller.py:756-770,
+ * nn.CosineEmbeddingLoss(reduction="mean") on the rows the attention mask keeps):
+ *   cos_i = <x_i, y_i> / sqrt((|x_i|^2 + 1e-12)(|y_i|^2 + 1e-12))
+ *   loss  = weight * mean over rows with row_mask != 0 of (1 - cos_i)
+ *   gx    = d loss / d x, zero for the other rows (y is the detached teacher)
+ * x, y, gx: [n, c] contiguous; row_mask may be NULL (all rows); gx may be NULL.
+ * workspace: ts_cosine_workspace_bytes(n) bytes, 16-byte aligned. */
+size_t ts_cosine_workspace_bytes(int64_t n);
+
+int ts_cosine_fwd_bwd(const void* x, const void* y, const uint8_t* row_mask, int64_t n, int64_t c,
+                      float weight, void* workspace, float* loss_out, void* gx, int dtype,
+                      ts_stream_t stream);
 
 /* ------------------------------------------------------------------------ */
 /* MoCo-v3 InfoNCE loss, forward and backward, logits never stored.      */

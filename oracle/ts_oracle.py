@@ -54,6 +54,36 @@ def distil_ce(s_logits: Tensor, t_logits: Tensor, row_mask: Tensor, temperature:
     return alpha_ce * ce
 
 
+def soft_target_tspipe_loss(model_out: Tensor, ema_model_out: Tensor, label: Tensor, T: float,
+                            lambda_kd: float) -> Tensor:
+    """benchmarks/soft_target/train_kd.py:439-453 with kd_mode == 'st'."""
+    cls_loss = nn.CrossEntropyLoss()(model_out, label)
+    kd_loss = kd_soft_target(model_out, ema_model_out.detach(), T) * lambda_kd
+    return cls_loss + kd_loss
+
+
+def distil_loss(s_logits: Tensor, t_logits: Tensor, s_hidden: Optional[Tensor], t_hidden: Optional[Tensor],
+                lm_labels: Tensor, attention_mask: Tensor, alpha_ce: float, alpha_mlm: float, alpha_cos: float,
+                temperature: float, restrict_ce_to_mask: bool) -> Tensor:
+    """benchmarks/distilbert/distiller.py:711-772 without the clm and mse terms:
+    masked KD (719-740), masked-LM cross entropy with ignore_index=-100 (742-744,
+    lm_loss_fct at 117), cosine embedding loss on the last hidden states (756-770)."""
+    mask2d = (lm_labels > -1) if restrict_ce_to_mask else attention_mask
+    loss = distil_ce(s_logits, t_logits, mask2d, temperature, alpha_ce)
+    if alpha_mlm > 0.0:
+        loss_mlm = nn.CrossEntropyLoss(ignore_index=-100)(s_logits.view(-1, s_logits.size(-1)), lm_labels.view(-1))
+        loss = loss + alpha_mlm * loss_mlm
+    if alpha_cos > 0.0:
+        mask = attention_mask.unsqueeze(-1).expand_as(s_hidden)
+        dim = s_hidden.size(-1)
+        s_sel = torch.masked_select(s_hidden, mask).view(-1, dim)
+        t_sel = torch.masked_select(t_hidden, mask).view(-1, dim)
+        target = s_sel.new(s_sel.size(0)).fill_(1)
+        loss_cos = nn.CosineEmbeddingLoss(reduction="mean")(s_sel, t_sel, target)
+        loss = loss + alpha_cos * loss_cos
+    return loss
+
+
 # -- BYOL / MoCo --------------------------------------------------------------
 
 def byol_regression_loss(x: Tensor, y: Tensor) -> Tensor:

@@ -160,7 +160,11 @@ def test_device_entry_points_validate_before_launching():
     assert lib.ts_bn_apply(p, None, p, p, None, None, 2, 3, 4, 0, 1e-5, None) == -1
     assert lib.ts_bn_backward(p, p, p, p, None, p, p, None, p, 2, 3, 4, 1, None) == -1
     assert lib.ts_scale_rows(p, 4, 10, 9, p, 0, None) == -1
-    assert lib.ts_kd_workspace_bytes(0, 100, 0) == 32 and lib.ts_kd_workspace_bytes(5, 100, 0) == 96
-    assert lib.ts_kd_workspace_bytes(4096, 30522, 1) == 32 + 2 * 4096 * 4 + 4096 * 4 * 32  # 4 parts per wide row
+    assert lib.ts_kd_workspace_bytes(0, 100, 0) == 32 and lib.ts_kd_workspace_bytes(5, 100, 0) == 32 + 3 * 32
+    assert lib.ts_kd_workspace_bytes(4096, 30522, 1) == 32 + 3 * 4096 * 4 + 4096 * 4 * 32  # 4 parts per wide row
+    assert lib.ts_kdce_fwd_bwd(p, p, None, p + 4, -100, 4, 10, 10, 10, 1.0, 1.0, 1.0, p, p, None, 10, 0, None) == -4  # labels not 8-byte aligned
+    assert lib.ts_kdce_fwd_bwd(p, p, None, None, -100, 4, 10, 10, 10, 0.0, 1.0, 1.0, p, p, None, 10, 0, None) == -1    # inv_T must be positive
+    assert lib.ts_cosine_fwd_bwd(p, None, None, 4, 8, 1.0, p, p, None, 0, None) == -1
+    assert lib.ts_cosine_workspace_bytes(5) == 48
     assert lib.ts_infonce_workspace_bytes(4096, 256, 1) > 4096 * 256 * 4
     assert lib.ts_infonce_workspace_bytes(4096, 256, 3) == 0

@@ -226,3 +226,104 @@ def test_infonce_fp32_inputs_and_identities(device):
     l1 = ta.infonce_loss(qb.to(device), kb.to(device), 0.2).item()
     l2 = ta.infonce_loss((qb * 4).to(device), (kb * 0.5).to(device), 0.2).item()
     assert rel_err(l2, l1) < 1e-4
+
+
+# ---- KD + hard-label CE in one pass, cosine loss, the full loss_fn plug-ins ----
+
+@pytest.mark.parametrize("rows,V,dtype", [(256, 100, torch.float32), (37, 1000, torch.float32), (9, 5000, torch.float32),
+                                          (64, 30522, torch.bfloat16)])
+def test_soft_target_tspipe_loss(device, rows, V, dtype):
+    from argparse import Namespace
+    g = seeded(200 + V)
+    s = (torch.randn(rows, V, generator=g) * 3).to(dtype)
+    t = (torch.randn(rows, V, generator=g) * 3).to(dtype)
+    y = torch.randint(0, V, (rows,), generator=g)
+    want, (gw,) = _oracle_grad(lambda a, b: ts_oracle.soft_target_tspipe_loss(a, b, y, 4.0, 0.7), s, others=(t,))
+    sd = s.to(device).requires_grad_()
+    args = Namespace(kd_mode="st", T=4.0, lambda_kd=0.7)
+    loss = ta.soft_target_tspipe_loss(sd, t.to(device), y.to(device), None, args, 0)
+    loss.backward()
+    tol = 1e-5 if dtype == torch.float32 else 1e-3
+    assert rel_err(loss.item(), want) < tol
+    peak = gw.abs().max().item()
+    slack = gw.abs() * (2.0 ** -8 if dtype != torch.float32 else 0.0)
+    assert ((sd.grad.cpu().double() - gw).abs() <= tol * peak + slack).all()
+
+
+def test_kd_ce_row_sets_and_ignore_index(device):
+    g = seeded(210)
+    rows, V = 40, 257
+    s = torch.randn(rows, V, generator=g) * 2
+    t = torch.randn(rows, V, generator=g) * 2
+    mask = torch.rand(rows, generator=g) < 0.4
+    y = torch.randint(0, V, (rows,), generator=g)
+    y[torch.rand(rows, generator=g) < 0.5] = -100
+    assert (mask & (y == -100)).any() and (~mask & (y != -100)).any() and (~mask & (y == -100)).any()
+
+    def ref(a, b):
+        kd = ts_oracle.distil_ce(a.view(1, rows, V), b.view(1, rows, V), mask.view(1, rows), 2.0, 0.5)
+        ce = torch.nn.CrossEntropyLoss(ignore_index=-100)(a, y)
+        return kd + 2.0 * ce
+    want, (gw,) = _oracle_grad(ref, s, others=(t,))
+    sd = s.to(device).requires_grad_()
+    loss = ta.kd_ce_loss(sd, t.to(device), y.to(device), 2.0, kd_weight=0.5, ce_weight=2.0, row_mask=mask.to(device))
+    loss.backward()
+    assert rel_err(loss.item(), want) < 1e-5
+    assert max_rel_to_peak(sd.grad, gw) < 1e-5
+    idle = ~mask & (y == -100)
+    assert (sd.grad.cpu()[idle] == 0).all()
+    # no valid label at all: the CE mean is 0/0 = NaN, as torch gives
+    none = torch.full((rows,), -100, dtype=torch.long)
+    l = ta.kd_ce_loss(s.to(device), t.to(device), none.to(device), 2.0, row_mask=mask.to(device))
+    assert torch.isnan(l).item() and torch.isnan(torch.nn.CrossEntropyLoss(ignore_index=-100)(s, none)).item()
+
+
+def test_cosine_embedding_loss(device):
+    g = seeded(220)
+    x = torch.randn(3, 7, 48, generator=g)
+    y = torch.randn(3, 7, 48, generator=g)
+    att = torch.rand(3, 7, generator=g) < 0.6
+
+    def ref(a, b):
+        m = att.unsqueeze(-1).expand_as(a)
+        a2, b2 = torch.masked_select(a, m).view(-1, 48), torch.masked_select(b, m).view(-1, 48)
+        return 1.5 * torch.nn.CosineEmbeddingLoss()(a2, b2, a2.new_ones(a2.size(0)))
+    want, (gw,) = _oracle_grad(ref, x, others=(y,))
+    xd = x.to(device).requires_grad_()
+    loss = ta.cosine_embedding_loss(xd, y.to(device), att.to(device), 1.5)
+    loss.backward()
+    assert rel_err(loss.item(), want) < 1e-5
+    assert max_rel_to_peak(xd.grad, gw) < 1e-5
+    assert (xd.grad.cpu()[~att] == 0).all()
+    full = ta.cosine_embedding_loss(x.to(device), y.to(device)).item()
+    assert rel_err(full, torch.nn.CosineEmbeddingLoss()(x.view(-1, 48).double(), y.view(-1, 48).double(),
+                                                      torch.ones(21, dtype=torch.float64)).item()) < 1e-5
+
+
+@pytest.mark.parametrize("restrict", [True, False])
+def test_distil_loss_fn_plugin(device, restrict):
+    from argparse import Namespace
+    g = seeded(230)
+    bs, seq, V, H = 4, 16, 30522, 64
+    s = (torch.randn(bs, seq, V, generator=g) * 2).to(torch.bfloat16)
+    t = (torch.randn(bs, seq, V, generator=g) * 2).to(torch.bfloat16)
+    sh = torch.randn(bs, seq, H, generator=g).to(torch.bfloat16)
+    th = torch.randn(bs, seq, H, generator=g).to(torch.bfloat16)
+    lm = torch.full((bs, seq), -100, dtype=torch.long)
+    pick = torch.rand(bs, seq, generator=g) < 0.15
+    lm[pick] = torch.randint(0, V, (int(pick.sum()),), generator=g)
+    att = torch.rand(bs, seq, generator=g) < 0.8
+    params = Namespace(alpha_ce=0.5, alpha_mlm=2.0, alpha_clm=0.0, alpha_mse=0.0, alpha_cos=1.0, temperature=2.0,
+                       restrict_ce_to_mask=restrict)
+    want, (gs, gh) = _oracle_grad(
+        lambda a, h, b, hb: ts_oracle.distil_loss(a, b, h, hb, lm, att, 0.5, 2.0, 1.0, 2.0, restrict), s, sh,
+        others=(t, th))
+    sd, shd = s.to(device).requires_grad_(), sh.to(device).requires_grad_()
+    loss = ta.distil_loss_fn({"logits": sd, "hidden_states": (shd,)},
+                             {"logits": t.to(device), "hidden_states": (th.to(device),)},
+                             (lm.to(device), att.to(device)), None, params, 0)
+    loss.backward()
+    assert rel_err(loss.item(), want) < 1e-3
+    for got, ref in ((sd.grad, gs), (shd.grad, gh)):
+        peak = ref.abs().max().item()
+        assert ((got.cpu().double() - ref).abs() <= 1e-3 * peak + ref.abs() * 2.0 ** -8).all()

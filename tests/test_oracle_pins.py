@@ -325,3 +325,48 @@ def test_scatter_gather_oracle_identities():
     sizes = (ctypes.c_int64 * 3)(*[p.numel() * 4 for p in pieces])
     _c_oracle().cat_ref(ptrs, sizes, ctypes.c_int64(3), ctypes.c_void_p(out.data_ptr()))
     assert torch.equal(out, want)
+
+
+# ---------------------------------------------------------------- combined distillation losses
+
+def test_soft_target_tspipe_loss_closed_form():
+    g = seeded(10)
+    s = torch.randn(7, 9, generator=g, dtype=torch.float64) * 2
+    t = torch.randn(7, 9, generator=g, dtype=torch.float64) * 2
+    y = torch.randint(0, 9, (7,), generator=g)
+    kd, gkd = _kd_closed_form(s.numpy(), t.numpy(), 4.0)
+    sn = s.numpy()
+    lse = np.log(np.exp(sn - sn.max(1, keepdims=True)).sum(1)) + sn.max(1)
+    ce = (lse - sn[np.arange(7), y.numpy()]).mean()
+    sr = s.clone().requires_grad_()
+    loss = ts_oracle.soft_target_tspipe_loss(sr, t, y, 4.0, 0.7)
+    loss.backward()
+    assert abs(loss.item() - (ce + 0.7 * kd)) < 1e-12
+    soft = np.exp(sn - lse[:, None])
+    onehot = np.eye(9)[y.numpy()]
+    assert np.abs(sr.grad.numpy() - (0.7 * gkd + (soft - onehot) / 7)).max() < 1e-13
+
+
+def test_distil_loss_terms_use_their_own_row_sets():
+    g = seeded(11)
+    bs, seq, V, H = 2, 5, 11, 6
+    s = torch.randn(bs, seq, V, generator=g, dtype=torch.float64)
+    t = torch.randn(bs, seq, V, generator=g, dtype=torch.float64)
+    sh = torch.randn(bs, seq, H, generator=g, dtype=torch.float64)
+    th = torch.randn(bs, seq, H, generator=g, dtype=torch.float64)
+    lm = torch.full((bs, seq), -100, dtype=torch.long)
+    lm[0, 1], lm[1, 3], lm[1, 4] = 3, 0, 10
+    att = torch.tensor([[1, 1, 1, 0, 0], [1, 1, 1, 1, 1]], dtype=torch.bool)
+    for restrict in (True, False):
+        got = ts_oracle.distil_loss(s, t, sh, th, lm, att, 0.5, 2.0, 1.5, 2.0, restrict).item()
+        kd_rows = (lm.reshape(-1) > -1) if restrict else att.reshape(-1)
+        kd, _ = _kd_closed_form(s.reshape(-1, V)[kd_rows].numpy(), t.reshape(-1, V)[kd_rows].numpy(), 2.0)
+        ce_rows = lm.reshape(-1) != -100
+        sn = s.reshape(-1, V)[ce_rows].numpy()
+        lab = lm.reshape(-1)[ce_rows].numpy()
+        lse = np.log(np.exp(sn).sum(1))
+        ce = (lse - sn[np.arange(len(lab)), lab]).mean()
+        a, b = sh.reshape(-1, H)[att.reshape(-1)].numpy(), th.reshape(-1, H)[att.reshape(-1)].numpy()
+        cos = (a * b).sum(1) / np.sqrt(((a * a).sum(1) + 1e-12) * ((b * b).sum(1) + 1e-12))
+        want = 0.5 * kd + 2.0 * ce + 1.5 * (1 - cos).mean()
+        assert abs(got - want) < 1e-12

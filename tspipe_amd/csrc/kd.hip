@@ -1,0 +1,762 @@
+// Distillation row losses, forward and backward fused:
+//   KD soft target   KL(softmax(t/T) || softmax(s/T)) over rows selected by a mask,
+//   hard-label CE    cross entropy of softmax(s) against integer labels with an
+//                    ignore index, optionally in the same pass over the rows.
+// A "group" of threads owns a row: 16/32/64 lanes of a wavefront for narrow
+// rows, a 256-thread workgroup for medium ones; wide (vocabulary-sized) rows
+// are cut into parts handled by short-lived workgroups in two launches.
+// Accumulation is fp32 in the log2 domain (v_exp_f32 / v_log_f32); storage is
+// fp32, bf16 or fp16.
+#include "common.h"
+
+namespace ts {
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+constexpr float kNegBig = -3.0e38f;  // finite stand-in for -inf: keeps 2^((m_old - m_new) k) NaN-free
+
+// Online soft-max state of part of a row.  Maxima are kept in raw logit
+// units; k = inv_T * log2(e) scales differences into the log2 domain.
+//   teacher: m = max t, z = sum 2^((t-m)k), a = sum 2^((t-m)k) (t - s)
+//   student: m = max s, z = sum 2^((s-m)k), z1 = sum 2^((s-m) log2e)   (z1: temperature 1, for the CE term)
+struct TStat {
+  float m, z, a;
+};
+struct SStat {
+  float m, z, z1;
+};
+
+__device__ __forceinline__ TStat tstat_init() { return TStat{kNegBig, 0.f, 0.f}; }
+__device__ __forceinline__ SStat sstat_init() { return SStat{kNegBig, 0.f, 0.f}; }
+
+__device__ __forceinline__ TStat merge(TStat p, TStat q, float k) {
+  const float m = fmaxf(p.m, q.m);
+  const float rp = fast_exp2((p.m - m) * k), rq = fast_exp2((q.m - m) * k);
+  return TStat{m, p.z * rp + q.z * rq, p.a * rp + q.a * rq};
+}
+
+template <bool CE>
+__device__ __forceinline__ SStat merge(SStat p, SStat q, float k) {
+  const float m = fmaxf(p.m, q.m);
+  const float dp = p.m - m, dq = q.m - m;
+  SStat r{m, p.z * fast_exp2(dp * k) + q.z * fast_exp2(dq * k), 0.f};
+  if (CE) r.z1 = p.z1 * fast_exp2(dp * kLog2e) + q.z1 * fast_exp2(dq * kLog2e);
+  return r;
+}
+
+// Reduction over WIDTH (<= 64, power of two) adjacent lanes.
+template <int WIDTH, bool CE>
+__device__ __forceinline__ void lane_reduce(TStat& t, SStat& s, float k) {
+#pragma unroll
+  for (int off = WIDTH / 2; off > 0; off >>= 1) {
+    const TStat ot{__shfl_xor(t.m, off, kWave), __shfl_xor(t.z, off, kWave), __shfl_xor(t.a, off, kWave)};
+    SStat os{__shfl_xor(s.m, off, kWave), __shfl_xor(s.z, off, kWave), 0.f};
+    if (CE) os.z1 = __shfl_xor(s.z1, off, kWave);
+    t = merge(t, ot, k);
+    s = merge<CE>(s, os, k);
+  }
+}
+
+// Folds N (teacher, student) logit pairs into the states.  The block's own
+// maxima are taken first, so each element costs one fma and one exp2 per
+// operand (two for the student when the CE term is on), and the running
+// states are rescaled once per block.
+template <int N, bool CE>
+__device__ __forceinline__ void fold(TStat& st, SStat& ss, const float (&t)[N], const float (&s)[N], float k) {
+  float mt = t[0], ms = s[0];
+#pragma unroll
+  for (int i = 1; i < N; ++i) {
+    mt = fmaxf(mt, t[i]);
+    ms = fmaxf(ms, s[i]);
+  }
+  const float mtk = mt * k, msk = ms * k, ms1 = ms * kLog2e;
+  float zt = 0.f, at = 0.f, zs = 0.f, z1 = 0.f;
+#pragma unroll
+  for (int i = 0; i < N; ++i) {
+    const float et = fast_exp2(fmaf(t[i], k, -mtk));
+    zt += et;
+    at = fmaf(et, t[i] - s[i], at);
+    zs += fast_exp2(fmaf(s[i], k, -msk));
+    if (CE) z1 += fast_exp2(fmaf(s[i], kLog2e, -ms1));
+  }
+  st = merge(st, TStat{mt, zt, at}, k);
+  ss = merge<CE>(ss, SStat{ms, zs, z1}, k);
+}
+
+template <typename T>
+struct Vec16 {
+  static constexpr int N = 16 / sizeof(T);
+  T v[N];
+};
+
+template <typename T>
+__device__ __forceinline__ Vec16<T> load16(const T* p) {
+  const u32x4 raw = *reinterpret_cast<const u32x4*>(p);
+  Vec16<T> r;
+  __builtin_memcpy(&r, &raw, 16);
+  return r;
+}
+
+template <typename T>
+__device__ __forceinline__ void store16(T* p, const Vec16<T>& v) {
+  u32x4 raw;
+  __builtin_memcpy(&raw, &v, 16);
+  *reinterpret_cast<u32x4*>(p) = raw;
+}
+
+// Everything a row kernel needs; passed by value.
+struct KdArgs {
+  const void* s;
+  const void* t;
+  const uint8_t* mask;    // KD row selection, may be null (all rows)
+  const int64_t* labels;  // CE labels, may be null (no CE term)
+  int64_t ignore_index;
+  int64_t n_rows, V, ld_s, ld_t, ld_g;
+  float k;          // inv_T * log2(e)
+  float kd_gscale;  // kd_scale * inv_T   (gradient factor of the KD term before the 1/B)
+  float ce_weight;
+  const int* counts;  // device: [0] KD rows, [1] CE rows, [2] rows with any term; null = all n_rows carry KD only
+  float* row_kd;      // per-row KD loss terms (0 for unselected rows)
+  float* row_ce;      // per-row CE loss terms
+  void* grad;         // may be null
+};
+
+struct RowJob {
+  bool kd, ce;
+  int64_t label;
+};
+
+__device__ __forceinline__ RowJob row_job(const KdArgs& a, int64_t row) {
+  RowJob j;
+  j.kd = a.mask ? (a.mask[row] != 0) : true;
+  j.ce = false;
+  j.label = 0;
+  if (a.labels) {
+    j.label = a.labels[row];
+    j.ce = (j.label != a.ignore_index) && j.label >= 0 && j.label < a.V;
+  }
+  return j;
+}
+
+// Final per-row numbers from the merged states.
+struct RowFinal {
+  float lse_t, lse_s, lse1;  // log2 domain
+  float g_kd, g_ce;          // gradient factors (0 when the term is off for this row)
+};
+
+template <typename T, bool CE>
+__device__ __forceinline__ RowFinal finish_row(const KdArgs& a, const RowJob& j, int64_t row, const TStat& st,
+                                               const SStat& ss, const T* srow, bool writer) {
+  RowFinal f;
+  f.lse_t = st.m * a.k + log2f(st.z);
+  f.lse_s = ss.m * a.k + log2f(ss.z);
+  f.lse1 = CE ? ss.m * kLog2e + log2f(ss.z1) : 0.f;
+  const float n_kd = a.counts ? (float)a.counts[0] : (float)a.n_rows;
+  f.g_kd = j.kd ? a.kd_gscale / n_kd : 0.f;
+  f.g_ce = (CE && j.ce) ? a.ce_weight / (float)a.counts[1] : 0.f;
+  if (writer) {
+    a.row_kd[row] = j.kd ? kLn2 * (a.k * st.a / st.z - f.lse_t + f.lse_s) : 0.f;
+    if (CE) a.row_ce[row] = j.ce ? kLn2 * (f.lse1 - to_f32(srow[j.label]) * kLog2e) : 0.f;
+  }
+  return f;
+}
+
+template <typename T, bool CE>
+__device__ __forceinline__ T grad_one(T tv, T sv, bool hit, float k, const RowFinal& f) {
+  const float sf = to_f32(sv);
+  const float p = fast_exp2(fmaf(to_f32(tv), k, -f.lse_t));
+  const float q = fast_exp2(fmaf(sf, k, -f.lse_s));
+  float g = f.g_kd * (q - p);
+  if (CE) {
+    const float r = fast_exp2(fmaf(sf, kLog2e, -f.lse1));
+    g = fmaf(f.g_ce, r - (hit ? 1.f : 0.f), g);
+  }
+  return from_f32<T>(g);
+}
+
+template <typename T, int GROUP>
+__device__ __forceinline__ void zero_row(T* grow, int64_t V, int gtid) {
+  constexpr int VEC = Vec16<T>::N;
+  const uint32_t mis = (uint32_t)((uintptr_t)grow & 15u);
+  int64_t head = (int64_t)(((16u - mis) & 15u) / sizeof(T));
+  if (head > V) head = V;
+  const int64_t nvec = (V - head) / VEC, tail0 = head + nvec * VEC;
+  const T zero = from_f32<T>(0.f);
+  Vec16<T> z;
+#pragma unroll
+  for (int i = 0; i < VEC; ++i) z.v[i] = zero;
+  for (int64_t i = gtid; i < head; i += GROUP) grow[i] = zero;
+  for (int64_t v = gtid; v < nvec; v += GROUP) store16(grow + head + v * VEC, z);
+  for (int64_t i = tail0 + gtid; i < V; i += GROUP) grow[i] = zero;
+}
+
+struct RowGeom {
+  int64_t head, nvec, tail0;
+};
+
+// Split of a row into scalar head, 16-byte vectors and scalar tail by the
+// common misalignment of its pointers; everything is "head" when they disagree.
+template <typename T>
+__device__ __forceinline__ RowGeom row_geom(const T* srow, const T* trow, const T* grow, int64_t V) {
+  constexpr int VEC = Vec16<T>::N;
+  const uint32_t mis_s = (uint32_t)((uintptr_t)srow & 15u), mis_t = (uint32_t)((uintptr_t)trow & 15u);
+  const uint32_t mis_g = grow ? (uint32_t)((uintptr_t)grow & 15u) : mis_s;
+  RowGeom g;
+  g.head = (mis_s == mis_t && mis_s == mis_g) ? (int64_t)(((16u - mis_s) & 15u) / sizeof(T)) : V;
+  if (g.head > V) g.head = V;
+  g.nvec = (V - g.head) / VEC;
+  g.tail0 = g.head + g.nvec * VEC;
+  return g;
+}
+
+// ---------------------------------------------------------------------------
+// Narrow and medium rows: one launch.  The row pair is held in registers
+// between the statistics and the gradient (KREG 16-byte vectors per thread
+// and operand, all loads issued up front), so each logit is read once; the
+// launcher guarantees ceil(V / VEC) + 1 <= KREG * GROUP.
+// ---------------------------------------------------------------------------
+template <typename T, int BLOCK, int GROUP, int KREG, bool CE>
+__global__ __launch_bounds__(BLOCK) void kd_rows_kernel(const KdArgs a) {
+  constexpr int VEC = Vec16<T>::N;
+  constexpr int NW = GROUP / kWave;  // wavefronts per group (0 for sub-wavefront groups)
+  __shared__ TStat lds_t[BLOCK / kWave];
+  __shared__ SStat lds_s[BLOCK / kWave];
+
+  const int gtid = threadIdx.x % GROUP;
+  const int64_t row = (int64_t)blockIdx.x * (BLOCK / GROUP) + threadIdx.x / GROUP;
+  // With GROUP == BLOCK the whole workgroup shares one row, so the early
+  // exits below are uniform; smaller groups never reach a __syncthreads and
+  // only shuffle among their own lanes.
+  if (row >= a.n_rows) return;
+  const T* srow = reinterpret_cast<const T*>(a.s) + row * a.ld_s;
+  const T* trow = reinterpret_cast<const T*>(a.t) + row * a.ld_t;
+  T* grow = a.grad ? reinterpret_cast<T*>(a.grad) + row * a.ld_g : nullptr;
+  const RowJob job = row_job(a, row);
+  const int64_t V = a.V;
+
+  if (!job.kd && !job.ce) {
+    if (gtid == 0) {
+      a.row_kd[row] = 0.f;
+      if (CE) a.row_ce[row] = 0.f;
+    }
+    if (grow) zero_row<T, GROUP>(grow, V, gtid);
+    return;
+  }
+
+  const RowGeom g = row_geom<T>(srow, trow, grow, V);
+  Vec16<T> rt[KREG], rs[KREG];
+#pragma unroll
+  for (int j = 0; j < KREG; ++j) {
+    const int64_t v = gtid + (int64_t)j * GROUP;
+    if (v < g.nvec) {
+      rt[j] = load16(trow + g.head + v * VEC);
+      rs[j] = load16(srow + g.head + v * VEC);
+    }
+  }
+
+  TStat st = tstat_init();
+  SStat ss = sstat_init();
+  {
+    float xt1[1], xs1[1];
+    for (int64_t i = gtid; i < g.head; i += GROUP) {
+      xt1[0] = to_f32(trow[i]);
+      xs1[0] = to_f32(srow[i]);
+      fold<1, CE>(st, ss, xt1, xs1, a.k);
+    }
+    for (int64_t i = g.tail0 + gtid; i < V; i += GROUP) {
+      xt1[0] = to_f32(trow[i]);
+      xs1[0] = to_f32(srow[i]);
+      fold<1, CE>(st, ss, xt1, xs1, a.k);
+    }
+    float xt[VEC], xs[VEC];
+#pragma unroll
+    for (int j = 0; j < KREG; ++j) {
+      if (gtid + (int64_t)j * GROUP < g.nvec) {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+          xt[i] = to_f32(rt[j].v[i]);
+          xs[i] = to_f32(rs[j].v[i]);
+        }
+        fold<VEC, CE>(st, ss, xt, xs, a.k);
+      }
+    }
+  }
+
+  lane_reduce<(GROUP < kWave ? GROUP : kWave), CE>(st, ss, a.k);
+  if (NW > 1) {
+    const int w = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    if (lane == 0) {
+      lds_t[w] = st;
+      lds_s[w] = ss;
+    }
+    __syncthreads();
+    st = lds_t[0];
+    ss = lds_s[0];
+#pragma unroll
+    for (int i = 1; i < NW; ++i) {
+      st = merge(st, lds_t[i], a.k);
+      ss = merge<CE>(ss, lds_s[i], a.k);
+    }
+  }
+
+  const RowFinal f = finish_row<T, CE>(a, job, row, st, ss, srow, gtid == 0);
+  if (!grow) return;
+
+  for (int64_t i = gtid; i < g.head; i += GROUP) grow[i] = grad_one<T, CE>(trow[i], srow[i], i == job.label, a.k, f);
+  for (int64_t i = g.tail0 + gtid; i < V; i += GROUP)
+    grow[i] = grad_one<T, CE>(trow[i], srow[i], i == job.label, a.k, f);
+#pragma unroll
+  for (int j = 0; j < KREG; ++j) {
+    const int64_t v = gtid + (int64_t)j * GROUP;
+    if (v < g.nvec) {
+      Vec16<T> o;
+      const int64_t e0 = g.head + v * VEC;
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) o.v[i] = grad_one<T, CE>(rt[j].v[i], rs[j].v[i], e0 + i == job.label, a.k, f);
+      store16(grow + e0, o);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Wide rows: a row is cut into parts of kPartVecs 16-byte vectors, one
+// short-lived 256-thread workgroup per (row, part), two launches:
+//   pass 1, grid = every (row, part): rows with a loss term -> partial state
+//           of the part (part_stats[row][part]); other rows -> zero-fill of
+//           the part's gradient.  The first kind is bound by exp2 throughput,
+//           the second by HBM writes, and they overlap.
+//   pass 2, bounded grid walking the (row with a term, part) items of the
+//           compacted row list: merges the row's partial states, writes the
+//           part's gradient.  Its reads come out of the 256 MB last-level
+//           cache when those rows fit there.
+// ---------------------------------------------------------------------------
+constexpr int kPartBlock = 256;
+constexpr int kPartPerThread = 4;
+constexpr int kPartVecs = kPartBlock * kPartPerThread;
+constexpr int kPass2MaxGrid = 8192;
+
+struct PartStat {  // 32 bytes
+  float mt, zt, at, ms, zs, z1, pad0, pad1;
+};
+
+template <typename T, bool CE>
+__global__ __launch_bounds__(kPartBlock) void kd_wide_pass1_kernel(const KdArgs a, int parts,
+                                                                   PartStat* __restrict__ part_stats) {
+  constexpr int VEC = Vec16<T>::N;
+  __shared__ TStat lds_t[kPartBlock / kWave];
+  __shared__ SStat lds_s[kPartBlock / kWave];
+  const int64_t row = blockIdx.x / parts;
+  const int part = (int)(blockIdx.x % parts);
+  const int tid = threadIdx.x;
+  const int64_t v0 = (int64_t)part * kPartVecs;
+  const int64_t V = a.V;
+  const RowJob job = row_job(a, row);
+
+  if (!job.kd && !job.ce) {
+    if (part == 0 && tid == 0) {
+      a.row_kd[row] = 0.f;
+      if (CE) a.row_ce[row] = 0.f;
+    }
+    if (!a.grad) return;
+    T* grow = reinterpret_cast<T*>(a.grad) + row * a.ld_g;
+    const uint32_t mis = (uint32_t)((uintptr_t)grow & 15u);
+    int64_t head = (int64_t)(((16u - mis) & 15u) / sizeof(T));
+    if (head > V) head = V;
+    const int64_t nvec = (V - head) / VEC, tail0 = head + nvec * VEC;
+    const T zero = from_f32<T>(0.f);
+    Vec16<T> z;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) z.v[i] = zero;
+    if (part == 0)
+      for (int64_t i = tid; i < head; i += kPartBlock) grow[i] = zero;
+    if (part == parts - 1)
+      for (int64_t i = tail0 + tid; i < V; i += kPartBlock) grow[i] = zero;
+#pragma unroll
+    for (int j = 0; j < kPartPerThread; ++j) {
+      const int64_t v = v0 + tid + j * kPartBlock;
+      if (v < nvec) store16(grow + head + v * VEC, z);
+    }
+    return;
+  }
+
+  const T* srow = reinterpret_cast<const T*>(a.s) + row * a.ld_s;
+  const T* trow = reinterpret_cast<const T*>(a.t) + row * a.ld_t;
+  // the row is cut by the alignment of s and t alone; pass 2 cuts it the same way
+  const RowGeom g = row_geom<T>(srow, trow, nullptr, V);
+  Vec16<T> rt[kPartPerThread], rs[kPartPerThread];
+#pragma unroll
+  for (int j = 0; j < kPartPerThread; ++j) {
+    const int64_t v = v0 + tid + j * kPartBlock;
+    if (v < g.nvec) {
+      rt[j] = load16(trow + g.head + v * VEC);
+      rs[j] = load16(srow + g.head + v * VEC);
+    }
+  }
+  // Ragged ends of the row (fewer than VEC elements each, unless the rows are
+  // misaligned against each other and everything is "head"): folded into
+  // per-thread states the slow way.
+  TStat st = tstat_init();
+  SStat ss = sstat_init();
+  float xt1[1], xs1[1];
+  if (part == 0) {
+    for (int64_t i = tid; i < g.head; i += kPartBlock) {
+      xt1[0] = to_f32(trow[i]);
+      xs1[0] = to_f32(srow[i]);
+      fold<1, CE>(st, ss, xt1, xs1, a.k);
+    }
+  }
+  if (part == parts - 1) {
+    for (int64_t i = g.tail0 + tid; i < V; i += kPartBlock) {
+      xt1[0] = to_f32(trow[i]);
+      xs1[0] = to_f32(srow[i]);
+      fold<1, CE>(st, ss, xt1, xs1, a.k);
+    }
+  }
+  // Vector body.  The maxima are settled first, over the thread's vectors and
+  // then across the wavefront, so that every lane exponentiates against the
+  // same reference and the sums combine by plain addition: no per-step
+  // rescaling and no exp2 in the cross-lane reduction.
+  float mt = st.m, ms = ss.m;
+  float ft[kPartPerThread][VEC], fs[kPartPerThread][VEC];
+#pragma unroll
+  for (int j = 0; j < kPartPerThread; ++j) {
+    if (v0 + tid + j * kPartBlock < g.nvec) {
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) {
+        ft[j][i] = to_f32(rt[j].v[i]);
+        fs[j][i] = to_f32(rs[j].v[i]);
+        mt = fmaxf(mt, ft[j][i]);
+        ms = fmaxf(ms, fs[j][i]);
+      }
+    }
+  }
+  const float wmt = wave_max(mt), wms = wave_max(ms);
+  const float wmtk = wmt * a.k, wmsk = wms * a.k, wms1 = wms * kLog2e;
+  // ragged-end sums re-based onto the wavefront's maxima
+  const float rbt = fast_exp2((st.m - wmt) * a.k), rbs = fast_exp2((ss.m - wms) * a.k);
+  float zt = st.z * rbt, at = st.a * rbt, zs = ss.z * rbs;
+  float z1 = CE ? ss.z1 * fast_exp2((ss.m - wms) * kLog2e) : 0.f;
+#pragma unroll
+  for (int j = 0; j < kPartPerThread; ++j) {
+    if (v0 + tid + j * kPartBlock < g.nvec) {
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) {
+        const float et = fast_exp2(fmaf(ft[j][i], a.k, -wmtk));
+        zt += et;
+        at = fmaf(et, ft[j][i] - fs[j][i], at);
+        zs += fast_exp2(fmaf(fs[j][i], a.k, -wmsk));
+        if (CE) z1 += fast_exp2(fmaf(fs[j][i], kLog2e, -wms1));
+      }
+    }
+  }
+  zt = wave_sum(zt);
+  at = wave_sum(at);
+  zs = wave_sum(zs);
+  if (CE) z1 = wave_sum(z1);
+  const int w = tid / kWave, lane = tid % kWave;
+  if (lane == 0) {
+    lds_t[w] = TStat{wmt, zt, at};
+    lds_s[w] = SStat{wms, zs, z1};
+  }
+  __syncthreads();
+  if (tid == 0) {
+    TStat bt = lds_t[0];
+    SStat bs = lds_s[0];
+#pragma unroll
+    for (int i = 1; i < kPartBlock / kWave; ++i) {
+      bt = merge(bt, lds_t[i], a.k);
+      bs = merge<CE>(bs, lds_s[i], a.k);
+    }
+    part_stats[row * parts + part] = PartStat{bt.m, bt.z, bt.a, bs.m, bs.z, bs.z1, 0.f, 0.f};
+  }
+}
+
+template <typename T, bool CE>
+__global__ __launch_bounds__(kPartBlock) void kd_wide_pass2_kernel(const KdArgs a, int parts,
+                                                                   const PartStat* __restrict__ part_stats,
+                                                                   const int* __restrict__ sel_rows) {
+  constexpr int VEC = Vec16<T>::N;
+  const int64_t items = (a.counts ? (int64_t)a.counts[2] : a.n_rows) * parts;
+  const int tid = threadIdx.x;
+  const int64_t V = a.V;
+
+  for (int64_t item = blockIdx.x; item < items; item += gridDim.x) {
+    const int64_t row = sel_rows ? (int64_t)sel_rows[item / parts] : item / parts;
+    const int part = (int)(item % parts);
+    const int64_t v0 = (int64_t)part * kPartVecs;
+    const T* srow = reinterpret_cast<const T*>(a.s) + row * a.ld_s;
+    const T* trow = reinterpret_cast<const T*>(a.t) + row * a.ld_t;
+    T* grow = a.grad ? reinterpret_cast<T*>(a.grad) + row * a.ld_g : nullptr;
+    const RowJob job = row_job(a, row);
+    const RowGeom g = row_geom<T>(srow, trow, nullptr, V);
+    const bool gvec = grow && (((uintptr_t)grow & 15u) == ((uintptr_t)srow & 15u));
+
+    Vec16<T> rt[kPartPerThread], rs[kPartPerThread];
+    if (grow) {
+#pragma unroll
+      for (int j = 0; j < kPartPerThread; ++j) {
+        const int64_t v = v0 + tid + j * kPartBlock;
+        if (v < g.nvec) {
+          rt[j] = load16(trow + g.head + v * VEC);
+          rs[j] = load16(srow + g.head + v * VEC);
+        }
+      }
+    }
+    // every thread merges the row's few partial states itself (uniform loads)
+    TStat st = tstat_init();
+    SStat ss = sstat_init();
+    for (int p = 0; p < parts; ++p) {
+      const PartStat ps = part_stats[row * parts + p];
+      st = merge(st, TStat{ps.mt, ps.zt, ps.at}, a.k);
+      ss = merge<CE>(ss, SStat{ps.ms, ps.zs, ps.z1}, a.k);
+    }
+    const RowFinal f = finish_row<T, CE>(a, job, row, st, ss, srow, part == 0 && tid == 0);
+    if (!grow) continue;
+    if (part == 0)
+      for (int64_t i = tid; i < g.head; i += kPartBlock)
+        grow[i] = grad_one<T, CE>(trow[i], srow[i], i == job.label, a.k, f);
+    if (part == parts - 1)
+      for (int64_t i = g.tail0 + tid; i < V; i += kPartBlock)
+        grow[i] = grad_one<T, CE>(trow[i], srow[i], i == job.label, a.k, f);
+#pragma unroll
+    for (int j = 0; j < kPartPerThread; ++j) {
+      const int64_t v = v0 + tid + j * kPartBlock;
+      if (v < g.nvec) {
+        Vec16<T> o;
+        const int64_t e0 = g.head + v * VEC;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) o.v[i] = grad_one<T, CE>(rt[j].v[i], rs[j].v[i], e0 + i == job.label, a.k, f);
+        if (gvec) {
+          store16(grow + e0, o);
+        } else {
+#pragma unroll
+          for (int i = 0; i < VEC; ++i) grow[e0 + i] = o.v[i];
+        }
+      }
+    }
+  }
+}
+
+// Parts a row of V elements of T is cut into (0: the row is narrow enough for
+// the single-launch kernel).
+template <typename T>
+inline int64_t kd_parts(int64_t V) {
+  const int64_t vecs = (V + Vec16<T>::N - 1) / Vec16<T>::N + 1;
+  if (vecs <= 256 * 4) return 0;
+  return (vecs + kPartVecs - 1) / kPartVecs;
+}
+
+// counts[0] = rows with the KD term, counts[1] = rows with the CE term,
+// counts[2] = rows with either; sel_rows (optional) = indices of the latter in
+// ascending order.  One workgroup; thread i owns the i-th contiguous slice.
+__global__ __launch_bounds__(1024) void kd_count_kernel(const KdArgs a, int* __restrict__ counts,
+                                                        int* __restrict__ sel_rows) {
+  __shared__ int scan[1024];
+  __shared__ int tot_kd[1024 / kWave], tot_ce[1024 / kWave];
+  const int tid = threadIdx.x;
+  const int64_t n = a.n_rows;
+  const int64_t per = (n + 1023) / 1024;
+  const int64_t lo = tid * per, hi = (lo + per < n) ? lo + per : n;
+  int c_any = 0, c_kd = 0, c_ce = 0;
+  for (int64_t i = lo; i < hi; ++i) {
+    const RowJob j = row_job(a, i);
+    c_kd += j.kd;
+    c_ce += j.ce;
+    c_any += (j.kd || j.ce);
+  }
+  // the two plain totals: wavefront sums (exact in float up to 2^24 rows), then one thread adds them
+  const float wkd = wave_sum((float)c_kd), wce = wave_sum((float)c_ce);
+  if (tid % kWave == 0) {
+    tot_kd[tid / kWave] = (int)wkd;
+    tot_ce[tid / kWave] = (int)wce;
+  }
+  scan[tid] = c_any;
+  __syncthreads();
+  // inclusive Hillis-Steele scan over the 1024 per-thread counts
+  for (int off = 1; off < 1024; off <<= 1) {
+    const int add = (tid >= off) ? scan[tid - off] : 0;
+    __syncthreads();
+    scan[tid] += add;
+    __syncthreads();
+  }
+  if (tid == 0) {
+    int k = 0, c = 0;
+    for (int i = 0; i < 1024 / kWave; ++i) {
+      k += tot_kd[i];
+      c += tot_ce[i];
+    }
+    counts[0] = k;
+    counts[1] = c;
+    counts[2] = scan[1023];
+  }
+  if (sel_rows) {
+    int pos = scan[tid] - c_any;
+    for (int64_t i = lo; i < hi; ++i) {
+      const RowJob j = row_job(a, i);
+      if (j.kd || j.ce) sel_rows[pos++] = (int)i;
+    }
+  }
+}
+
+// loss = kd_scale * sum(row_kd) / counts[0] + ce_weight * sum(row_ce) / counts[1], fixed summation order.
+__global__ __launch_bounds__(1024) void kd_finalize_kernel(const float* __restrict__ row_kd,
+                                                           const float* __restrict__ row_ce, int64_t n,
+                                                           float kd_scale, float ce_weight,
+                                                           const int* __restrict__ counts /* null: n KD rows */,
+                                                           float* __restrict__ out) {
+  __shared__ float lds[1024 / kWave];
+  float akd = 0.f, ace = 0.f;
+  for (int64_t i = threadIdx.x; i < n; i += 1024) {
+    akd += row_kd[i];
+    if (row_ce) ace += row_ce[i];
+  }
+  const float skd = block_sum<1024 / kWave>(akd, lds);
+  const float sce = block_sum<1024 / kWave>(ace, lds);
+  if (threadIdx.x == 0) {
+    // 0/0 = NaN for an empty selection, as the reference gives
+    float loss = kd_scale * (skd / (counts ? (float)counts[0] : (float)n));
+    if (row_ce) loss += ce_weight * (sce / (float)counts[1]);
+    *out = loss;
+  }
+}
+
+struct KdWorkspace {
+  int* counts;
+  float* row_kd;
+  float* row_ce;
+  int* sel_rows;
+  PartStat* part_stats;
+};
+
+inline size_t kd_rows4(int64_t n_rows) { return (size_t)((n_rows * 4 + 31) / 32) * 32; }
+
+inline KdWorkspace kd_carve(void* ws, int64_t n_rows) {
+  char* b = reinterpret_cast<char*>(ws);
+  const size_t r4 = kd_rows4(n_rows);
+  KdWorkspace w;
+  w.counts = reinterpret_cast<int*>(b);
+  w.row_kd = reinterpret_cast<float*>(b + 32);
+  w.row_ce = reinterpret_cast<float*>(b + 32 + r4);
+  w.sel_rows = reinterpret_cast<int*>(b + 32 + 2 * r4);
+  w.part_stats = reinterpret_cast<PartStat*>(b + 32 + 3 * r4);
+  return w;
+}
+
+template <typename T, bool CE>
+int launch_kd_t(KdArgs a, float kd_scale, void* ws, float* loss_out, hipStream_t stream) {
+  const KdWorkspace w = kd_carve(ws, a.n_rows);
+  const int64_t parts = kd_parts<T>(a.V);
+  const bool counted = a.mask || a.labels;  // otherwise all rows carry the KD term and nothing else
+  a.counts = counted ? w.counts : nullptr;
+  a.row_kd = w.row_kd;
+  a.row_ce = w.row_ce;
+  const bool compact = parts && counted;
+  int rc = TS_OK;
+  if (counted) {
+    hipLaunchKernelGGL(kd_count_kernel, dim3(1), dim3(1024), 0, stream, a, w.counts,
+                       compact ? w.sel_rows : (int*)nullptr);
+    rc = check_launch();
+    if (rc) return rc;
+  }
+  if (a.n_rows == 0) {
+    hipLaunchKernelGGL(kd_finalize_kernel, dim3(1), dim3(1024), 0, stream, w.row_kd,
+                       CE ? w.row_ce : (const float*)nullptr, (int64_t)0, kd_scale, a.ce_weight, a.counts, loss_out);
+    return check_launch();
+  }
+  // 16-byte vectors a row can span, counting a ragged first and last one
+  const int64_t vecs = (a.V + Vec16<T>::N - 1) / Vec16<T>::N + 1;
+#define TS_KD_LAUNCH(BLOCK, GROUP, KREG)                                                                     \
+  hipLaunchKernelGGL((kd_rows_kernel<T, BLOCK, GROUP, KREG, CE>),                                            \
+                     dim3((unsigned)((a.n_rows + (BLOCK / GROUP) - 1) / (BLOCK / GROUP))), dim3(BLOCK), 0,   \
+                     stream, a)
+  if (vecs <= 16 * 2) {
+    TS_KD_LAUNCH(256, 16, 2);
+  } else if (vecs <= 32 * 2) {
+    TS_KD_LAUNCH(256, 32, 2);
+  } else if (vecs <= 64 * 4) {
+    TS_KD_LAUNCH(256, 64, 4);
+  } else if (parts == 0) {
+    TS_KD_LAUNCH(256, 256, 4);
+  } else {
+    const int64_t items = a.n_rows * parts;
+    if (items > 0x7fffffffLL) return TS_ERR_RANGE;
+    hipLaunchKernelGGL((kd_wide_pass1_kernel<T, CE>), dim3((unsigned)items), dim3(kPartBlock), 0, stream, a,
+                       (int)parts, w.part_stats);
+    rc = check_launch();
+    if (rc) return rc;
+    const int64_t grid2 = items < kPass2MaxGrid ? items : kPass2MaxGrid;
+    hipLaunchKernelGGL((kd_wide_pass2_kernel<T, CE>), dim3((unsigned)grid2), dim3(kPartBlock), 0, stream, a,
+                       (int)parts, w.part_stats, compact ? w.sel_rows : (const int*)nullptr);
+  }
+#undef TS_KD_LAUNCH
+  rc = check_launch();
+  if (rc) return rc;
+  hipLaunchKernelGGL(kd_finalize_kernel, dim3(1), dim3(1024), 0, stream, w.row_kd, CE ? w.row_ce : (const float*)nullptr,
+                     a.n_rows, kd_scale, a.ce_weight, a.counts, loss_out);
+  return check_launch();
+}
+
+template <typename T>
+int launch_kd(const KdArgs& a, float kd_scale, void* ws, float* loss_out, hipStream_t stream) {
+  return a.labels ? launch_kd_t<T, true>(a, kd_scale, ws, loss_out, stream)
+                  : launch_kd_t<T, false>(a, kd_scale, ws, loss_out, stream);
+}
+
+}  // namespace ts
+
+extern "C" {
+
+size_t ts_kd_workspace_bytes(int64_t n_rows, int64_t V, int dtype) {
+  if (n_rows < 0) n_rows = 0;
+  if (V < 0) V = 0;
+  const int64_t parts = (dtype == TS_F32) ? ts::kd_parts<float>(V) : ts::kd_parts<ts::bf16_t>(V);
+  return 32 + 3 * ts::kd_rows4(n_rows) + (size_t)(n_rows * parts) * sizeof(ts::PartStat);
+}
+
+int ts_kdce_fwd_bwd(const void* s, const void* t, const uint8_t* row_mask, const int64_t* labels,
+                    int64_t ignore_index, int64_t n_rows, int64_t V, int64_t ld_s, int64_t ld_t, float inv_T,
+                    float kd_scale, float ce_weight, void* workspace, float* loss_out, void* grad, int64_t ld_g,
+                    int dtype, ts_stream_t stream) {
+  if (!s || !t || !workspace || !loss_out) return TS_ERR_ARG;
+  if (n_rows < 0 || V <= 0 || ld_s < V || ld_t < V || (grad && ld_g < V)) return TS_ERR_ARG;
+  if (dtype != TS_F32 && dtype != TS_BF16 && dtype != TS_F16) return TS_ERR_ARG;
+  if (!(inv_T > 0.f)) return TS_ERR_ARG;
+  // one workgroup (or group of lanes) per row; counts are summed as floats
+  if (n_rows > (1 << 24)) return TS_ERR_RANGE;
+  const uintptr_t esz = (dtype == TS_F32) ? 4 : 2;
+  if (((uintptr_t)s | (uintptr_t)t | (uintptr_t)grad) & (esz - 1)) return TS_ERR_ALIGN;
+  if ((uintptr_t)labels & 7u) return TS_ERR_ALIGN;
+  if ((uintptr_t)workspace & 31u) return TS_ERR_ALIGN;
+  ts::KdArgs a;
+  a.s = s;
+  a.t = t;
+  a.mask = row_mask;
+  a.labels = labels;
+  a.ignore_index = ignore_index;
+  a.n_rows = n_rows;
+  a.V = V;
+  a.ld_s = ld_s;
+  a.ld_t = ld_t;
+  a.ld_g = ld_g;
+  a.k = inv_T * ts::kLog2e;
+  a.kd_gscale = kd_scale * inv_T;
+  a.ce_weight = ce_weight;
+  a.counts = nullptr;
+  a.row_kd = a.row_ce = nullptr;
+  a.grad = grad;
+  hipStream_t st = (hipStream_t)stream;
+  switch (dtype) {
+    case TS_F32: return ts::launch_kd<float>(a, kd_scale, workspace, loss_out, st);
+    case TS_BF16: return ts::launch_kd<ts::bf16_t>(a, kd_scale, workspace, loss_out, st);
+    default: return ts::launch_kd<ts::f16_t>(a, kd_scale, workspace, loss_out, st);
+  }
+}
+
+int ts_kd_fwd_bwd(const void* s, const void* t, const uint8_t* row_mask, int64_t n_rows, int64_t V, int64_t ld_s,
+                  int64_t ld_t, float inv_T, float loss_scale, void* workspace, float* loss_out, void* grad,
+                  int64_t ld_g, int dtype, ts_stream_t stream) {
+  return ts_kdce_fwd_bwd(s, t, row_mask, nullptr, 0, n_rows, V, ld_s, ld_t, inv_T, loss_scale, 0.f, workspace,
+                         loss_out, grad, ld_g, dtype, stream);
+}
+
+}  // extern "C"

@@ -49,9 +49,13 @@ def _scale_saved_grad(grad: Tensor, grad_output: Tensor, rows: int, cols: int) -
 # ---------------------------------------------------------------------------
 
 class _KDSoftTargetFn(torch.autograd.Function):
+    """KD soft-target term, optionally with the hard-label CE term, in one pass
+    over the student logits."""
+
     @staticmethod
-    def forward(ctx, out_s: Tensor, out_t: Tensor, row_mask: Optional[Tensor], T: float, weight: float):
-        _require_cuda(out_s, out_t, row_mask)
+    def forward(ctx, out_s: Tensor, out_t: Tensor, row_mask: Optional[Tensor], T: float, weight: float,
+                labels: Optional[Tensor] = None, ce_weight: float = 0.0, ignore_index: int = -100):
+        _require_cuda(out_s, out_t, row_mask, labels)
         if out_s.shape != out_t.shape:
             raise ValueError(f"student/teacher logits differ in shape: {tuple(out_s.shape)} vs {tuple(out_t.shape)}")
         if out_s.dtype != out_t.dtype:
@@ -71,18 +75,28 @@ class _KDSoftTargetFn(torch.autograd.Function):
                 m = m != 0
             m = m.contiguous().view(torch.uint8)
             mask_ptr = m.data_ptr()
+        label_ptr = None
+        if labels is not None:
+            lab = labels.detach().reshape(-1)
+            if lab.numel() != rows:
+                raise ValueError(f"{lab.numel()} labels for {rows} rows")
+            if lab.dtype != torch.int64:
+                lab = lab.to(torch.int64)
+            lab = lab.contiguous()
+            label_ptr = lab.data_ptr()
         need_grad = ctx.needs_input_grad[0]
         lib = _lib.lib()
         dev = s.device
-        ws = torch.empty(lib.ts_kd_workspace_bytes(rows, V, _lib.dtype_code(s.dtype)), dtype=torch.uint8, device=dev)
+        code = _lib.dtype_code(s.dtype)
+        ws = torch.empty(lib.ts_kd_workspace_bytes(rows, V, code), dtype=torch.uint8, device=dev)
         loss = torch.empty((), dtype=torch.float32, device=dev)
         grad = torch.empty_like(s) if need_grad else None
         with torch.cuda.device(dev):
-            status = lib.ts_kd_fwd_bwd(s.data_ptr(), t.data_ptr(), mask_ptr, rows, V, V, V, 1.0 / T,
-                                       T * T * weight, ws.data_ptr(), loss.data_ptr(),
-                                       None if grad is None else grad.data_ptr(), V,
-                                       _lib.dtype_code(s.dtype), _lib.current_stream_ptr(dev))
-        _lib.check(status, "ts_kd_fwd_bwd")
+            status = lib.ts_kdce_fwd_bwd(s.data_ptr(), t.data_ptr(), mask_ptr, label_ptr, int(ignore_index), rows, V,
+                                         V, V, 1.0 / T, T * T * weight, float(ce_weight), ws.data_ptr(),
+                                         loss.data_ptr(), None if grad is None else grad.data_ptr(), V, code,
+                                         _lib.current_stream_ptr(dev))
+        _lib.check(status, "ts_kdce_fwd_bwd")
         ctx.grad = grad
         ctx.shape = out_s.shape
         ctx.dims = (rows, V)
@@ -92,10 +106,10 @@ class _KDSoftTargetFn(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_output: Tensor):
         if ctx.grad is None:
-            return None, None, None, None, None
+            return (None,) * 8
         _once(ctx)
         grad = _scale_saved_grad(ctx.grad, grad_output, *ctx.dims)
-        return grad.view(ctx.shape), None, None, None, None
+        return (grad.view(ctx.shape),) + (None,) * 7
 
 
 def kd_soft_target_loss(out_s: Tensor, out_t: Tensor, T: float, weight: float = 1.0,
@@ -128,6 +142,67 @@ def distil_ce_loss(s_logits: Tensor, t_logits: Tensor, row_mask: Tensor, tempera
     selected rows, times ``temperature**2`` and ``alpha_ce``.  No row is copied:
     the kernel reads the mask and writes a dense gradient with zeros elsewhere."""
     return _KDSoftTargetFn.apply(s_logits, t_logits, row_mask, float(temperature), float(alpha_ce))
+
+
+def kd_ce_loss(out_s: Tensor, out_t: Tensor, labels: Tensor, T: float, kd_weight: float = 1.0,
+               ce_weight: float = 1.0, row_mask: Optional[Tensor] = None, ignore_index: int = -100) -> Tensor:
+    """``kd_weight * T^2 * KL(...)`` over the rows of ``row_mask`` plus
+    ``ce_weight * CrossEntropy(out_s, labels)`` over the rows whose label is not
+    ``ignore_index``, both means over their own row sets, in one pass over the
+    logits (benchmarks/soft_target/train_kd.py:439-453;
+    benchmarks/distilbert/distiller.py:719-744)."""
+    return _KDSoftTargetFn.apply(out_s, out_t, row_mask, float(T), float(kd_weight), labels, float(ce_weight),
+                                 int(ignore_index))
+
+
+class _CosineFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x: Tensor, y: Tensor, row_mask: Optional[Tensor], weight: float):
+        _require_cuda(x, y, row_mask)
+        if x.shape != y.shape or x.dtype != y.dtype:
+            raise ValueError("cosine loss inputs must agree in shape and dtype")
+        c = int(x.shape[-1])
+        xs = x.detach().reshape(-1, c)
+        ys = y.detach().reshape(-1, c)
+        xs = xs if xs.is_contiguous() else xs.contiguous()
+        ys = ys if ys.is_contiguous() else ys.contiguous()
+        n = int(xs.shape[0])
+        mask_ptr = None
+        if row_mask is not None:
+            m = row_mask.detach().reshape(-1)
+            if m.numel() != n:
+                raise ValueError(f"row mask has {m.numel()} entries for {n} rows")
+            if m.dtype != torch.bool:
+                m = m != 0
+            m = m.contiguous().view(torch.uint8)
+            mask_ptr = m.data_ptr()
+        lib = _lib.lib()
+        dev = xs.device
+        ws = torch.empty(lib.ts_cosine_workspace_bytes(n), dtype=torch.uint8, device=dev)
+        loss = torch.empty((), dtype=torch.float32, device=dev)
+        gx = torch.empty_like(xs) if ctx.needs_input_grad[0] else None
+        with torch.cuda.device(dev):
+            status = lib.ts_cosine_fwd_bwd(xs.data_ptr(), ys.data_ptr(), mask_ptr, n, c, weight, ws.data_ptr(),
+                                           loss.data_ptr(), None if gx is None else gx.data_ptr(),
+                                           _lib.dtype_code(xs.dtype), _lib.current_stream_ptr(dev))
+        _lib.check(status, "ts_cosine_fwd_bwd")
+        ctx.gx, ctx.shape, ctx.dims = gx, x.shape, (n, c)
+        ctx.backward_done = False
+        return loss
+
+    @staticmethod
+    def backward(ctx, grad_output: Tensor):
+        if ctx.gx is None:
+            return None, None, None, None
+        _once(ctx)
+        return _scale_saved_grad(ctx.gx, grad_output, *ctx.dims).view(ctx.shape), None, None, None
+
+
+def cosine_embedding_loss(x: Tensor, y: Tensor, row_mask: Optional[Tensor] = None, weight: float = 1.0) -> Tensor:
+    """``weight * CosineEmbeddingLoss(reduction="mean")(x[rows], y[rows], +1)`` over
+    the rows (last dimension = features) kept by ``row_mask``; gradient to ``x``
+    only (benchmarks/distilbert/distiller.py:756-770)."""
+    return _CosineFn.apply(x, y, row_mask, float(weight))
 
 
 # ---------------------------------------------------------------------------
@@ -257,3 +332,40 @@ def moco_contrastive_loss(online_view_1, online_view_2, target_view_1, target_vi
     temperature comes from ``extra_args.moco_t``."""
     return moco_contrastive_loss_pair(online_view_1, online_view_2, target_view_1, target_view_2,
                                       float(extra_args.moco_t))
+
+
+def soft_target_tspipe_loss(model_out: Tensor, ema_model_out: Tensor, label: Tensor, tspipe_args, args,
+                            epoch: int) -> Tensor:
+    """``tspipe_loss`` of benchmarks/soft_target/train_kd.py:439-453 for
+    ``args.kd_mode == 'st'``: hard-label cross entropy plus ``lambda_kd`` times
+    the soft-target KD term, both in one kernel pass."""
+    if getattr(args, "kd_mode", "st") != "st":
+        raise NotImplementedError("only kd_mode='st' runs on the fused kernel (kd_mode='logits' is a plain MSE)")
+    return kd_ce_loss(model_out, ema_model_out.detach(), label, args.T, kd_weight=args.lambda_kd, ce_weight=1.0)
+
+
+def distil_loss_fn(student_outputs, teacher_outputs, labels, tspipe_args, params, epoch: int) -> Tensor:
+    """``TSPipeDistiller.loss_fn`` of benchmarks/distilbert/distiller.py:711-772:
+    ``alpha_ce`` x masked KD, ``alpha_mlm`` x masked-LM cross entropy
+    (ignore_index -100) -- both in one pass over the logits -- and ``alpha_cos``
+    x cosine embedding loss on the last hidden states.  ``params`` carries
+    ``alpha_ce, alpha_mlm, alpha_clm, alpha_mse, alpha_cos, temperature,
+    restrict_ce_to_mask`` like the reference's LossComputeParam."""
+    s_logits, t_logits = student_outputs["logits"], teacher_outputs["logits"]
+    lm_labels, attention_mask = labels
+    if getattr(params, "alpha_clm", 0.0) > 0.0:
+        raise NotImplementedError("the causal-LM term (alpha_clm) is not on the fused path")
+    if getattr(params, "alpha_mse", 0.0) > 0.0:
+        raise NotImplementedError("the logits-MSE term (alpha_mse) is not on the fused path")
+    mask = (lm_labels > -1) if params.restrict_ce_to_mask else attention_mask
+    alpha_mlm = float(getattr(params, "alpha_mlm", 0.0))
+    if alpha_mlm > 0.0:
+        loss = kd_ce_loss(s_logits, t_logits, lm_labels, params.temperature, kd_weight=params.alpha_ce,
+                          ce_weight=alpha_mlm, row_mask=mask, ignore_index=-100)
+    else:
+        loss = distil_ce_loss(s_logits, t_logits, mask, params.temperature, params.alpha_ce)
+    if getattr(params, "alpha_cos", 0.0) > 0.0:
+        s_hid = student_outputs["hidden_states"][-1]
+        t_hid = teacher_outputs["hidden_states"][-1]
+        loss = loss + cosine_embedding_loss(s_hid, t_hid, attention_mask, params.alpha_cos)
+    return loss
