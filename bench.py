@@ -193,6 +193,17 @@ def run_kernel_table(dev):
         del teacher, student, st
     ema_mod.release_pool()
 
+    # student clone fused into the EMA launch (16 B per parameter: read s, t; write s', t')
+    teacher = [(torch.randn(s, generator=g) * 0.02).to(dev) for s in vit]
+    student = [(torch.randn(s, generator=g) * 0.02).to(dev) for s in vit]
+    keep = {}
+
+    def fused():
+        keep["c"], keep["t"] = ta.clone_and_update(0.99, student, teacher)
+    out["ema_clone_fused_vit_base"] = entry(16 * sum(numel(s) for s in vit), _time_stream(fused, 30), None, 1)
+    del teacher, student, keep
+    ema_mod.release_pool()
+
     def kd_call(s, t, mask, T, grad):
         rows, V = s.shape[0] * (s.shape[1] if s.dim() == 3 else 1), s.shape[-1]
         code = _lib.dtype_code(s.dtype)

@@ -86,6 +86,17 @@ int64_t ts_ema_plan(const void* const* t, const void* const* s, void* const* out
 int ts_ema_multi(const ts_ema_chunk* table_dev, int64_t n_chunks, int64_t chunk_elems, float m32,
                  float c32, ts_stream_t stream);
 
+/* The same launch, also writing a clone of the student values: for every
+ * chunk, s is copied to (char*)out + clone_offset_bytes.  Fuses the pipeline's
+ * `online_new_param = [t.detach().clone() for t in online_prev_param]`
+ * (tspipe/gpu_task.py:398) into the EMA that follows it (403-406), so the
+ * optimizer-step tail moves 16 B per parameter instead of 8 + 12.  The caller
+ * lays the clone buffer out exactly like the EMA output buffer (same offsets),
+ * which is what makes one offset enough; clone_offset_bytes is a non-zero
+ * multiple of 4 (of 16 for the vector path). */
+int ts_ema_clone_multi(const ts_ema_chunk* table_dev, int64_t n_chunks, int64_t chunk_elems, float m32,
+                       float c32, int64_t clone_offset_bytes, ts_stream_t stream);
+
 /* ------------------------------------------------------------------------ */
 /* Multi-segment copy: micro-batch gather (torch.cat on dim 0,      */
 /* tspipe/batch_ops.py:186-205, tspipe/utils.py:280), the owning form of     */

@@ -204,3 +204,24 @@ def test_clone_and_copy_in_of_a_parameter_list(device):
         ta.copy_params_(live[:2], clones[:1])
     with pytest.raises(ValueError):
         ta.copy_params_([live[0]], [clones[1]])
+
+
+@pytest.mark.parametrize("shapes", [[(64, 3, 7, 7), (64,), (129, 33), (5,)], resnet18_shapes()])
+def test_clone_and_update_fused(device, shapes):
+    from tspipe_amd import ema as ema_mod
+    ema_mod.release_pool()
+    teacher, student = param_lists(shapes, 13)
+    t_dev = [t.to(device) for t in teacher]
+    s_dev = [torch.nn.Parameter(s.to(device)) for s in student]
+    clones, new_t = ta.clone_and_update(0.996, s_dev, t_dev)
+    want = ts_oracle.ema_update(0.996, student, teacher)
+    assert len(clones) == len(new_t) == len(shapes)
+    for c, n, s0, w, sd, td, t0 in zip(clones, new_t, student, want, s_dev, t_dev, teacher):
+        assert bits_equal(c, s0) and bits_equal(n, w)
+        assert c.data_ptr() not in (sd.data_ptr(), n.data_ptr()) and not c.requires_grad
+        assert bits_equal(sd, s0) and bits_equal(td, t0)  # inputs untouched
+    # the same through the unfused pair of calls
+    clones2 = ta.clone_params(s_dev)
+    new_t2 = ta.momentum_update(0.996, clones2, t_dev)
+    assert all(bits_equal(a, b) for a, b in zip(new_t, new_t2))
+    ema_mod.release_pool()

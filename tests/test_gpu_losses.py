@@ -327,3 +327,39 @@ def test_distil_loss_fn_plugin(device, restrict):
     for got, ref in ((sd.grad, gs), (shd.grad, gh)):
         peak = ref.abs().max().item()
         assert ((got.cpu().double() - ref).abs() <= 1e-3 * peak + ref.abs() * 2.0 ** -8).all()
+
+
+def test_kd_masked_cfg3_full_size_properties(device):
+    # [32, 128, 30522] bf16, 15 % token mask, gathered from 4 micro-batches: too large for the
+    # fp64 oracle, so checked through properties that do not depend on the size
+    g = seeded(2)
+    pieces_s = [(torch.randn(8, 128, 30522, generator=g) * 2).to(torch.bfloat16).to(device) for _ in range(4)]
+    pieces_t = [(torch.randn(8, 128, 30522, generator=g) * 2).to(torch.bfloat16).to(device) for _ in range(4)]
+    mask = (torch.rand(32, 128, generator=g) < 0.15).to(device)
+    s = ta.gather([ta.Batch(p) for p in pieces_s]).requires_grad_()
+    t = ta.gather([ta.Batch(p) for p in pieces_t])
+    loss = ta.distil_ce_loss(s, t, mask, 2.0)
+    loss.backward()
+    n_sel = int(mask.sum())
+    assert 400 < n_sel < 900
+    # (1) same rows through the unmasked narrow-free path: compact them with torch indexing first
+    s_sel = s.detach()[mask].clone().requires_grad_()
+    t_sel = t[mask].clone()
+    loss2 = ta.kd_soft_target_loss(s_sel, t_sel, 2.0)
+    loss2.backward()
+    assert rel_err(loss.item(), loss2.item()) < 1e-5
+    # same arithmetic up to summation order (the compacted rows are aligned differently): one bf16 ulp
+    assert torch.allclose(s.grad[mask].float(), s_sel.grad.float(), rtol=2.0 ** -7, atol=1e-12)
+    # (2) nothing outside the mask, (3) gradient rows sum to ~0, (4) loss > 0
+    assert (s.grad[~mask] == 0).all()
+    sums = s.grad[mask].float().sum(dim=1).abs().max().item()
+    assert sums < 5e-3 * s.grad[mask].float().abs().sum(dim=1).max().item()
+    assert loss.item() > 0
+    # (5) a 64-row sample against the fp64 oracle
+    rows = mask.reshape(-1).nonzero().squeeze(1)[:64].cpu()
+    ss = s.detach().reshape(-1, 30522)[rows.to(device)].cpu().double().requires_grad_()
+    tt = t.reshape(-1, 30522)[rows.to(device)].cpu().double()
+    (ts_oracle.kd_soft_target(ss, tt, 2.0) * 64 / n_sel).backward()
+    got = s.grad.reshape(-1, 30522)[rows.to(device)].cpu().double()
+    peak = ss.grad.abs().max().item()
+    assert ((got - ss.grad).abs() <= 1e-3 * peak + ss.grad.abs() * 2.0 ** -8).all()

@@ -6,7 +6,7 @@ library is loaded on the first kernel call (see ``_lib``).
 from .batch_ops import (Batch, ScatterGatherFn, batch_size, check, defaultScatterGatherFn, gather,
                         generic_gather, generic_scatter, scatter, scatter_copy)
 from .batchnorm import DeferredBatchNorm
-from .ema import (calculate_target_network_parameters, calculate_updated_momentum_encoder, clone_params,
+from .ema import (calculate_target_network_parameters, calculate_updated_momentum_encoder, clone_and_update, clone_params,
                   copy_params_, momentum_update, update_target_network_parameters_)
 from .losses import (SoftTarget, byol_contrastive_loss, byol_loss, cosine_embedding_loss, distil_ce_loss,
                      distil_loss_fn, infonce_loss, kd_ce_loss, kd_soft_target_loss, moco_contrastive_loss,

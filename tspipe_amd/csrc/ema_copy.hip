@@ -25,8 +25,13 @@ __device__ __forceinline__ float ema1(float t, float s, float m, float c) {
   return a + b;
 }
 
+// CLONE: the student values are also written to `out + clone_offset`, which
+// fuses the pipeline's clone of the student parameters into the same pass
+// (16 B per parameter instead of 8 + 12 for a separate copy).
+template <bool CLONE>
 __global__ __launch_bounds__(kEmaBlock) void ema_multi_kernel(const ts_ema_chunk* __restrict__ table,
-                                                              uint32_t subs, float m, float c) {
+                                                              uint32_t subs, float m, float c,
+                                                              int64_t clone_offset) {
   // Uniform per workgroup: the compiler turns these into scalar loads.
   const uint32_t chunk = blockIdx.x / subs, sub = blockIdx.x % subs;
   const ts_ema_chunk ch = table[chunk];
@@ -36,9 +41,11 @@ __global__ __launch_bounds__(kEmaBlock) void ema_multi_kernel(const ts_ema_chunk
   const float* __restrict__ tp = ch.t + begin;
   const float* __restrict__ sp = ch.s + begin;
   float* __restrict__ op = ch.out + begin;
+  float* __restrict__ cp = reinterpret_cast<float*>(reinterpret_cast<char*>(op) + clone_offset);
   const uint32_t tid = threadIdx.x;
 
-  if (ch.flags & 1u) {
+  // the vector path also needs the clone destination on a 16-byte boundary
+  if ((ch.flags & 1u) && (!CLONE || (clone_offset & 15) == 0)) {
     const uint32_t n4 = n >> 2;
     if (tid < n4) {
       const f32x4 a = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(tp) + tid);
@@ -49,11 +56,14 @@ __global__ __launch_bounds__(kEmaBlock) void ema_multi_kernel(const ts_ema_chunk
       r.z = ema1(a.z, b.z, m, c);
       r.w = ema1(a.w, b.w, m, c);
       __builtin_nontemporal_store(r, reinterpret_cast<f32x4*>(op) + tid);
+      if (CLONE) __builtin_nontemporal_store(b, reinterpret_cast<f32x4*>(cp) + tid);
     }
     const uint32_t rem = n & 3u;
     if (tid < rem) {
       const uint32_t i = (n4 << 2) + tid;
-      op[i] = ema1(tp[i], sp[i], m, c);
+      const float sv = sp[i];
+      op[i] = ema1(tp[i], sv, m, c);
+      if (CLONE) cp[i] = sv;
     }
   } else {
     // Views whose storage offset breaks 16-byte alignment: 4-byte accesses,
@@ -61,7 +71,11 @@ __global__ __launch_bounds__(kEmaBlock) void ema_multi_kernel(const ts_ema_chunk
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const uint32_t i = u * kEmaBlock + tid;
-      if (i < n) op[i] = ema1(tp[i], sp[i], m, c);
+      if (i < n) {
+        const float sv = sp[i];
+        op[i] = ema1(tp[i], sv, m, c);
+        if (CLONE) cp[i] = sv;
+      }
     }
   }
 }
@@ -116,8 +130,22 @@ int ts_ema_multi(const ts_ema_chunk* table_dev, int64_t n_chunks, int64_t chunk_
   if (!table_dev) return TS_ERR_ARG;
   const int64_t subs = chunk_elems / ts::kSubElems;
   if (subs > 0x7fffffffLL || n_chunks * subs > 0x7fffffffLL) return TS_ERR_RANGE;
-  hipLaunchKernelGGL(ts::ema_multi_kernel, dim3((unsigned)(n_chunks * subs)), dim3(ts::kEmaBlock), 0,
-                     (hipStream_t)stream, table_dev, (uint32_t)subs, m32, c32);
+  hipLaunchKernelGGL(ts::ema_multi_kernel<false>, dim3((unsigned)(n_chunks * subs)), dim3(ts::kEmaBlock), 0,
+                     (hipStream_t)stream, table_dev, (uint32_t)subs, m32, c32, (int64_t)0);
+  return ts::check_launch();
+}
+
+int ts_ema_clone_multi(const ts_ema_chunk* table_dev, int64_t n_chunks, int64_t chunk_elems, float m32,
+                       float c32, int64_t clone_offset_bytes, ts_stream_t stream) {
+  if (n_chunks < 0 || chunk_elems <= 0 || chunk_elems % ts::kSubElems != 0) return TS_ERR_ARG;
+  if (clone_offset_bytes == 0) return TS_ERR_ARG;  // the clone cannot alias the EMA output
+  if (clone_offset_bytes & 3) return TS_ERR_ALIGN;
+  if (n_chunks == 0) return TS_OK;
+  if (!table_dev) return TS_ERR_ARG;
+  const int64_t subs = chunk_elems / ts::kSubElems;
+  if (subs > 0x7fffffffLL || n_chunks * subs > 0x7fffffffLL) return TS_ERR_RANGE;
+  hipLaunchKernelGGL(ts::ema_multi_kernel<true>, dim3((unsigned)(n_chunks * subs)), dim3(ts::kEmaBlock), 0,
+                     (hipStream_t)stream, table_dev, (uint32_t)subs, m32, c32, clone_offset_bytes);
   return ts::check_launch();
 }
 

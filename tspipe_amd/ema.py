@@ -256,6 +256,29 @@ def update_target_network_parameters_(online_params: Iterable[torch.Tensor],
             live.detach().copy_(work)
 
 
+@torch.no_grad()
+def clone_and_update(m: float, online_param: Iterable[torch.Tensor], target_param: Iterable[torch.Tensor]):
+    """Fuses the pipeline's student clone with the EMA that follows it
+    (tspipe/gpu_task.py:398 and 403-406): returns
+    ``([p.detach().clone() for p in online_param], [t*m + p*(1-m) ...])`` from one
+    kernel launch that reads every student and teacher value once."""
+    students, teachers, shapes = _prepare(online_param, target_param, skip_none=False)
+    if not teachers:
+        return [], []
+    ema_arena = _acquire_arena(teachers, shapes)
+    views = list(ema_arena.views)  # held, so the second acquire cannot hand the same arena out
+    clone_arena = _acquire_arena(teachers, shapes)
+    offset = clone_arena.flat.data_ptr() - ema_arena.flat.data_ptr()
+    device = teachers[0].device
+    with torch.cuda.device(device):
+        table = _tables.stage_ema(_ptrs(teachers), _ptrs(students), ema_arena.ptrs, ema_arena.numels, device)
+        status = _lib.lib().ts_ema_clone_multi(table.dev_ptr, table.n_chunks, table.chunk, float(m), 1.0 - float(m),
+                                              offset, _lib.current_stream_ptr(device))
+        _lib.check(status, "ts_ema_clone_multi")
+        table.done()
+    return list(clone_arena.views), views
+
+
 # ---------------------------------------------------------------------------
 # The EMA's neighbours in the optimizer step: whole-list clone and copy-in
 # ---------------------------------------------------------------------------
