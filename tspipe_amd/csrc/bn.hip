@@ -38,50 +38,75 @@ __device__ __forceinline__ PlaneSplit split_plane(const float* p, int64_t HW) {
 
 // Accumulates (a, b) over the slab's elements of x (and optionally a second
 // tensor y with the same layout) through a functor: f(xv, yv, a, b).
+// Planes are taken two at a time so that the loads of both are in flight
+// before either is consumed (a plane of a small feature map is only a few
+// vectors per thread).
 template <bool TWO, typename F>
 __device__ __forceinline__ void slab_reduce(const float* __restrict__ x, const float* __restrict__ y,
                                             int64_t n0, int64_t n1, int64_t C, int64_t c, int64_t HW,
                                             float& a, float& b, F f) {
+  constexpr int PL = 2;
   const int tid = threadIdx.x;
-  for (int64_t n = n0; n < n1; ++n) {
-    const int64_t off = (n * C + c) * HW;
-    const float* px = x + off;
-    const float* py = TWO ? y + off : nullptr;
-    const PlaneSplit sp = split_plane(px, HW);
-    const bool yvec = !TWO || ((((uintptr_t)py) & 15u) == (((uintptr_t)px) & 15u));
-    if (tid < sp.head) f(px[tid], TWO ? py[tid] : 0.f, a, b);
-    const f32x4* px4 = reinterpret_cast<const f32x4*>(px + sp.head);
-    const f32x4* py4 = reinterpret_cast<const f32x4*>(py + sp.head);
-    for (int64_t base = 0; base < sp.nvec; base += kBnBlock * kBnUnroll) {
-      f32x4 vx[kBnUnroll], vy[kBnUnroll];
+  for (int64_t n = n0; n < n1; n += PL) {
+    const float* px[PL];
+    const float* py[PL];
+    PlaneSplit sp[PL];
+    bool yvec[PL], live[PL];
+    int64_t maxvec = 0;
 #pragma unroll
-      for (int u = 0; u < kBnUnroll; ++u) {
-        const int64_t i = base + u * kBnBlock + tid;
-        if (i < sp.nvec) {
-          vx[u] = px4[i];
-          if (TWO) {
-            if (yvec) {
-              vy[u] = py4[i];
-            } else {
-              const float* q = py + sp.head + (i << 2);
-              vy[u] = f32x4{q[0], q[1], q[2], q[3]};
+    for (int p = 0; p < PL; ++p) {
+      live[p] = n + p < n1;
+      const int64_t off = ((live[p] ? n + p : n) * C + c) * HW;
+      px[p] = x + off;
+      py[p] = TWO ? y + off : nullptr;
+      sp[p] = split_plane(px[p], HW);
+      yvec[p] = !TWO || ((((uintptr_t)py[p]) & 15u) == (((uintptr_t)px[p]) & 15u));
+      if (live[p] && sp[p].nvec > maxvec) maxvec = sp[p].nvec;
+    }
+#pragma unroll
+    for (int p = 0; p < PL; ++p) {
+      if (live[p]) {
+        if (tid < sp[p].head) f(px[p][tid], TWO ? py[p][tid] : 0.f, a, b);
+        const int64_t it = sp[p].tail0 + tid;
+        if (it < HW) f(px[p][it], TWO ? py[p][it] : 0.f, a, b);
+      }
+    }
+    for (int64_t base = 0; base < maxvec; base += kBnBlock * kBnUnroll) {
+      f32x4 vx[PL][kBnUnroll], vy[PL][kBnUnroll];
+#pragma unroll
+      for (int p = 0; p < PL; ++p) {
+        const f32x4* px4 = reinterpret_cast<const f32x4*>(px[p] + sp[p].head);
+        const f32x4* py4 = reinterpret_cast<const f32x4*>(py[p] + sp[p].head);
+#pragma unroll
+        for (int u = 0; u < kBnUnroll; ++u) {
+          const int64_t i = base + u * kBnBlock + tid;
+          if (live[p] && i < sp[p].nvec) {
+            vx[p][u] = px4[i];
+            if (TWO) {
+              if (yvec[p]) {
+                vy[p][u] = py4[i];
+              } else {
+                const float* q = py[p] + sp[p].head + (i << 2);
+                vy[p][u] = f32x4{q[0], q[1], q[2], q[3]};
+              }
             }
           }
         }
       }
 #pragma unroll
-      for (int u = 0; u < kBnUnroll; ++u) {
-        const int64_t i = base + u * kBnBlock + tid;
-        if (i < sp.nvec) {
-          f(vx[u].x, TWO ? vy[u].x : 0.f, a, b);
-          f(vx[u].y, TWO ? vy[u].y : 0.f, a, b);
-          f(vx[u].z, TWO ? vy[u].z : 0.f, a, b);
-          f(vx[u].w, TWO ? vy[u].w : 0.f, a, b);
+      for (int p = 0; p < PL; ++p) {
+#pragma unroll
+        for (int u = 0; u < kBnUnroll; ++u) {
+          const int64_t i = base + u * kBnBlock + tid;
+          if (live[p] && i < sp[p].nvec) {
+            f(vx[p][u].x, TWO ? vy[p][u].x : 0.f, a, b);
+            f(vx[p][u].y, TWO ? vy[p][u].y : 0.f, a, b);
+            f(vx[p][u].z, TWO ? vy[p][u].z : 0.f, a, b);
+            f(vx[p][u].w, TWO ? vy[p][u].w : 0.f, a, b);
+          }
         }
       }
     }
-    const int64_t it = sp.tail0 + tid;
-    if (it < HW) f(px[it], TWO ? py[it] : 0.f, a, b);
   }
 }
 
@@ -315,6 +340,7 @@ __global__ __launch_bounds__(kBnBlock) void bn_bwd_dx_kernel(const float* __rest
 // not degenerate into one workgroup per few hundred bytes.
 inline int64_t bn_slab(int64_t N, int64_t HW) {
   int64_t s = (8192 + HW - 1) / HW;
+  s += s & 1;  // planes are consumed in pairs
   if (s < 1) s = 1;
   if (s > N) s = N;
   return s;
