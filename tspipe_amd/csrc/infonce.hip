@@ -233,7 +233,9 @@ __global__ __launch_bounds__(kNceBlock) void nce_main_kernel(const uint16_t* __r
 #pragma unroll
     for (int i = 0; i < 16; ++i) oacc[fb][i] = 0.f;
   float lsum = 0.f;  // sum_j P_ij
-  float asum = 0.f;  // sum_j P_ij x_ij (x: logit in the log2 domain) = <qh_i, sum_j P_ij kh_j> * log2e/tau
+  float asum = 0.f;  // sum_j P_ij (x_ij - x_max), x: logit in the log2 domain; x_max * l is added at the end
+  // tiles from this one on contain padded keys (never reached when n is a multiple of the tile)
+  const int64_t t_pad = n / kKTile;
 
   // global -> register staging of one key tile (K rows, K^T rows, rk)
   constexpr int KCH = kKTile * C / 8 / kNceBlock;  // 16-byte chunks per thread, K tile
@@ -330,9 +332,27 @@ __global__ __launch_bounds__(kNceBlock) void nce_main_kernel(const uint16_t* __r
     __builtin_amdgcn_sched_barrier(0);
 
     // P = 2^(S * rq_i * rk_j * log2e/tau - x_max); keys this lane holds:
-    // key(i) = (i%4) + 4h + 8(i/4).  Padded keys have rk = 0 and are masked.
-    const int64_t key0 = t * kKTile;
-    const bool ragged = key0 + kKTile > n;  // only the last tile can hold padded keys
+    // key(i) = (i%4) + 4h + 8(i/4).  With u = x - x_max the kernel sums
+    // l = sum P and a' = sum P u; sum P x follows as a' + x_max l at the end.
+    float pv[16], uv[16];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const f32x4 rk4 = (g == 0) ? rk0 : (g == 1) ? rk1 : (g == 2) ? rk2 : rk3;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int i = 4 * g + j;
+        uv[i] = fmaf(sacc[i], sc_i * rk4[j], -scale2);
+        pv[i] = fast_exp2(uv[i]);
+      }
+    }
+    if (t >= t_pad) {
+      // padded keys, only at the very end of the key range (their rk is 0,
+      // which zeroes the second product, but not the row sums)
+      const int keyb = (int)(t * kKTile) + 4 * h;
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+        if (keyb + 8 * (i / 4) + (i % 4) >= (int)n) pv[i] = 0.f;
+    }
     bf16x8 pb[2];
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
@@ -340,13 +360,9 @@ __global__ __launch_bounds__(kNceBlock) void nce_main_kernel(const uint16_t* __r
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int i = 4 * g + j;
-        const float rkj = rk4[j];
-        const float x = sacc[i] * (sc_i * rkj);
-        float p = fast_exp2(x - scale2);
-        if (ragged && key0 + 8 * g + 4 * h + j >= n) p = 0.f;
-        lsum += p;
-        asum += p * x;
-        pb[g / 2][(g % 2) * 4 + j] = (__bf16)(p * rkj);
+        lsum += pv[i];
+        asum = fmaf(pv[i], uv[i], asum);
+        pb[g / 2][(g % 2) * 4 + j] = (__bf16)(pv[i] * rk4[j]);
       }
     }
 
@@ -363,7 +379,8 @@ __global__ __launch_bounds__(kNceBlock) void nce_main_kernel(const uint16_t* __r
 
   // partial results, register-native order: [split][q tile of 32][fb][i][lane]
   const float ltot = lsum + __shfl_xor(lsum, 32, kWave);
-  const float atot = asum + __shfl_xor(asum, 32, kWave);
+  // sum_j P_ij x_ij = <qh_i, sum_j P_ij kh_j> * log2e/tau
+  const float atot = asum + __shfl_xor(asum, 32, kWave) + scale2 * ltot;
   if (h == 0) {
     lpart[(int64_t)split * npad + qtile * kQTile + w * 32 + col] = ltot;
     apart[(int64_t)split * npad + qtile * kQTile + w * 32 + col] = atot;
