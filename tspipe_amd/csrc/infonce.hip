@@ -17,14 +17,25 @@
 //     the MFMA and no rounded copy of qh / kh is ever made.
 //
 // Kernels:
-//   prep     per row: rq = 1/max(|q|,eps), rk, the diagonal logit, and K^T
-//            (bf16, [C][Npad]) so that the second contraction can read keys
-//            contiguously; fp32 inputs are also rounded to bf16 copies here.
-//   main     grid (q tile of 128 rows, key split, pair); 4 wavefronts, each
-//            owning 32 q rows; per 32-key tile: S^T = K Q^T (MFMA 32x32x16),
-//            P = 2^(S*scale - x_max), l += P, O^T += K^T (P*rk) (MFMA).
-//            Writes per-split partial l and O^T in register-native order.
+//   prep     per row: rq = 1/max(|q|,eps), rk, the diagonal logit; the keys,
+//            normalised and rounded to bf16, are written as "tile images":
+//            for every 32 keys the exact bytes, in the exact order, that the
+//            main kernel's MFMA operand reads want to find in LDS (below).
+//            fp32 queries are also rounded to a bf16 copy here.
+//   main     grid (key split, q tile of 128 rows); 4 wavefronts, each owning
+//            32 q rows; per 32-key tile: S^T = Kh Q^T (MFMA 32x32x16),
+//            P = 2^(S*scale - x_max), l += P, O^T += Kh^T P (MFMA).  Tile
+//            images go from global memory straight into LDS (no registers),
+//            two tiles ahead.  Writes per-split partial l and O^T in
+//            register-native order.
 //   combine  per 32-row q tile: adds the splits, forms loss rows and dq.
+//
+// Tile image (C features, KK = C/16, FB = C/32; 1 KB fragments, lane L =
+// 32h + col reads bytes 16L..16L+15 of a fragment as one MFMA A operand):
+//   fragment kk < KK        : Kh[key = col][16kk + 8h .. +7]       (first product)
+//   fragment KK + tt*FB + fb: Kh[16tt + 8gg + 4h + j][32fb + col],  (second product)
+//                             gg = 0,1, j = 0..3 -> element 4gg + j
+// so every operand read is a linear, conflict-free 1 KB of LDS.
 //
 // MFMA 32x32x16 operand layout used throughout (lane l, half h = l/32):
 //   A: row l%32, contraction slots 8h..8h+7;  B: column l%32, same slots;
@@ -55,7 +66,22 @@ struct NceLayout {
   int64_t npad;
   int splits;
   size_t head_bytes;
-  size_t off_rq, off_rk, off_diag, off_lpart, off_apart, off_kt, off_qb, off_kb, off_opart, pair_bytes;
+  size_t off_rq, off_rk, off_diag, off_lpart, off_apart, off_kimg, off_qb, off_opart, pair_bytes;
+};
+
+// One (q, k) pair's pointers; the kernels pick theirs by blockIdx.z, so the two
+// pairs of the symmetric loss share every launch.
+struct NcePair {
+  const void* q;
+  const void* k;
+  void* dq;
+  const uint16_t* qsrc;  // bf16 queries the MFMA reads: q itself or the rounded copy
+  float *rq, *rk, *diag, *lpart, *apart, *opart, *row_loss;
+  uint8_t* kimg;
+  uint16_t* qb;
+};
+struct NceArgs {
+  NcePair p[2];
 };
 
 inline size_t nce_align(size_t x) { return (x + 255) & ~(size_t)255; }
@@ -81,34 +107,46 @@ inline NceLayout nce_layout(int64_t n, int64_t c, int n_pairs, bool fp32_in) {
   L.off_diag = o;     o += nce_align(L.npad * 4);
   L.off_lpart = o;    o += nce_align((size_t)L.splits * L.npad * 4);
   L.off_apart = o;    o += nce_align((size_t)L.splits * L.npad * 4);
-  L.off_kt = o;       o += nce_align((size_t)c * L.npad * 2);
+  L.off_kimg = o;     o += nce_align((size_t)L.npad * c * 4);  // npad/32 tile images of 128 c bytes
   L.off_qb = o;       o += fp32_in ? nce_align((size_t)L.npad * c * 2) : 0;
-  L.off_kb = o;       o += fp32_in ? nce_align((size_t)L.npad * c * 2) : 0;
   L.off_opart = o;    o += nce_align((size_t)L.splits * L.npad * c * 4);
   L.pair_bytes = o;
   return L;
 }
 
 // ---------------------------------------------------------------------------
-// prep: 16-byte row loads, a group of C/VEC lanes per row; the K rows of the
-// workgroup pass through LDS to come out transposed
+// prep: 16-byte row loads, a group of C/VEC lanes per row; one workgroup per
+// 32 rows, whose normalised keys pass through LDS to come out as a tile image
 // ---------------------------------------------------------------------------
-template <typename T, int C>
-struct NcePrep {
-  static constexpr int VEC = 16 / sizeof(T);               // elements per 16-byte load
-  static constexpr int LPR = C / VEC;                      // lanes per row (8 .. 64)
-  static constexpr int RPP = kWave / LPR;                  // rows per wavefront pass
-  static constexpr int ROWS = (4 * RPP > 16) ? 4 * RPP : 16;  // rows per workgroup
-  static constexpr int LD = C + 8;                         // bf16 per LDS row (16-byte aligned rows)
+template <int C>
+struct NceTile {
+  static constexpr int KK = C / 16;             // contraction steps of S^T = fragments of the first product
+  static constexpr int FB = C / 32;             // feature blocks of O^T
+  static constexpr int FRAGS = KK + 2 * FB;     // 1 KB fragments per image
+  static constexpr int BYTES = FRAGS * 1024;    // 32 KB at C = 256
 };
 
 template <typename T, int C>
-__global__ __launch_bounds__(kNceBlock) void nce_prep_kernel(const T* __restrict__ q, const T* __restrict__ k,
-                                                             int64_t n, int64_t npad, float scale2,
-                                                             float* __restrict__ rq, float* __restrict__ rk,
-                                                             float* __restrict__ diag, uint16_t* __restrict__ kt,
-                                                             uint16_t* __restrict__ qb, uint16_t* __restrict__ kb) {
+struct NcePrep {
+  static constexpr int VEC = 16 / sizeof(T);  // elements per 16-byte load
+  static constexpr int LPR = C / VEC;         // lanes per row (8 .. 64)
+  static constexpr int RPP = kWave / LPR;     // rows per wavefront pass
+  static constexpr int ROWS = kKTile;         // rows per workgroup: one key tile
+  static constexpr int LD = C + 8;            // bf16 per LDS row (16-byte aligned rows)
+};
+
+template <typename T, int C>
+__global__ __launch_bounds__(kNceBlock) void nce_prep_kernel(NceArgs args, int64_t n, int64_t npad, float scale2) {
+  const NcePair& pr = args.p[blockIdx.z];
+  const T* __restrict__ q = (const T*)pr.q;
+  const T* __restrict__ k = (const T*)pr.k;
+  float* __restrict__ rq = pr.rq;
+  float* __restrict__ rk = pr.rk;
+  float* __restrict__ diag = pr.diag;
+  uint8_t* __restrict__ kimg = pr.kimg;
+  uint16_t* __restrict__ qb = pr.qb;
   using P = NcePrep<T, C>;
+  using TI = NceTile<C>;
   __shared__ __attribute__((aligned(16))) uint16_t tile[P::ROWS * P::LD];
   const int lane = threadIdx.x % kWave, w = threadIdx.x / kWave;
   const int sub = lane / P::LPR, li = lane % P::LPR;  // row within the pass, lane within the row
@@ -133,88 +171,112 @@ __global__ __launch_bounds__(kNceBlock) void nce_prep_kernel(const T* __restrict
 #pragma unroll
       for (int e = 0; e < P::VEC; ++e) qv[e] = kv[e] = 0.f;
     }
-    float sqq = 0.f, skk = 0.f, sqk = 0.f;
-    uint16_t qbits[P::VEC], kbits[P::VEC];
+    float sqq = 0.f, skk = 0.f;
 #pragma unroll
     for (int e = 0; e < P::VEC; ++e) {
-      qbits[e] = f32_to_bf16_bits(qv[e]);
-      kbits[e] = f32_to_bf16_bits(kv[e]);
       sqq += qv[e] * qv[e];
       skk += kv[e] * kv[e];
-      // the diagonal logit uses the values the MFMA will see
-      sqk += bf16_bits_to_f32(qbits[e]) * bf16_bits_to_f32(kbits[e]);
-    }
-#pragma unroll
-    for (int e = 0; e < P::VEC; ++e) tile[r * P::LD + li * P::VEC + e] = kbits[e];
-    if (qb) {
-#pragma unroll
-      for (int e = 0; e < P::VEC; ++e) {
-        qb[row * C + li * P::VEC + e] = qbits[e];
-        kb[row * C + li * P::VEC + e] = kbits[e];
-      }
     }
 #pragma unroll
     for (int off = P::LPR / 2; off > 0; off >>= 1) {
       sqq += __shfl_xor(sqq, off, kWave);
       skk += __shfl_xor(skk, off, kWave);
-      sqk += __shfl_xor(sqk, off, kWave);
     }
+    const float a = live ? 1.f / fmaxf(sqrtf(sqq), kNormEps) : 0.f;
+    const float b = live ? 1.f / fmaxf(sqrtf(skk), kNormEps) : 0.f;
+    // the diagonal logit uses the values the MFMA will see: q rounded to
+    // bf16, k normalised and then rounded
+    float sqk = 0.f;
+    uint16_t qbits[P::VEC];
+#pragma unroll
+    for (int e = 0; e < P::VEC; ++e) {
+      qbits[e] = f32_to_bf16_bits(qv[e]);
+      const uint16_t kbits = f32_to_bf16_bits(kv[e] * b);
+      tile[r * P::LD + li * P::VEC + e] = kbits;
+      sqk += bf16_bits_to_f32(qbits[e]) * bf16_bits_to_f32(kbits);
+    }
+    if (qb) {
+#pragma unroll
+      for (int e = 0; e < P::VEC; ++e) qb[row * C + li * P::VEC + e] = qbits[e];
+    }
+#pragma unroll
+    for (int off = P::LPR / 2; off > 0; off >>= 1) sqk += __shfl_xor(sqk, off, kWave);
     if (li == 0) {
-      const float a = live ? 1.f / fmaxf(sqrtf(sqq), kNormEps) : 0.f;
-      const float b = live ? 1.f / fmaxf(sqrtf(skk), kNormEps) : 0.f;
       rq[row] = a;
       rk[row] = b;
-      diag[row] = sqk * a * b * scale2;
+      diag[row] = sqk * a * scale2;
     }
   }
   __syncthreads();
-  // transposed write: K^T[f][row0 + 8*chunk .. +7], 16 bytes per store
-  for (int id = threadIdx.x; id < C * (P::ROWS / 8); id += kNceBlock) {
-    const int f = id / (P::ROWS / 8), chunk = id % (P::ROWS / 8);
+  // the tile image, 16 bytes per store, consecutive threads -> consecutive chunks
+  uint8_t* img = kimg + (int64_t)blockIdx.x * TI::BYTES;
+  for (int id = threadIdx.x; id < TI::FRAGS * kWave; id += kNceBlock) {
+    const int fr = id / kWave, L = id % kWave;
+    const int col = L % 32, h = L / 32;
     u16x8 v;
+    if (fr < TI::KK) {
+      v = *reinterpret_cast<const u16x8*>(&tile[col * P::LD + fr * 16 + h * 8]);
+    } else {
+      const int tt = (fr - TI::KK) / TI::FB, fb = (fr - TI::KK) % TI::FB;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) v[e] = tile[(chunk * 8 + e) * P::LD + f];
-    *reinterpret_cast<u16x8*>(kt + (int64_t)f * npad + row0 + chunk * 8) = v;
+      for (int e = 0; e < 8; ++e) v[e] = tile[(16 * tt + 8 * (e / 4) + 4 * h + (e % 4)) * P::LD + fb * 32 + col];
+    }
+    *reinterpret_cast<u16x8*>(img + (int64_t)id * 16) = v;
   }
 }
 
 // ---------------------------------------------------------------------------
 // main
 // ---------------------------------------------------------------------------
-template <int C>
-struct NceSmem {
-  static constexpr int KLD = C + 8;       // bf16 per K-tile row (16-byte pad: rows start on different banks)
-  static constexpr int TLD = kKTile + 4;  // bf16 per K^T-tile row: 72 bytes, so 16 consecutive rows start on
-                                          // 16 different bank pairs and the 8-byte operand reads do not collide
-  uint16_t k[2][kKTile * KLD];
-  uint16_t kt[2][C * TLD];
-  float rk[2][kKTile];
-};
+typedef __attribute__((address_space(3))) void nce_lds_void;
+typedef __attribute__((address_space(1))) const void nce_glb_void;
+constexpr int kNceBufs = 3;  // tile images in LDS: the one in use and two on their way
 
 template <int C>
-__global__ __launch_bounds__(kNceBlock) void nce_main_kernel(const uint16_t* __restrict__ qg,
-                                                             const uint16_t* __restrict__ kg,
-                                                             const uint16_t* __restrict__ ktg,
-                                                             const float* __restrict__ rq,
-                                                             const float* __restrict__ rk, int64_t n, int64_t npad,
-                                                             int splits, float scale2 /* log2(e)/tau */,
-                                                             float* __restrict__ lpart, float* __restrict__ apart,
-                                                             float* __restrict__ opart) {
-  using Smem = NceSmem<C>;
-  __shared__ __attribute__((aligned(16))) Smem sm;
-  constexpr int KK = C / 16;  // contraction steps of S^T
-  constexpr int FB = C / 32;  // feature blocks of O^T
+__global__ __launch_bounds__(kNceBlock) void nce_main_kernel(NceArgs args, int64_t n, int64_t npad, int splits,
+                                                             float scale2 /* log2(e)/tau */) {
+  const NcePair& pr = args.p[blockIdx.z];
+  const uint16_t* __restrict__ qg = pr.qsrc;
+  const uint8_t* __restrict__ kimg = pr.kimg;
+  const float* __restrict__ rq = pr.rq;
+  float* __restrict__ lpart = pr.lpart;
+  float* __restrict__ apart = pr.apart;
+  float* __restrict__ opart = pr.opart;
+  using TI = NceTile<C>;
+  constexpr int KK = TI::KK, FB = TI::FB;
+  __shared__ __attribute__((aligned(16))) uint8_t sm[kNceBufs][TI::BYTES];
   const int tid = threadIdx.x, lane = tid % kWave, w = tid / kWave;
   const int col = lane % 32, h = lane / 32;
   // Workgroup ids are dealt round-robin to the 8 XCDs.  With the key split as
   // the fastest index (and 8 splits), every XCD keeps seeing the same eighth
-  // of K and K^T, which then stays in that XCD's own L2.
+  // of the key images, which then stays in that XCD's own L2.
   const int split = blockIdx.x;
   const int64_t qtile = blockIdx.y;
   const int64_t qrow = qtile * kQTile + w * 32 + col;  // the q row this lane is a column of
 
   const int64_t ktiles = npad / kKTile;
   const int64_t t0 = ktiles * split / splits, t1 = ktiles * (split + 1) / splits;
+
+  // Global -> LDS without passing through registers: every wavefront moves a
+  // quarter of the image, 1 KB (16 bytes per lane) per instruction, and the
+  // hardware writes lane L's bytes at (LDS base) + 16 L, which is exactly
+  // the image's own order.  Completion is the issuing wavefront's vector
+  // memory counter; the barrier after it makes all four quarters visible.
+  constexpr int FPW = TI::FRAGS / 4;  // fragments per wavefront
+  auto fetch_tile = [&](int64_t t, int buf) {
+    const uint8_t* src = kimg + t * TI::BYTES + (w * FPW) * 1024 + lane * 16;
+#pragma unroll
+    for (int u = 0; u < FPW; ++u)
+      __builtin_amdgcn_global_load_lds((nce_glb_void*)(src + u * 1024),
+                                       (nce_lds_void*)(&sm[buf][(w * FPW + u) * 1024]), 16, 0, 0);
+  };
+  auto wait_fetches_and_sync = [&]() {
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wavefront's fetches have landed
+    __syncthreads();
+  };
+
+  if (t0 < t1) fetch_tile(t0, 0);
+  if (t0 + 1 < t1) fetch_tile(t0 + 1, 1);
 
   // Q fragments: B operand of S^T, resident for the whole kernel.
   bf16x8 qf[KK];
@@ -237,117 +299,63 @@ __global__ __launch_bounds__(kNceBlock) void nce_main_kernel(const uint16_t* __r
   // tiles from this one on contain padded keys (never reached when n is a multiple of the tile)
   const int64_t t_pad = n / kKTile;
 
-  // global -> register staging of one key tile (K rows, K^T rows, rk)
-  constexpr int KCH = kKTile * C / 8 / kNceBlock;  // 16-byte chunks per thread, K tile
-  constexpr int TCH = C * kKTile / 8 / kNceBlock;  // same, K^T tile
-  u32x4 stage_k[KCH], stage_t[TCH];
-  float stage_rk = 0.f;
-  auto load_tile = [&](int64_t t) {
-    const int64_t key0 = t * kKTile;
-#pragma unroll
-    for (int u = 0; u < KCH; ++u) {
-      const int id = tid + u * kNceBlock;
-      const int r = id / (C / 8), c8 = id % (C / 8);
-      u32x4 v = {0u, 0u, 0u, 0u};
-      if (key0 + r < n) v = *reinterpret_cast<const u32x4*>(kg + (key0 + r) * C + c8 * 8);
-      stage_k[u] = v;
-    }
-#pragma unroll
-    for (int u = 0; u < TCH; ++u) {
-      const int id = tid + u * kNceBlock;
-      const int f = id / (kKTile / 8), c8 = id % (kKTile / 8);
-      stage_t[u] = *reinterpret_cast<const u32x4*>(ktg + (int64_t)f * npad + key0 + c8 * 8);
-    }
-    if (tid < kKTile) stage_rk = rk[key0 + tid];  // zero for padded keys
-  };
-  auto store_tile = [&](int buf) {
-#pragma unroll
-    for (int u = 0; u < KCH; ++u) {
-      const int id = tid + u * kNceBlock;
-      const int r = id / (C / 8), c8 = id % (C / 8);
-      *reinterpret_cast<u32x4*>(&sm.k[buf][r * Smem::KLD + c8 * 8]) = stage_k[u];
-    }
-#pragma unroll
-    for (int u = 0; u < TCH; ++u) {
-      const int id = tid + u * kNceBlock;
-      const int f = id / (kKTile / 8), c8 = id % (kKTile / 8);
-      // rows are only 8-byte aligned: two 8-byte stores
-      uint2 lo = {stage_t[u].x, stage_t[u].y}, hi = {stage_t[u].z, stage_t[u].w};
-      *reinterpret_cast<uint2*>(&sm.kt[buf][f * Smem::TLD + c8 * 8]) = lo;
-      *reinterpret_cast<uint2*>(&sm.kt[buf][f * Smem::TLD + c8 * 8 + 4]) = hi;
-    }
-    if (tid < kKTile) sm.rk[buf][tid] = stage_rk;
-  };
-
-  if (t0 < t1) {
-    load_tile(t0);
-    store_tile(0);
-  }
-  __syncthreads();
-
-  for (int64_t t = t0; t < t1; ++t) {
-    const int buf = (int)((t - t0) & 1);
-    const bool more = t + 1 < t1;
-    if (more) load_tile(t + 1);  // in flight while this tile is computed
-
-    // All operand fragments of a phase are read from LDS into their own
-    // registers before the phase's MFMAs start: with one wavefront per SIMD
-    // nothing else hides the LDS latency, and a read-wait-multiply chain per
-    // MFMA would pay it 48 times per tile.
-    bf16x8 ka[KK];
+  // Operand fragments live in registers one phase ahead of the MFMAs that use
+  // them, so that the LDS reads of one product overlap the MFMAs of the
+  // other: tile t's K^T fragments are read while its first product runs, tile
+  // t+1's K fragments while tile t's second product runs.
+  bf16x8 ka[KK];
+  auto read_ka = [&](int buf) {
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) {
-      const u32x4 raw = *reinterpret_cast<const u32x4*>(&sm.k[buf][col * Smem::KLD + kk * 16 + h * 8]);
+      const u32x4 raw = *reinterpret_cast<const u32x4*>(&sm[buf][kk * 1024 + lane * 16]);
       __builtin_memcpy(&ka[kk], &raw, 16);
     }
-    __builtin_amdgcn_sched_barrier(0);  // keep the reads above from being sunk next to their MFMAs
-    const f32x4 rk0 = *reinterpret_cast<const f32x4*>(&sm.rk[buf][4 * h]);
-    const f32x4 rk1 = *reinterpret_cast<const f32x4*>(&sm.rk[buf][8 + 4 * h]);
-    const f32x4 rk2 = *reinterpret_cast<const f32x4*>(&sm.rk[buf][16 + 4 * h]);
-    const f32x4 rk3 = *reinterpret_cast<const f32x4*>(&sm.rk[buf][24 + 4 * h]);
+  };
+  wait_fetches_and_sync();
+  read_ka(0);
 
-    // S^T[key][q] = sum_f K[key][f] Q[q][f]
-    f32x16 sacc;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) sacc[i] = 0.f;
-#pragma unroll
-    for (int kk = 0; kk < KK; ++kk) sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[kk], qf[kk], sacc, 0, 0, 0);
+  int cur = 0;
+  for (int64_t t = t0; t < t1; ++t) {
+    const int nxt = (cur == kNceBufs - 1) ? 0 : cur + 1;
+    const int nn = (nxt == kNceBufs - 1) ? 0 : nxt + 1;
+    // After this barrier tile t+1 is complete in LDS (its fetches were issued
+    // a whole tile ago) and every wavefront has finished reading tile t-1,
+    // whose buffer the fetch below overwrites.
+    wait_fetches_and_sync();
 
-    // K^T fragments for the second product: issued now, they land while the
-    // soft-max arithmetic below runs.  Contraction slot 8h + 4gg + j of step
-    // tt is key 16tt + 8gg + 4h + j on both operands.
-    bf16x8 ta[FB][2];
+    bf16x8 ta[2 * FB];
 #pragma unroll
-    for (int fb = 0; fb < FB; ++fb) {
-#pragma unroll
-      for (int tt = 0; tt < 2; ++tt) {
-        const uint2* base =
-            reinterpret_cast<const uint2*>(&sm.kt[buf][(fb * 32 + col) * Smem::TLD + 16 * tt + 4 * h]);
-        const uint2 lo = base[0], hi = base[2];
-        const u32x4 raw = {lo.x, lo.y, hi.x, hi.y};
-        __builtin_memcpy(&ta[fb][tt], &raw, 16);
-      }
+    for (int x = 0; x < 2 * FB; ++x) {
+      const u32x4 raw = *reinterpret_cast<const u32x4*>(&sm[cur][(KK + x) * 1024 + lane * 16]);
+      __builtin_memcpy(&ta[x], &raw, 16);
     }
+    if (t + 2 < t1) fetch_tile(t + 2, nn);
+    __builtin_amdgcn_sched_barrier(0);  // the reads above are issued before the MFMAs below
 
+    // S^T[key][q] = sum_f Kh[key][f] Q[q][f], as two independent accumulation
+    // chains: a dependent MFMA waits for its predecessor's result.
+    f32x16 sacc0, sacc1;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) sacc0[i] = sacc1[i] = 0.f;
+#pragma unroll
+    for (int kk = 0; kk < KK; kk += 2) {
+      sacc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[kk], qf[kk], sacc0, 0, 0, 0);
+      sacc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[kk + 1], qf[kk + 1], sacc1, 0, 0, 0);
+    }
     __builtin_amdgcn_sched_barrier(0);
 
-    // P = 2^(S * rq_i * rk_j * log2e/tau - x_max); keys this lane holds:
+    // P = 2^(S * rq_i * log2e/tau - x_max); keys this lane holds:
     // key(i) = (i%4) + 4h + 8(i/4).  With u = x - x_max the kernel sums
     // l = sum P and a' = sum P u; sum P x follows as a' + x_max l at the end.
     float pv[16], uv[16];
 #pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const f32x4 rk4 = (g == 0) ? rk0 : (g == 1) ? rk1 : (g == 2) ? rk2 : rk3;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int i = 4 * g + j;
-        uv[i] = fmaf(sacc[i], sc_i * rk4[j], -scale2);
-        pv[i] = fast_exp2(uv[i]);
-      }
+    for (int i = 0; i < 16; ++i) {
+      uv[i] = fmaf(sacc0[i] + sacc1[i], sc_i, -scale2);
+      pv[i] = fast_exp2(uv[i]);
     }
     if (t >= t_pad) {
-      // padded keys, only at the very end of the key range (their rk is 0,
-      // which zeroes the second product, but not the row sums)
+      // padded keys, only at the very end of the key range (their image rows
+      // are zero, which zeroes the second product, but not the row sums)
       const int keyb = (int)(t * kKTile) + 4 * h;
 #pragma unroll
       for (int i = 0; i < 16; ++i)
@@ -355,26 +363,24 @@ __global__ __launch_bounds__(kNceBlock) void nce_main_kernel(const uint16_t* __r
     }
     bf16x8 pb[2];
 #pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const f32x4 rk4 = (g == 0) ? rk0 : (g == 1) ? rk1 : (g == 2) ? rk2 : rk3;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int i = 4 * g + j;
-        lsum += pv[i];
-        asum = fmaf(pv[i], uv[i], asum);
-        pb[g / 2][(g % 2) * 4 + j] = (__bf16)(pv[i] * rk4[j]);
-      }
+    for (int i = 0; i < 16; ++i) {
+      lsum += pv[i];
+      asum = fmaf(pv[i], uv[i], asum);
+      pb[i / 8][i % 8] = (__bf16)pv[i];
     }
+    __builtin_amdgcn_sched_barrier(0);
+    read_ka(nxt);  // next tile's K fragments (stale bytes after the last tile, never used)
+    __builtin_amdgcn_sched_barrier(0);
 
-    // O^T[f][q] += sum_key K^T[f][key] * (P*rk)[key][q]
+    // O^T[f][q] += sum_key Kh^T[f][key] * P[key][q]; contraction slot
+    // 8h + 4gg + j of step tt is key 16tt + 8gg + 4h + j on both operands.
 #pragma unroll
     for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
       for (int fb = 0; fb < FB; ++fb)
-        oacc[fb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ta[fb][tt], pb[tt], oacc[fb], 0, 0, 0);
-
-    if (more) store_tile(buf ^ 1);
-    __syncthreads();
+        oacc[fb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ta[tt * FB + fb], pb[tt], oacc[fb], 0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    cur = nxt;
   }
 
   // partial results, register-native order: [split][q tile of 32][fb][i][lane]
@@ -399,15 +405,19 @@ __global__ __launch_bounds__(kNceBlock) void nce_main_kernel(const uint16_t* __r
 //   <qh_i, sum_j P_ij kh_j> = (tau/log2e) A_i / l_i,  <qh_i, kh_i> = (tau/log2e) diag_i
 // ---------------------------------------------------------------------------
 template <typename T, int C>
-__global__ __launch_bounds__(kNceBlock) void nce_combine_kernel(const T* __restrict__ q, const T* __restrict__ k,
-                                                                const float* __restrict__ rq,
-                                                                const float* __restrict__ rk,
-                                                                const float* __restrict__ diag,
-                                                                const float* __restrict__ lpart,
-                                                                const float* __restrict__ apart,
-                                                                const float* __restrict__ opart, int64_t n,
-                                                                int64_t npad, int splits, float scale2,
-                                                                float* __restrict__ row_loss, T* __restrict__ dq) {
+__global__ __launch_bounds__(kNceBlock) void nce_combine_kernel(NceArgs args, int64_t n, int64_t npad, int splits,
+                                                                float scale2) {
+  const NcePair& pr = args.p[blockIdx.z];
+  const T* __restrict__ q = (const T*)pr.q;
+  const T* __restrict__ k = (const T*)pr.k;
+  const float* __restrict__ rq = pr.rq;
+  const float* __restrict__ rk = pr.rk;
+  const float* __restrict__ diag = pr.diag;
+  const float* __restrict__ lpart = pr.lpart;
+  const float* __restrict__ apart = pr.apart;
+  const float* __restrict__ opart = pr.opart;
+  float* __restrict__ row_loss = pr.row_loss;
+  T* __restrict__ dq = (T*)pr.dq;
   constexpr int FB = C / 32;
   const int lane = threadIdx.x % kWave, w = threadIdx.x / kWave;
   const int col = lane % 32, h = lane / 32;
@@ -458,46 +468,30 @@ __global__ __launch_bounds__(kNceBlock) void nce_combine_kernel(const T* __restr
 }
 
 template <typename T, int C>
-int nce_run_pair(const void* q, const void* k, void* dq, int64_t n, float tau, char* ws, float* row_loss,
-                 const NceLayout& L, hipStream_t stream) {
-  constexpr bool kF32 = sizeof(T) == 4;
-  float* rq = (float*)(ws + L.off_rq);
-  float* rk = (float*)(ws + L.off_rk);
-  float* diag = (float*)(ws + L.off_diag);
-  float* lpart = (float*)(ws + L.off_lpart);
-  float* apart = (float*)(ws + L.off_apart);
-  uint16_t* kt = (uint16_t*)(ws + L.off_kt);
-  uint16_t* qb = kF32 ? (uint16_t*)(ws + L.off_qb) : nullptr;
-  uint16_t* kb = kF32 ? (uint16_t*)(ws + L.off_kb) : nullptr;
-  float* opart = (float*)(ws + L.off_opart);
+int nce_run(const NceArgs& args, int pairs, int64_t n, float tau, const NceLayout& L, hipStream_t stream) {
   const float scale2 = kNceLog2e / tau;
-
-  hipLaunchKernelGGL((nce_prep_kernel<T, C>), dim3((unsigned)(L.npad / NcePrep<T, C>::ROWS)), dim3(kNceBlock), 0,
-                     stream, (const T*)q, (const T*)k, n, L.npad, scale2, rq, rk, diag, kt, qb, kb);
+  const unsigned z = (unsigned)pairs;
+  hipLaunchKernelGGL((nce_prep_kernel<T, C>), dim3((unsigned)(L.npad / kKTile), 1, z), dim3(kNceBlock), 0, stream, args,
+                     n, L.npad, scale2);
   int rc = check_launch();
   if (rc) return rc;
-  const uint16_t* qsrc = kF32 ? qb : (const uint16_t*)q;
-  const uint16_t* ksrc = kF32 ? kb : (const uint16_t*)k;
-  // with bf16 copies the rows beyond n exist (zero); the kernel guards by n either way
-  hipLaunchKernelGGL((nce_main_kernel<C>), dim3((unsigned)L.splits, (unsigned)(L.npad / kQTile)),
-                     dim3(kNceBlock), 0, stream, qsrc, ksrc, kt, rq, rk, n, L.npad, L.splits, scale2, lpart,
-                     apart, opart);
+  hipLaunchKernelGGL((nce_main_kernel<C>), dim3((unsigned)L.splits, (unsigned)(L.npad / kQTile), z), dim3(kNceBlock),
+                     0, stream, args, n, L.npad, L.splits, scale2);
   rc = check_launch();
   if (rc) return rc;
   const int64_t items = L.npad / 32 * (C / 32);  // a multiple of 4: npad is a multiple of 128
-  hipLaunchKernelGGL((nce_combine_kernel<T, C>), dim3((unsigned)(items / 4)), dim3(kNceBlock), 0, stream,
-                     (const T*)q, (const T*)k, rq, rk, diag, lpart, apart, opart, n, L.npad, L.splits, scale2,
-                     row_loss, (T*)dq);
+  hipLaunchKernelGGL((nce_combine_kernel<T, C>), dim3((unsigned)(items / 4), 1, z), dim3(kNceBlock), 0, stream, args,
+                     n, L.npad, L.splits, scale2);
   return check_launch();
 }
 
 template <typename T>
-int nce_dispatch_c(const void* q, const void* k, void* dq, int64_t n, int64_t c, float tau, char* ws,
-                   float* row_loss, const NceLayout& L, hipStream_t stream) {
+int nce_dispatch_c(const NceArgs& args, int pairs, int64_t n, int64_t c, float tau, const NceLayout& L,
+                   hipStream_t stream) {
   switch (c) {
-    case 64: return nce_run_pair<T, 64>(q, k, dq, n, tau, ws, row_loss, L, stream);
-    case 128: return nce_run_pair<T, 128>(q, k, dq, n, tau, ws, row_loss, L, stream);
-    case 256: return nce_run_pair<T, 256>(q, k, dq, n, tau, ws, row_loss, L, stream);
+    case 64: return nce_run<T, 64>(args, pairs, n, tau, L, stream);
+    case 128: return nce_run<T, 128>(args, pairs, n, tau, L, stream);
+    case 256: return nce_run<T, 256>(args, pairs, n, tau, L, stream);
     default: return TS_ERR_ARG;
   }
 }
@@ -536,16 +530,28 @@ int ts_infonce_fwd_bwd(const void* q1, const void* k1, const void* q2, const voi
   const ts::NceLayout L = ts::nce_layout(n, c, pairs, true);
   char* ws = (char*)workspace;
   float* row_loss = (float*)ws;
-  for (int p = 0; p < pairs; ++p) {
-    const void* q = p ? q2 : q1;
-    const void* k = p ? k2 : k1;
-    void* dq = p ? dq2 : dq1;
-    char* wsp = ws + L.head_bytes + (size_t)p * L.pair_bytes;
-    float* rl = row_loss + (size_t)p * L.npad;
-    int rc = (dtype == TS_F32) ? ts::nce_dispatch_c<float>(q, k, dq, n, c, tau, wsp, rl, L, st)
-                               : ts::nce_dispatch_c<ts::bf16_t>(q, k, dq, n, c, tau, wsp, rl, L, st);
-    if (rc) return rc;
+  ts::NceArgs args;
+  for (int p = 0; p < 2; ++p) {
+    const int src = p < pairs ? p : 0;  // an unused second slot mirrors the first
+    char* wsp = ws + L.head_bytes + (size_t)src * L.pair_bytes;
+    ts::NcePair& P = args.p[p];
+    P.q = src ? q2 : q1;
+    P.k = src ? k2 : k1;
+    P.dq = src ? dq2 : dq1;
+    P.rq = (float*)(wsp + L.off_rq);
+    P.rk = (float*)(wsp + L.off_rk);
+    P.diag = (float*)(wsp + L.off_diag);
+    P.lpart = (float*)(wsp + L.off_lpart);
+    P.apart = (float*)(wsp + L.off_apart);
+    P.opart = (float*)(wsp + L.off_opart);
+    P.kimg = (uint8_t*)(wsp + L.off_kimg);
+    P.qb = dtype == TS_F32 ? (uint16_t*)(wsp + L.off_qb) : nullptr;
+    P.qsrc = dtype == TS_F32 ? P.qb : (const uint16_t*)P.q;
+    P.row_loss = row_loss + (size_t)src * L.npad;
   }
+  const int rc = (dtype == TS_F32) ? ts::nce_dispatch_c<float>(args, pairs, n, c, tau, L, st)
+                                   : ts::nce_dispatch_c<ts::bf16_t>(args, pairs, n, c, tau, L, st);
+  if (rc) return rc;
   // loss = 2 tau / n * sum over all pairs' rows (padding rows hold zero)
   return ts::launch_sum_scale(row_loss, (int64_t)pairs * L.npad, 2.f * tau, (float)n, loss_out, st);
 }
