@@ -26,7 +26,7 @@
 //            32 q rows; per 32-key tile: S^T = Kh Q^T (MFMA 32x32x16),
 //            P = 2^(S*scale - x_max), l += P, O^T += Kh^T P (MFMA).  Tile
 //            images go from global memory straight into LDS (no registers),
-//            two tiles ahead.  Writes per-split partial l and O^T in
+//            three tiles ahead.  Writes per-split partial l and O^T in
 //            register-native order.
 //   combine  per 32-row q tile: adds the splits, forms loss rows and dq.
 //
@@ -230,7 +230,7 @@ __global__ __launch_bounds__(kNceBlock) void nce_prep_kernel(NceArgs args, int64
 // ---------------------------------------------------------------------------
 typedef __attribute__((address_space(3))) void nce_lds_void;
 typedef __attribute__((address_space(1))) const void nce_glb_void;
-constexpr int kNceBufs = 3;  // tile images in LDS: the one in use and two on their way
+constexpr int kNceBufs = 4;  // tile images in LDS: two in use (tiles t, t+1), two on their way
 
 template <int C>
 __global__ __launch_bounds__(kNceBlock) void nce_main_kernel(NceArgs args, int64_t n, int64_t npad, int splits,
@@ -277,6 +277,7 @@ __global__ __launch_bounds__(kNceBlock) void nce_main_kernel(NceArgs args, int64
 
   if (t0 < t1) fetch_tile(t0, 0);
   if (t0 + 1 < t1) fetch_tile(t0 + 1, 1);
+  if (t0 + 2 < t1) fetch_tile(t0 + 2, 2);
 
   // Q fragments: B operand of S^T, resident for the whole kernel.
   bf16x8 qf[KK];
@@ -299,10 +300,12 @@ __global__ __launch_bounds__(kNceBlock) void nce_main_kernel(NceArgs args, int64
   // tiles from this one on contain padded keys (never reached when n is a multiple of the tile)
   const int64_t t_pad = n / kKTile;
 
-  // Operand fragments live in registers one phase ahead of the MFMAs that use
-  // them, so that the LDS reads of one product overlap the MFMAs of the
-  // other: tile t's K^T fragments are read while its first product runs, tile
-  // t+1's K fragments while tile t's second product runs.
+  // The loop is software-pipelined so that the matrix pipe and the vector
+  // ALU work at the same time: tile t+1's first product is issued before
+  // tile t's soft-max, whose exponentials then run while those MFMAs execute.
+  // Operand fragments are read from LDS a phase ahead of their MFMAs for the
+  // same reason: tile t's K^T fragments while tile t+1's first product runs,
+  // tile t+2's K fragments while tile t's second product runs.
   bf16x8 ka[KK];
   auto read_ka = [&](int buf) {
 #pragma unroll
@@ -311,55 +314,55 @@ __global__ __launch_bounds__(kNceBlock) void nce_main_kernel(NceArgs args, int64
       __builtin_memcpy(&ka[kk], &raw, 16);
     }
   };
-  wait_fetches_and_sync();
-  read_ka(0);
+  // S^T[key][q] = sum_f Kh[key][f] Q[q][f], as two independent accumulation
+  // chains: a dependent MFMA waits for its predecessor's result.
+  struct SAcc {
+    f32x16 a, b;
+  };
+  auto first_product = [&](SAcc& s) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) s.a[i] = s.b[i] = 0.f;
+#pragma unroll
+    for (int kk = 0; kk < KK; kk += 2) {
+      s.a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[kk], qf[kk], s.a, 0, 0, 0);
+      s.b = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[kk + 1], qf[kk + 1], s.b, 0, 0, 0);
+    }
+  };
 
-  int cur = 0;
-  for (int64_t t = t0; t < t1; ++t) {
-    const int nxt = (cur == kNceBufs - 1) ? 0 : cur + 1;
-    const int nn = (nxt == kNceBufs - 1) ? 0 : nxt + 1;
-    // After this barrier tile t+1 is complete in LDS (its fetches were issued
+  int cur = 0;  // buffer of tile t
+  auto next_buf = [](int b) { return b == kNceBufs - 1 ? 0 : b + 1; };
+
+  // One tile; sa holds S^T of tile t on entry, sb receives tile t+1's.
+  auto step = [&](int64_t t, const SAcc& sa, SAcc& sb) {
+    const int b1 = next_buf(cur), b2 = next_buf(b1), b3 = next_buf(b2);
+    // After this barrier tile t+2 is complete in LDS (its fetches were issued
     // a whole tile ago) and every wavefront has finished reading tile t-1,
     // whose buffer the fetch below overwrites.
     wait_fetches_and_sync();
 
+    // no branch (one would split the scheduling regions below): near the end
+    // the fetch repeats the last tile into a buffer nobody reads any more
+    fetch_tile(t + 3 < ktiles ? t + 3 : ktiles - 1, b3);
+    __builtin_amdgcn_sched_barrier(0);
+
+    // Phase 1: tile t+1's first product; in its shadow tile t's soft-max and
+    // the reads of tile t's K^T fragments, which take over the registers of
+    // the K fragments as the MFMAs release them.
+    first_product(sb);  // stale operands after the last tile: result unused
     bf16x8 ta[2 * FB];
 #pragma unroll
     for (int x = 0; x < 2 * FB; ++x) {
       const u32x4 raw = *reinterpret_cast<const u32x4*>(&sm[cur][(KK + x) * 1024 + lane * 16]);
       __builtin_memcpy(&ta[x], &raw, 16);
     }
-    if (t + 2 < t1) fetch_tile(t + 2, nn);
-    __builtin_amdgcn_sched_barrier(0);  // the reads above are issued before the MFMAs below
-
-    // S^T[key][q] = sum_f Kh[key][f] Q[q][f], as two independent accumulation
-    // chains: a dependent MFMA waits for its predecessor's result.
-    f32x16 sacc0, sacc1;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) sacc0[i] = sacc1[i] = 0.f;
-#pragma unroll
-    for (int kk = 0; kk < KK; kk += 2) {
-      sacc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[kk], qf[kk], sacc0, 0, 0, 0);
-      sacc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[kk + 1], qf[kk + 1], sacc1, 0, 0, 0);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-
     // P = 2^(S * rq_i * log2e/tau - x_max); keys this lane holds:
     // key(i) = (i%4) + 4h + 8(i/4).  With u = x - x_max the kernel sums
     // l = sum P and a' = sum P u; sum P x follows as a' + x_max l at the end.
     float pv[16], uv[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
-      uv[i] = fmaf(sacc0[i] + sacc1[i], sc_i, -scale2);
+      uv[i] = fmaf(sa.a[i] + sa.b[i], sc_i, -scale2);
       pv[i] = fast_exp2(uv[i]);
-    }
-    if (t >= t_pad) {
-      // padded keys, only at the very end of the key range (their image rows
-      // are zero, which zeroes the second product, but not the row sums)
-      const int keyb = (int)(t * kKTile) + 4 * h;
-#pragma unroll
-      for (int i = 0; i < 16; ++i)
-        if (keyb + 8 * (i / 4) + (i % 4) >= (int)n) pv[i] = 0.f;
     }
     bf16x8 pb[2];
 #pragma unroll
@@ -368,19 +371,66 @@ __global__ __launch_bounds__(kNceBlock) void nce_main_kernel(NceArgs args, int64
       asum = fmaf(pv[i], uv[i], asum);
       pb[i / 8][i % 8] = (__bf16)pv[i];
     }
-    __builtin_amdgcn_sched_barrier(0);
-    read_ka(nxt);  // next tile's K fragments (stale bytes after the last tile, never used)
+    // An MFMA occupies the matrix pipe for tens of cycles, but the wavefront
+    // issues in order: only instructions placed between two MFMAs run in
+    // their shadow.  Ask the scheduler for that interleaving.
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                    // one MFMA
+      __builtin_amdgcn_sched_group_barrier(0x100, (2 * FB + KK - 1) / KK, 0);  // LDS reads
+      __builtin_amdgcn_sched_group_barrier(0x002, (112 + KK - 1) / KK, 0);  // its share of the soft-max
+    }
     __builtin_amdgcn_sched_barrier(0);
 
-    // O^T[f][q] += sum_key Kh^T[f][key] * P[key][q]; contraction slot
+    // Phase 2: O^T[f][q] += sum_key Kh^T[f][key] * P[key][q]; contraction slot
     // 8h + 4gg + j of step tt is key 16tt + 8gg + 4h + j on both operands.
+    // In its shadow the reads of tile t+2's K fragments (stale bytes near the
+    // end, never used), into the registers the K^T fragments release.
 #pragma unroll
     for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
       for (int fb = 0; fb < FB; ++fb)
         oacc[fb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ta[tt * FB + fb], pb[tt], oacc[fb], 0, 0, 0);
+    read_ka(b2);
+#pragma unroll
+    for (int x = 0; x < 2 * FB; ++x) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, (KK + 2 * FB - 1) / (2 * FB), 0);
+    }
     __builtin_amdgcn_sched_barrier(0);
-    cur = nxt;
+    cur = b1;
+  };
+
+  // prologue: S^T of the first tile, K fragments of the second
+  SAcc sx, sy;
+  wait_fetches_and_sync();
+  read_ka(0);
+  first_product(sx);
+  __builtin_amdgcn_sched_barrier(0);
+  read_ka(1);
+  __builtin_amdgcn_sched_barrier(0);
+
+  // two tiles per trip, so that the S^T registers alternate without copies
+  for (int64_t t = t0; t < t1; t += 2) {
+    step(t, sx, sy);
+    if (t + 1 < t1) step(t + 1, sy, sx);
+  }
+
+  // The last trips fetched tiles nobody reads; they must have landed before
+  // this workgroup's LDS can be handed to another one.
+  __builtin_amdgcn_s_waitcnt(0x0f70);
+
+  // Padded keys (image rows of zeros) took part in the row sums with the same
+  // term for every row, 2^(0 - x_max); take this lane's share of them out.
+  {
+    int cnt = 0;
+    for (int64_t t = (t0 > t_pad ? t0 : t_pad); t < t1; ++t)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) cnt += (t * kKTile + 4 * h + 8 * (i / 4) + (i % 4) >= n) ? 1 : 0;
+    const float u0 = fmaf(0.f, sc_i, -scale2);
+    const float c0 = (float)cnt * fast_exp2(u0);
+    lsum -= c0;
+    asum = fmaf(-c0, u0, asum);
   }
 
   // partial results, register-native order: [split][q tile of 32][fb][i][lane]
