@@ -433,7 +433,7 @@ __global__ __launch_bounds__(kNceBlock) void nce_main_kernel(NceArgs args, int64
     asum = fmaf(-c0, u0, asum);
   }
 
-  // partial results, register-native order: [split][q tile of 32][fb][i][lane]
+  // partial results in register-native order
   const float ltot = lsum + __shfl_xor(lsum, 32, kWave);
   // sum_j P_ij x_ij = <qh_i, sum_j P_ij kh_j> * log2e/tau
   const float atot = asum + __shfl_xor(asum, 32, kWave) + scale2 * ltot;
@@ -442,11 +442,15 @@ __global__ __launch_bounds__(kNceBlock) void nce_main_kernel(NceArgs args, int64
     apart[(int64_t)split * npad + qtile * kQTile + w * 32 + col] = atot;
   }
   const int64_t tile32 = qtile * (kQTile / 32) + w;
-  float* op = opart + (((int64_t)split * (npad / 32) + tile32) * FB) * 16 * kWave;
+  // [split][q tile of 32][fb][i/4][lane][i%4]: 16 bytes per lane and store
+  f32x4* op = reinterpret_cast<f32x4*>(opart + (((int64_t)split * (npad / 32) + tile32) * FB) * 16 * kWave);
 #pragma unroll
   for (int fb = 0; fb < FB; ++fb)
 #pragma unroll
-    for (int i = 0; i < 16; ++i) op[(fb * 16 + i) * kWave + lane] = oacc[fb][i];
+    for (int g = 0; g < 4; ++g) {
+      const f32x4 v = {oacc[fb][4 * g], oacc[fb][4 * g + 1], oacc[fb][4 * g + 2], oacc[fb][4 * g + 3]};
+      op[(fb * 4 + g) * kWave + lane] = v;
+    }
 }
 
 // ---------------------------------------------------------------------------
@@ -487,13 +491,35 @@ __global__ __launch_bounds__(kNceBlock) void nce_combine_kernel(NceArgs args, in
   if (fb == 0 && h == 0) row_loss[row] = live ? kNceLn2 * (scale2 + log2f(l) - d) : 0.f;
   if (!dq) return;
 
+  // all loads of four splits are issued before the first add: the kernel is
+  // bound by memory latency, not by arithmetic
   float o[16];
 #pragma unroll
   for (int i = 0; i < 16; ++i) o[i] = 0.f;
-  for (int s = 0; s < splits; ++s) {
-    const float* op = opart + (((int64_t)s * (npad / 32) + tile32) * FB + fb) * 16 * kWave;
+  const int64_t split_stride = (npad / 32) * FB * 16 * kWave;  // floats
+  const f32x4* op0 = reinterpret_cast<const f32x4*>(opart + (tile32 * FB + fb) * 16 * kWave) + lane;
+  int s0 = 0;
+  for (; s0 + 4 <= splits; s0 += 4) {
+    f32x4 v[4][4];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) o[i] += op[i * kWave + lane];
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int g = 0; g < 4; ++g)
+        v[u][g] = reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(op0) + (s0 + u) * split_stride)[g * kWave];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int g = 0; g < 4; ++g)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) o[4 * g + j] += v[u][g][j];
+  }
+  for (; s0 < splits; ++s0) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const f32x4 v = reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(op0) + s0 * split_stride)[g * kWave];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) o[4 * g + j] += v[j];
+    }
   }
   if (!live) return;
   const float inv_l = 1.f / l;

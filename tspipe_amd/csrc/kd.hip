@@ -605,8 +605,19 @@ __global__ __launch_bounds__(1024) void kd_finalize_kernel(const float* __restri
                                                            const int* __restrict__ counts /* null: n KD rows */,
                                                            float* __restrict__ out) {
   __shared__ float lds[1024 / kWave];
-  float akd = 0.f, ace = 0.f;
-  for (int64_t i = threadIdx.x; i < n; i += 1024) {
+  // 16-byte loads, four of them in flight per thread: one block has to get
+  // through the whole array, so the loop is bound by memory latency
+  const int64_t n4 = n / 4;
+  const f32x4* kd4 = reinterpret_cast<const f32x4*>(row_kd);
+  const f32x4* ce4 = reinterpret_cast<const f32x4*>(row_ce);
+  f32x4 vkd = {0.f, 0.f, 0.f, 0.f}, vce = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+  for (int64_t i = threadIdx.x; i < n4; i += 1024) {
+    vkd += kd4[i];
+    if (row_ce) vce += ce4[i];
+  }
+  float akd = (vkd[0] + vkd[1]) + (vkd[2] + vkd[3]), ace = (vce[0] + vce[1]) + (vce[2] + vce[3]);
+  for (int64_t i = n4 * 4 + threadIdx.x; i < n; i += 1024) {
     akd += row_kd[i];
     if (row_ce) ace += row_ce[i];
   }
