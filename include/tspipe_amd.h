@@ -46,6 +46,14 @@ const char* ts_version(void);
 const char* ts_error_string(int status);
 /* Last HIP error code recorded by a failed launch in this thread (0 if none). */
 int ts_last_hip_error(void);
+/* Measurement aid, no counterpart in the reference.  Arms the calling thread:
+ * the next kernel launched by ts_ema_multi, ts_ema_clone_multi or
+ * ts_copy_segments from this thread records its own begin and end timestamps
+ * into the two HIP events (hipEvent_t, created with timing enabled), as
+ * hipExtLaunchKernel does; hipEventElapsedTime(start, stop) is then the
+ * kernel's duration without the marker packets an event pair recorded around
+ * the call would add.  Passing two nulls disarms. */
+int ts_time_next_launch(void* start_event, void* stop_event);
 
 /* ------------------------------------------------------------------------ */
 /* Momentum-teacher EMA over a whole parameter list, one launch.         */

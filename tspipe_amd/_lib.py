@@ -24,6 +24,7 @@ SIGNATURES = {
     "ts_version": (c_char_p, []),
     "ts_error_string": (c_char_p, [c_int]),
     "ts_last_hip_error": (c_int, []),
+    "ts_time_next_launch": (c_int, [c_void_p, c_void_p]),
     "ts_ema_auto_chunk": (c_int64, [c_int64]),
     "ts_ema_plan": (c_int64, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_int64]),
     "ts_ema_multi": (c_int, [c_void_p, c_int64, c_int64, c_float, c_float, c_void_p]),
@@ -128,6 +129,34 @@ def dtype_code(dtype) -> int:
     if dtype == torch.float16:
         return TS_F16
     raise TypeError(f"unsupported dtype {dtype}: the kernels take float32, bfloat16 or float16")
+
+
+_event_pool = []
+
+
+def prepare_timing_events(device, count: int) -> None:
+    """Creates ``count`` pairs of timing events ahead of time, so that
+    ``time_next_launch`` inside a timed region costs no event creation and no
+    extra marker packet on the stream."""
+    import torch
+    stream = torch.cuda.current_stream(device)
+    for _ in range(count):
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        # a first record creates the HIP events; the launch re-records them
+        start.record(stream)
+        end.record(stream)
+        _event_pool.append((start, end))
+
+
+def time_next_launch(device):
+    """Arms the calling thread so that the next EMA / copy kernel stamps its
+    own begin and end into a pair of timing events (measurement aid); returns
+    the pair for ``start.elapsed_time(end)`` after a synchronize."""
+    if not _event_pool:
+        prepare_timing_events(device, 1)
+    start, end = _event_pool.pop()
+    check(lib().ts_time_next_launch(start.cuda_event, end.cuda_event), "ts_time_next_launch")
+    return start, end
 
 
 def current_stream_ptr(device) -> int:

@@ -18,7 +18,7 @@ from . import _lib
 ENTRY_BYTES = 32
 _RING = 4
 # When set to a list, every multi-segment copy appends a (start, end) pair of
-# HIP events recorded on the launch stream around the kernel alone (profiling aid).
+# HIP events stamped with the kernel's own begin and end (profiling aid).
 kernel_events = None
 _tls = threading.local()
 
@@ -145,12 +145,10 @@ def copy_segments(srcs: Sequence[torch.Tensor], dsts: Sequence[torch.Tensor]) ->
     table = stage_copy(ptr_array(srcs), ptr_array(dsts), nbytes, device)
     timed = kernel_events is not None
     if timed:
-        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        start.record(torch.cuda.current_stream(device))
+        start, end = _lib.time_next_launch(device)
     _lib.check(_lib.lib().ts_copy_segments(table.dev_ptr, table.n_chunks, table.chunk,
                                            _lib.current_stream_ptr(device)),
                "ts_copy_segments")
     if timed:
-        end.record(torch.cuda.current_stream(device))
         kernel_events.append((start, end))
     table.done()

@@ -18,6 +18,9 @@ typedef uint16_t u16x8 __attribute__((ext_vector_type(8)));
 
 // Records the HIP error of a failed launch for ts_last_hip_error().
 void set_last_hip_error(int code);
+// Hands out (and clears) the events ts_time_next_launch() armed this thread
+// with; false when there are none.
+bool take_launch_events(hipEvent_t* start, hipEvent_t* stop);
 
 inline int check_launch() {
   hipError_t e = hipGetLastError();

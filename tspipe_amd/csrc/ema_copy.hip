@@ -9,6 +9,7 @@
 // 5.0-5.8 TB/s.  So a table entry (chunk) is cut into sub-blocks, one
 // workgroup each: blockIdx = chunk * subs + sub.
 #include "common.h"
+#include <hip/hip_ext.h>
 
 namespace ts {
 
@@ -121,6 +122,17 @@ __global__ __launch_bounds__(kCopyBlock) void copy_segments_kernel(const ts_copy
 
 }  // namespace ts
 
+// A launch that, when the thread is armed with timing events, stamps the
+// kernel's own begin and end into them (hipExtLaunchKernel semantics).
+#define TS_LAUNCH_TIMED(kernel, grid, block, stream, ...)                                  \
+  do {                                                                                     \
+    hipEvent_t ev0_, ev1_;                                                                 \
+    if (ts::take_launch_events(&ev0_, &ev1_))                                              \
+      hipExtLaunchKernelGGL(kernel, grid, block, 0, stream, ev0_, ev1_, 0, __VA_ARGS__);   \
+    else                                                                                   \
+      hipLaunchKernelGGL(kernel, grid, block, 0, stream, __VA_ARGS__);                     \
+  } while (0)
+
 extern "C" {
 
 int ts_ema_multi(const ts_ema_chunk* table_dev, int64_t n_chunks, int64_t chunk_elems, float m32,
@@ -130,8 +142,8 @@ int ts_ema_multi(const ts_ema_chunk* table_dev, int64_t n_chunks, int64_t chunk_
   if (!table_dev) return TS_ERR_ARG;
   const int64_t subs = chunk_elems / ts::kSubElems;
   if (subs > 0x7fffffffLL || n_chunks * subs > 0x7fffffffLL) return TS_ERR_RANGE;
-  hipLaunchKernelGGL(ts::ema_multi_kernel<false>, dim3((unsigned)(n_chunks * subs)), dim3(ts::kEmaBlock), 0,
-                     (hipStream_t)stream, table_dev, (uint32_t)subs, m32, c32, (int64_t)0);
+  TS_LAUNCH_TIMED(ts::ema_multi_kernel<false>, dim3((unsigned)(n_chunks * subs)), dim3(ts::kEmaBlock),
+                  (hipStream_t)stream, table_dev, (uint32_t)subs, m32, c32, (int64_t)0);
   return ts::check_launch();
 }
 
@@ -144,8 +156,8 @@ int ts_ema_clone_multi(const ts_ema_chunk* table_dev, int64_t n_chunks, int64_t 
   if (!table_dev) return TS_ERR_ARG;
   const int64_t subs = chunk_elems / ts::kSubElems;
   if (subs > 0x7fffffffLL || n_chunks * subs > 0x7fffffffLL) return TS_ERR_RANGE;
-  hipLaunchKernelGGL(ts::ema_multi_kernel<true>, dim3((unsigned)(n_chunks * subs)), dim3(ts::kEmaBlock), 0,
-                     (hipStream_t)stream, table_dev, (uint32_t)subs, m32, c32, clone_offset_bytes);
+  TS_LAUNCH_TIMED(ts::ema_multi_kernel<true>, dim3((unsigned)(n_chunks * subs)), dim3(ts::kEmaBlock),
+                  (hipStream_t)stream, table_dev, (uint32_t)subs, m32, c32, clone_offset_bytes);
   return ts::check_launch();
 }
 
@@ -156,7 +168,7 @@ int ts_copy_segments(const ts_copy_chunk* table_dev, int64_t n_chunks, int64_t c
   if (!table_dev) return TS_ERR_ARG;
   const int64_t subs = chunk_bytes / ts::kSubBytes;
   if (subs > 0x7fffffffLL || n_chunks * subs > 0x7fffffffLL) return TS_ERR_RANGE;
-  hipLaunchKernelGGL(ts::copy_segments_kernel, dim3((unsigned)(n_chunks * subs)), dim3(ts::kCopyBlock), 0,
+  TS_LAUNCH_TIMED(ts::copy_segments_kernel, dim3((unsigned)(n_chunks * subs)), dim3(ts::kCopyBlock),
                      (hipStream_t)stream, table_dev, (uint32_t)subs);
   return ts::check_launch();
 }

@@ -20,7 +20,7 @@ import torch
 from . import _lib, _tables
 
 # When set to a list, every EMA launch appends a (start, end) pair of HIP
-# events recorded on the launch stream around the kernel alone (profiling aid).
+# events stamped with the kernel's own begin and end (profiling aid).
 kernel_events = None
 
 
@@ -78,15 +78,13 @@ def _launch(m: float, students: Sequence[torch.Tensor], teachers: Sequence[torch
         table = _tables.stage_ema(_ptrs(teachers), _ptrs(students), out_ptrs, numels, device)
         timed = kernel_events is not None
         if timed:
-            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            start.record(torch.cuda.current_stream(device))
+            start, end = _lib.time_next_launch(device)
         # the reference multiplies by the Python doubles m and (1. - m); torch
         # rounds each to fp32 before the fp32 multiply, and so does ctypes here
         status = _lib.lib().ts_ema_multi(table.dev_ptr, table.n_chunks, table.chunk, float(m), 1.0 - float(m),
                                         _lib.current_stream_ptr(device))
         _lib.check(status, "ts_ema_multi")
         if timed:
-            end.record(torch.cuda.current_stream(device))
             kernel_events.append((start, end))
         table.done()
 
@@ -128,13 +126,11 @@ def _fast_update(m: float, online, target) -> Optional[List[torch.Tensor]]:
         table = _tables.stage_ema(tp[:n], sp[:n], arena.ptrs, arena.numels, device)
         timed = kernel_events is not None
         if timed:
-            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            start.record(torch.cuda.current_stream(device))
+            start, end = _lib.time_next_launch(device)
         status = _lib.lib().ts_ema_multi(table.dev_ptr, table.n_chunks, table.chunk, float(m), 1.0 - float(m),
                                         _lib.current_stream_ptr(device))
         _lib.check(status, "ts_ema_multi")
         if timed:
-            end.record(torch.cuda.current_stream(device))
             kernel_events.append((start, end))
         table.done()
     return list(arena.views)
@@ -272,9 +268,14 @@ def clone_and_update(m: float, online_param: Iterable[torch.Tensor], target_para
     device = teachers[0].device
     with torch.cuda.device(device):
         table = _tables.stage_ema(_ptrs(teachers), _ptrs(students), ema_arena.ptrs, ema_arena.numels, device)
+        timed = kernel_events is not None
+        if timed:
+            start, end = _lib.time_next_launch(device)
         status = _lib.lib().ts_ema_clone_multi(table.dev_ptr, table.n_chunks, table.chunk, float(m), 1.0 - float(m),
                                               offset, _lib.current_stream_ptr(device))
         _lib.check(status, "ts_ema_clone_multi")
+        if timed:
+            kernel_events.append((start, end))
         table.done()
     return list(clone_arena.views), views
 
