@@ -202,6 +202,26 @@ int ts_byol_fwd_bwd(const void* x1, const void* y1, const void* x2, const void* 
                     int64_t c, float* workspace, float* loss_out, void* gx1, void* gx2,
                     int dtype, ts_stream_t stream);
 
+/* Squared error between student and teacher logits, forward and backward:
+ *   Logits.forward (benchmarks/soft_target/kd_losses/logits.py:17-20), F.mse_loss
+ *     with its mean over all elements: per_element = 1, row_mask = NULL;
+ *   the alpha_mse term of DistilBERT's loss (benchmarks/distilbert/distiller.py:751-755),
+ *     MSELoss(reduction="sum") over the rows the mask keeps, divided by their
+ *     number: per_element = 0.
+ *   loss = weight * sum_{rows with row_mask != 0} sum_v (s - t)^2 / denom,
+ *   denom = selected rows (x V if per_element);  grad = d loss / d s, zero on
+ *   the other rows.  accumulate != 0 adds loss and gradient to what loss_out
+ *   and grad already hold (the term joins a KD gradient in place) and leaves
+ *   unselected rows untouched.
+ * s, t, grad: [n_rows, V] with leading dimensions; grad may be NULL.
+ * workspace: ts_mse_workspace_bytes(n_rows, V) bytes, 16-byte aligned. */
+size_t ts_mse_workspace_bytes(int64_t n_rows, int64_t V);
+
+int ts_mse_fwd_bwd(const void* s, const void* t, const uint8_t* row_mask, int64_t n_rows, int64_t V,
+                   int64_t ld_s, int64_t ld_t, float weight, int per_element, int accumulate,
+                   void* workspace, float* loss_out, void* grad, int64_t ld_g, int dtype,
+                   ts_stream_t stream);
+
 /* Cosine embedding loss with target +1, forward and backward: the hidden-state
  * term of DistilBERT's loss (benchmarks/distilbert/distiller.py:756-770,
  * nn.CosineEmbeddingLoss(reduction="mean") on the rows the attention mask keeps):

@@ -54,25 +54,50 @@ def distil_ce(s_logits: Tensor, t_logits: Tensor, row_mask: Tensor, temperature:
     return alpha_ce * ce
 
 
+def logits_mse(out_s: Tensor, out_t: Tensor) -> Tensor:
+    """benchmarks/soft_target/kd_losses/logits.py:17-20."""
+    return F.mse_loss(out_s, out_t)
+
+
 def soft_target_tspipe_loss(model_out: Tensor, ema_model_out: Tensor, label: Tensor, T: float,
-                            lambda_kd: float) -> Tensor:
-    """benchmarks/soft_target/train_kd.py:439-453 with kd_mode == 'st'."""
+                            lambda_kd: float, kd_mode: str = "st") -> Tensor:
+    """benchmarks/soft_target/train_kd.py:439-453."""
     cls_loss = nn.CrossEntropyLoss()(model_out, label)
-    kd_loss = kd_soft_target(model_out, ema_model_out.detach(), T) * lambda_kd
+    if kd_mode == "logits":
+        kd_loss = logits_mse(model_out, ema_model_out.detach()) * lambda_kd
+    elif kd_mode == "st":
+        kd_loss = kd_soft_target(model_out, ema_model_out.detach(), T) * lambda_kd
+    else:
+        assert False
     return cls_loss + kd_loss
 
 
 def distil_loss(s_logits: Tensor, t_logits: Tensor, s_hidden: Optional[Tensor], t_hidden: Optional[Tensor],
                 lm_labels: Tensor, attention_mask: Tensor, alpha_ce: float, alpha_mlm: float, alpha_cos: float,
-                temperature: float, restrict_ce_to_mask: bool) -> Tensor:
-    """benchmarks/distilbert/distiller.py:711-772 without the clm and mse terms:
-    masked KD (719-740), masked-LM cross entropy with ignore_index=-100 (742-744,
-    lm_loss_fct at 117), cosine embedding loss on the last hidden states (756-770)."""
+                temperature: float, restrict_ce_to_mask: bool, alpha_clm: float = 0.0,
+                alpha_mse: float = 0.0) -> Tensor:
+    """benchmarks/distilbert/distiller.py:711-772: masked KD (719-740), masked-LM
+    cross entropy with ignore_index=-100 (742-744, lm_loss_fct at 117),
+    causal-LM cross entropy on shifted logits (745-749), sum-of-squares of the
+    selected logits over their row count (751-755, mse_loss_fct at 119), cosine
+    embedding loss on the last hidden states (756-770)."""
     mask2d = (lm_labels > -1) if restrict_ce_to_mask else attention_mask
     loss = distil_ce(s_logits, t_logits, mask2d, temperature, alpha_ce)
     if alpha_mlm > 0.0:
         loss_mlm = nn.CrossEntropyLoss(ignore_index=-100)(s_logits.view(-1, s_logits.size(-1)), lm_labels.view(-1))
         loss = loss + alpha_mlm * loss_mlm
+    if alpha_clm > 0.0:
+        shift_logits = s_logits[..., :-1, :].contiguous()
+        shift_labels = lm_labels[..., 1:].contiguous()
+        loss_clm = nn.CrossEntropyLoss(ignore_index=-100)(shift_logits.view(-1, shift_logits.size(-1)),
+                                                          shift_labels.view(-1))
+        loss = loss + alpha_clm * loss_clm
+    if alpha_mse > 0.0:
+        mask = mask2d.unsqueeze(-1).expand_as(s_logits)
+        s_sel = torch.masked_select(s_logits, mask).view(-1, s_logits.size(-1))
+        t_sel = torch.masked_select(t_logits, mask).view(-1, s_logits.size(-1))
+        loss_mse = nn.MSELoss(reduction="sum")(s_sel, t_sel) / s_sel.size(0)
+        loss = loss + alpha_mse * loss_mse
     if alpha_cos > 0.0:
         mask = attention_mask.unsqueeze(-1).expand_as(s_hidden)
         dim = s_hidden.size(-1)

@@ -329,6 +329,79 @@ def test_distil_loss_fn_plugin(device, restrict):
         assert ((got.cpu().double() - ref).abs() <= 1e-3 * peak + ref.abs() * 2.0 ** -8).all()
 
 
+@pytest.mark.parametrize("mode", ["clm", "mse", "clm+mse"])
+def test_distil_loss_fn_clm_and_mse_terms(device, mode):
+    from argparse import Namespace
+    g = seeded(231)
+    bs, seq, V = 3, 12, 5000
+    s = (torch.randn(bs, seq, V, generator=g) * 2).to(torch.bfloat16)
+    t = (torch.randn(bs, seq, V, generator=g) * 2).to(torch.bfloat16)
+    lm = torch.full((bs, seq), -100, dtype=torch.long)
+    pick = torch.rand(bs, seq, generator=g) < 0.3
+    lm[pick] = torch.randint(0, V, (int(pick.sum()),), generator=g)
+    att = torch.rand(bs, seq, generator=g) < 0.8
+    a_clm = 1.5 if "clm" in mode else 0.0
+    a_mse = 0.05 if "mse" in mode else 0.0
+    params = Namespace(alpha_ce=0.5, alpha_mlm=0.0, alpha_clm=a_clm, alpha_mse=a_mse, alpha_cos=0.0, temperature=2.0,
+                       restrict_ce_to_mask=False)
+    want, (gs,) = _oracle_grad(
+        lambda a, b: ts_oracle.distil_loss(a, b, None, None, lm, att, 0.5, 0.0, 0.0, 2.0, False, alpha_clm=a_clm,
+                                           alpha_mse=a_mse), s, others=(t,))
+    sd = s.to(device).requires_grad_()
+    loss = ta.distil_loss_fn({"logits": sd, "hidden_states": None}, {"logits": t.to(device), "hidden_states": None},
+                             (lm.to(device), att.to(device)), None, params, 0)
+    loss.backward()
+    assert rel_err(loss.item(), want) < 1e-3
+    peak = gs.abs().max().item()
+    # the MSE term is added to a gradient already stored in bf16: two roundings
+    assert ((sd.grad.cpu().double() - gs).abs() <= 1e-3 * peak + gs.abs() * 2.0 ** -7).all()
+    with pytest.raises(NotImplementedError):
+        params.alpha_mlm, params.alpha_clm = 1.0, 1.0
+        ta.distil_loss_fn({"logits": sd, "hidden_states": None}, {"logits": t.to(device), "hidden_states": None},
+                          (lm.to(device), att.to(device)), None, params, 0)
+
+
+@pytest.mark.parametrize("rows,V,dtype", [(256, 100, torch.float32), (33, 5000, torch.float32),
+                                          (40, 30522, torch.bfloat16)])
+def test_logits_mse_and_kd_mode_logits(device, rows, V, dtype):
+    from argparse import Namespace
+    g = seeded(240 + V)
+    s = (torch.randn(rows, V, generator=g) * 3).to(dtype)
+    t = (torch.randn(rows, V, generator=g) * 3).to(dtype)
+    y = torch.randint(0, V, (rows,), generator=g)
+    tol = 1e-5 if dtype == torch.float32 else 1e-3
+    # the criterion alone (kd_losses/logits.py), module form
+    want, (gw,) = _oracle_grad(lambda a, b: ts_oracle.logits_mse(a, b), s, others=(t,))
+    sd = s.to(device).requires_grad_()
+    loss = ta.Logits()(sd, t.to(device))
+    loss.backward()
+    assert rel_err(loss.item(), want) < tol
+    peak = gw.abs().max().item()
+    slack = gw.abs() * (2.0 ** -8 if dtype != torch.float32 else 0.0)
+    assert ((sd.grad.cpu().double() - gw).abs() <= tol * peak + slack).all()
+    # masked rows, sum over columns / selected rows; zero gradient elsewhere
+    mask = torch.rand(rows, generator=g) < 0.5
+    sm, tm = s[mask].double(), t[mask].double()
+    sd2 = s.to(device).requires_grad_()
+    l2 = ta.logits_mse_loss(sd2, t.to(device), mask.to(device), weight=0.5, per_element=False)
+    l2.backward()
+    assert rel_err(l2.item(), 0.5 * ((sm - tm) ** 2).sum().item() / int(mask.sum())) < tol
+    assert (sd2.grad.cpu()[~mask] == 0).all()
+    gwant = 0.5 * 2 * (sm - tm) / int(mask.sum())
+    assert ((sd2.grad.cpu()[mask].double() - gwant).abs() <= tol * gwant.abs().max() + gwant.abs() * 2.0 ** -8).all()
+    # the whole plug-in with kd_mode == 'logits'
+    want, (gw,) = _oracle_grad(lambda a, b: ts_oracle.soft_target_tspipe_loss(a, b, y, 4.0, 0.7, kd_mode="logits"), s,
+                               others=(t,))
+    sd3 = s.to(device).requires_grad_()
+    args = Namespace(kd_mode="logits", T=4.0, lambda_kd=0.7)
+    loss = ta.soft_target_tspipe_loss(sd3, t.to(device), y.to(device), None, args, 0)
+    loss.backward()
+    assert rel_err(loss.item(), want) < tol
+    peak = gw.abs().max().item()
+    slack = gw.abs() * (2.0 ** -7 if dtype != torch.float32 else 0.0)
+    assert ((sd3.grad.cpu().double() - gw).abs() <= tol * peak + slack).all()
+
+
 def test_kd_masked_cfg3_full_size_properties(device):
     # [32, 128, 30522] bf16, 15 % token mask, gathered from 4 micro-batches: too large for the
     # fp64 oracle, so checked through properties that do not depend on the size

@@ -370,3 +370,51 @@ def test_distil_loss_terms_use_their_own_row_sets():
         cos = (a * b).sum(1) / np.sqrt(((a * a).sum(1) + 1e-12) * ((b * b).sum(1) + 1e-12))
         want = 0.5 * kd + 2.0 * ce + 1.5 * (1 - cos).mean()
         assert abs(got - want) < 1e-12
+
+
+def test_logits_mse_and_kd_mode_logits_closed_form():
+    g = seeded(12)
+    s = torch.randn(6, 10, generator=g, dtype=torch.float64) * 2
+    t = torch.randn(6, 10, generator=g, dtype=torch.float64) * 2
+    y = torch.randint(0, 10, (6,), generator=g)
+    sn, tn = s.numpy(), t.numpy()
+    assert abs(ts_oracle.logits_mse(s, t).item() - ((sn - tn) ** 2).mean()) < 1e-14
+    lse = np.log(np.exp(sn).sum(1))
+    ce = (lse - sn[np.arange(6), y.numpy()]).mean()
+    sr = s.clone().requires_grad_()
+    loss = ts_oracle.soft_target_tspipe_loss(sr, t, y, 4.0, 0.3, kd_mode="logits")
+    loss.backward()
+    assert abs(loss.item() - (ce + 0.3 * ((sn - tn) ** 2).mean())) < 1e-12
+    soft = np.exp(sn - lse[:, None])
+    want = (soft - np.eye(10)[y.numpy()]) / 6 + 0.3 * 2 * (sn - tn) / 60
+    assert np.abs(sr.grad.numpy() - want).max() < 1e-13
+    # the teacher gets no gradient
+    tr = t.clone().requires_grad_()
+    assert not ts_oracle.soft_target_tspipe_loss(s, tr, y, 4.0, 0.3, kd_mode="logits").requires_grad
+
+
+def test_distil_loss_clm_and_mse_terms_closed_form():
+    g = seeded(13)
+    bs, seq, V = 2, 5, 7
+    s = torch.randn(bs, seq, V, generator=g, dtype=torch.float64)
+    t = torch.randn(bs, seq, V, generator=g, dtype=torch.float64)
+    lm = torch.full((bs, seq), -100, dtype=torch.long)
+    lm[0, 0], lm[0, 2], lm[1, 4], lm[1, 1] = 5, 3, 6, 0
+    att = torch.tensor([[1, 1, 1, 1, 0], [1, 1, 0, 0, 0]], dtype=torch.bool)
+    sn, tn = s.numpy(), t.numpy()
+    lse = np.log(np.exp(sn).sum(-1))
+    for restrict in (True, False):
+        rows = ((lm > -1) if restrict else att).numpy()
+        kd, _ = _kd_closed_form(sn[rows], tn[rows], 2.0)
+        base = ts_oracle.distil_loss(s, t, None, None, lm, att, 0.5, 0.0, 0.0, 2.0, restrict).item()
+        assert abs(base - 0.5 * kd) < 1e-12
+        # causal LM: the logits at position p are scored against the label at p+1.
+        # Labelled positions: (0,0)->p=-1 (none), (0,2)->p=1, (1,4)->p=3, (1,1)->p=0
+        clm_terms = [lse[0, 1] - sn[0, 1, 3], lse[1, 3] - sn[1, 3, 6], lse[1, 0] - sn[1, 0, 0]]
+        got = ts_oracle.distil_loss(s, t, None, None, lm, att, 0.5, 0.0, 0.0, 2.0, restrict, alpha_clm=1.5).item()
+        assert abs(got - (0.5 * kd + 1.5 * np.mean(clm_terms))) < 1e-12
+        # squared error: summed over the selected rows, divided by their number (not by elements)
+        mse = ((sn[rows] - tn[rows]) ** 2).sum() / rows.sum()
+        got = ts_oracle.distil_loss(s, t, None, None, lm, att, 0.5, 0.0, 0.0, 2.0, restrict, alpha_mse=0.25).item()
+        assert abs(got - (0.5 * kd + 0.25 * mse)) < 1e-12
+

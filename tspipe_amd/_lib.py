@@ -40,6 +40,9 @@ SIGNATURES = {
     "ts_cosine_workspace_bytes": (c_size_t, [c_int64]),
     "ts_cosine_fwd_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_float, c_void_p, c_void_p,
                                   c_void_p, c_int, c_void_p]),
+    "ts_mse_workspace_bytes": (c_size_t, [c_int64, c_int64]),
+    "ts_mse_fwd_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_float, c_int, c_int,
+                               c_void_p, c_void_p, c_void_p, c_int64, c_int, c_void_p]),
     "ts_scale_rows": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_int, c_void_p]),
     "ts_byol_fwd_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_void_p,
                                 c_void_p, c_void_p, c_void_p, c_int, c_void_p]),

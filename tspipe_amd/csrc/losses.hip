@@ -1,6 +1,6 @@
-// Row-wise losses on embedding-sized rows with fused backward (BYOL normalised
-// MSE, cosine embedding) and the small shared reductions.  One 64-wide
-// wavefront owns one row.  All accumulation is fp32; storage is fp32, bf16 or
+// Row-wise losses with fused backward (BYOL normalised MSE and cosine embedding
+// on embedding-sized rows, one 64-wide wavefront per row; squared error
+// between logits) and the small shared reductions.  All accumulation is fp32; storage is fp32, bf16 or
 // fp16.
 #include "common.h"
 
@@ -135,6 +135,97 @@ __global__ __launch_bounds__(256) void cosine_rows_kernel(const T* __restrict__ 
   }
 }
 
+// ---- squared error between logits (fused backward) -----------------------
+//   loss = weight * sum over selected rows, all columns of (s - t)^2 / denom
+//   grad = d loss / d s = (2 weight / denom)(s - t) on selected rows, 0 elsewhere
+// denom = selected rows (x V when the mean runs over elements).  A workgroup
+// owns kMseSpan elements of one row and leaves one partial sum.
+constexpr int kMseBlock = 256;
+constexpr int kMseSpan = 2048;
+
+template <typename T>
+__global__ __launch_bounds__(kMseBlock) void mse_rows_kernel(const T* __restrict__ s, const T* __restrict__ t,
+                                                              const uint8_t* __restrict__ mask,
+                                                              const int* __restrict__ n_sel_dev, int64_t n_rows,
+                                                              int64_t V, int64_t ld_s, int64_t ld_t, int64_t ld_g,
+                                                              float weight, int per_element, int accumulate,
+                                                              float* __restrict__ partial, T* __restrict__ grad) {
+  __shared__ float lds[kMseBlock / kWave];
+  const int64_t parts = gridDim.x;
+  const float rows_sel = n_sel_dev ? (float)(*n_sel_dev) : (float)n_rows;
+  const float denom = per_element ? rows_sel * (float)V : rows_sel;
+  const float k = 2.f * weight / denom;
+  for (int64_t row = blockIdx.y; row < n_rows; row += gridDim.y) {
+    const bool sel = !mask || mask[row] != 0;
+    const int64_t i0 = (int64_t)blockIdx.x * kMseSpan + threadIdx.x;  // consecutive lanes, consecutive elements
+    float acc = 0.f;
+    if (sel) {
+      const T* sr = s + row * ld_s;
+      const T* tr = t + row * ld_t;
+      T* gr = grad ? grad + row * ld_g : nullptr;
+#pragma unroll
+      for (int j = 0; j < kMseSpan / kMseBlock; ++j) {
+        const int64_t i = i0 + j * kMseBlock;
+        if (i < V) {
+          const float d = to_f32(sr[i]) - to_f32(tr[i]);
+          acc += d * d;
+          if (gr) gr[i] = from_f32<T>(accumulate ? to_f32(gr[i]) + k * d : k * d);
+        }
+      }
+    } else if (grad && !accumulate) {
+      T* gr = grad + row * ld_g;
+#pragma unroll
+      for (int j = 0; j < kMseSpan / kMseBlock; ++j)
+        if (i0 + j * kMseBlock < V) gr[i0 + j * kMseBlock] = from_f32<T>(0.f);
+    }
+    const float tot = block_sum<kMseBlock / kWave>(acc, lds);
+    if (threadIdx.x == 0) partial[row * parts + blockIdx.x] = tot;
+    __syncthreads();  // lds is reused by the next row
+  }
+}
+
+// out (+)= weight * sum(partial) / denom, fixed summation order
+__global__ __launch_bounds__(1024) void mse_finalize_kernel(const float* __restrict__ partial, int64_t n,
+                                                            const int* __restrict__ n_sel_dev, int64_t n_rows,
+                                                            int64_t V, float weight, int per_element, int accumulate,
+                                                            float* __restrict__ out) {
+  __shared__ float lds[1024 / kWave];
+  float acc = 0.f;
+  for (int64_t i = threadIdx.x; i < n; i += 1024) acc += partial[i];
+  const float tot = block_sum<1024 / kWave>(acc, lds);
+  if (threadIdx.x == 0) {
+    const float rows_sel = n_sel_dev ? (float)(*n_sel_dev) : (float)n_rows;
+    const float denom = per_element ? rows_sel * (float)V : rows_sel;
+    const float v = weight * (tot / denom);  // 0/0 = NaN for an empty selection, as the reference gives
+    *out = accumulate ? *out + v : v;
+  }
+}
+
+inline int64_t mse_parts(int64_t V) { return (V + kMseSpan - 1) / kMseSpan; }
+
+template <typename T>
+int launch_mse(const void* s, const void* t, const uint8_t* mask, int64_t n_rows, int64_t V, int64_t ld_s,
+               int64_t ld_t, float weight, int per_element, int accumulate, void* ws, float* loss_out, void* grad,
+               int64_t ld_g, hipStream_t stream) {
+  int* n_sel = reinterpret_cast<int*>(ws);
+  float* partial = reinterpret_cast<float*>(reinterpret_cast<char*>(ws) + 16);
+  if (mask) {
+    hipLaunchKernelGGL(mask_count_kernel, dim3(1), dim3(1024), 0, stream, mask, n_rows, n_sel);
+    int rc = check_launch();
+    if (rc) return rc;
+  }
+  const int64_t parts = mse_parts(V);
+  const int64_t gy = n_rows < 65535 ? n_rows : 65535;
+  hipLaunchKernelGGL((mse_rows_kernel<T>), dim3((unsigned)parts, (unsigned)gy), dim3(kMseBlock), 0, stream,
+                     (const T*)s, (const T*)t, mask, mask ? n_sel : (const int*)nullptr, n_rows, V, ld_s, ld_t, ld_g,
+                     weight, per_element, accumulate, partial, (T*)grad);
+  int rc = check_launch();
+  if (rc) return rc;
+  hipLaunchKernelGGL(mse_finalize_kernel, dim3(1), dim3(1024), 0, stream, partial, n_rows * parts,
+                     mask ? n_sel : (const int*)nullptr, n_rows, V, weight, per_element, accumulate, loss_out);
+  return check_launch();
+}
+
 template <typename T>
 int launch_cosine(const void* x, const void* y, const uint8_t* mask, int64_t n, int64_t c, float weight, void* ws,
                   float* loss_out, void* gx, hipStream_t stream) {
@@ -204,6 +295,42 @@ int ts_cosine_fwd_bwd(const void* x, const void* y, const uint8_t* row_mask, int
     case TS_F32: return ts::launch_cosine<float>(x, y, row_mask, n, c, weight, workspace, loss_out, gx, st);
     case TS_BF16: return ts::launch_cosine<ts::bf16_t>(x, y, row_mask, n, c, weight, workspace, loss_out, gx, st);
     default: return ts::launch_cosine<ts::f16_t>(x, y, row_mask, n, c, weight, workspace, loss_out, gx, st);
+  }
+}
+
+
+size_t ts_mse_workspace_bytes(int64_t n_rows, int64_t V) {
+  if (n_rows < 0) n_rows = 0;
+  if (V < 1) V = 1;
+  return (size_t)(16 + ((n_rows * ts::mse_parts(V) * 4 + 15) / 16) * 16);
+}
+
+int ts_mse_fwd_bwd(const void* s, const void* t, const uint8_t* row_mask, int64_t n_rows, int64_t V, int64_t ld_s,
+                   int64_t ld_t, float weight, int per_element, int accumulate, void* workspace, float* loss_out,
+                   void* grad, int64_t ld_g, int dtype, ts_stream_t stream) {
+  if (!s || !t || !workspace || !loss_out) return TS_ERR_ARG;
+  if (n_rows < 0 || V <= 0 || ld_s < V || ld_t < V || (grad && ld_g < V)) return TS_ERR_ARG;
+  if (dtype != TS_F32 && dtype != TS_BF16 && dtype != TS_F16) return TS_ERR_ARG;
+  if (n_rows > (1 << 24) || n_rows * ts::mse_parts(V) > 0x7fffffffLL) return TS_ERR_RANGE;
+  if ((uintptr_t)workspace & 15u) return TS_ERR_ALIGN;
+  const size_t es = ts::dtype_size(dtype);
+  if (((uintptr_t)s | (uintptr_t)t | (uintptr_t)grad) & (es - 1)) return TS_ERR_ALIGN;
+  hipStream_t st = (hipStream_t)stream;
+  if (n_rows == 0) {
+    hipLaunchKernelGGL(ts::mse_finalize_kernel, dim3(1), dim3(1024), 0, st, (const float*)workspace, (int64_t)0,
+                       (const int*)nullptr, (int64_t)0, V, weight, per_element, accumulate, loss_out);
+    return ts::check_launch();
+  }
+  switch (dtype) {
+    case TS_F32:
+      return ts::launch_mse<float>(s, t, row_mask, n_rows, V, ld_s, ld_t, weight, per_element, accumulate, workspace,
+                                   loss_out, grad, ld_g, st);
+    case TS_BF16:
+      return ts::launch_mse<ts::bf16_t>(s, t, row_mask, n_rows, V, ld_s, ld_t, weight, per_element, accumulate,
+                                        workspace, loss_out, grad, ld_g, st);
+    default:
+      return ts::launch_mse<ts::f16_t>(s, t, row_mask, n_rows, V, ld_s, ld_t, weight, per_element, accumulate,
+                                       workspace, loss_out, grad, ld_g, st);
   }
 }
 

@@ -50,11 +50,13 @@ def _scale_saved_grad(grad: Tensor, grad_output: Tensor, rows: int, cols: int) -
 
 class _KDSoftTargetFn(torch.autograd.Function):
     """KD soft-target term, optionally with the hard-label CE term, in one pass
-    over the student logits."""
+    over the student logits; optionally followed by the logits-MSE term over
+    the same rows, added in place to the loss and to the gradient."""
 
     @staticmethod
     def forward(ctx, out_s: Tensor, out_t: Tensor, row_mask: Optional[Tensor], T: float, weight: float,
-                labels: Optional[Tensor] = None, ce_weight: float = 0.0, ignore_index: int = -100):
+                labels: Optional[Tensor] = None, ce_weight: float = 0.0, ignore_index: int = -100,
+                mse_weight: float = 0.0, mse_per_element: bool = False):
         _require_cuda(out_s, out_t, row_mask, labels)
         if out_s.shape != out_t.shape:
             raise ValueError(f"student/teacher logits differ in shape: {tuple(out_s.shape)} vs {tuple(out_t.shape)}")
@@ -97,6 +99,14 @@ class _KDSoftTargetFn(torch.autograd.Function):
                                          loss.data_ptr(), None if grad is None else grad.data_ptr(), V, code,
                                          _lib.current_stream_ptr(dev))
         _lib.check(status, "ts_kdce_fwd_bwd")
+        if mse_weight > 0.0:
+            ws2 = torch.empty(lib.ts_mse_workspace_bytes(rows, V), dtype=torch.uint8, device=dev)
+            with torch.cuda.device(dev):
+                status = lib.ts_mse_fwd_bwd(s.data_ptr(), t.data_ptr(), mask_ptr, rows, V, V, V, float(mse_weight),
+                                            1 if mse_per_element else 0, 1,
+                                            ws2.data_ptr(), loss.data_ptr(), None if grad is None else grad.data_ptr(),
+                                            V, code, _lib.current_stream_ptr(dev))
+            _lib.check(status, "ts_mse_fwd_bwd")
         ctx.grad = grad
         ctx.shape = out_s.shape
         ctx.dims = (rows, V)
@@ -106,10 +116,10 @@ class _KDSoftTargetFn(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_output: Tensor):
         if ctx.grad is None:
-            return (None,) * 8
+            return (None,) * 10
         _once(ctx)
         grad = _scale_saved_grad(ctx.grad, grad_output, *ctx.dims)
-        return (grad.view(ctx.shape),) + (None,) * 7
+        return (grad.view(ctx.shape),) + (None,) * 9
 
 
 def kd_soft_target_loss(out_s: Tensor, out_t: Tensor, T: float, weight: float = 1.0,
@@ -144,15 +154,82 @@ def distil_ce_loss(s_logits: Tensor, t_logits: Tensor, row_mask: Tensor, tempera
     return _KDSoftTargetFn.apply(s_logits, t_logits, row_mask, float(temperature), float(alpha_ce))
 
 
-def kd_ce_loss(out_s: Tensor, out_t: Tensor, labels: Tensor, T: float, kd_weight: float = 1.0,
-               ce_weight: float = 1.0, row_mask: Optional[Tensor] = None, ignore_index: int = -100) -> Tensor:
+def kd_ce_loss(out_s: Tensor, out_t: Tensor, labels: Optional[Tensor], T: float, kd_weight: float = 1.0,
+               ce_weight: float = 1.0, row_mask: Optional[Tensor] = None, ignore_index: int = -100,
+               mse_weight: float = 0.0, mse_per_element: bool = False) -> Tensor:
     """``kd_weight * T^2 * KL(...)`` over the rows of ``row_mask`` plus
     ``ce_weight * CrossEntropy(out_s, labels)`` over the rows whose label is not
     ``ignore_index``, both means over their own row sets, in one pass over the
     logits (benchmarks/soft_target/train_kd.py:439-453;
-    benchmarks/distilbert/distiller.py:719-744)."""
-    return _KDSoftTargetFn.apply(out_s, out_t, row_mask, float(T), float(kd_weight), labels, float(ce_weight),
-                                 int(ignore_index))
+    benchmarks/distilbert/distiller.py:719-744).  ``labels=None`` drops the CE
+    term.  ``mse_weight > 0`` adds ``mse_weight * sum((out_s - out_t)^2) / rows``
+    over the rows of ``row_mask`` (distiller.py:751-755; divided by the number
+    of elements instead with ``mse_per_element``, as ``F.mse_loss`` does),
+    accumulated into the same gradient buffer."""
+    return _KDSoftTargetFn.apply(out_s, out_t, row_mask, float(T), float(kd_weight), labels,
+                                 float(ce_weight) if labels is not None else 0.0, int(ignore_index),
+                                 float(mse_weight), bool(mse_per_element))
+
+
+class _LogitsMSEFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, out_s: Tensor, out_t: Tensor, row_mask: Optional[Tensor], weight: float, per_element: bool):
+        _require_cuda(out_s, out_t, row_mask)
+        if out_s.shape != out_t.shape or out_s.dtype != out_t.dtype:
+            raise ValueError("MSE inputs must agree in shape and dtype")
+        V = int(out_s.shape[-1])
+        s = out_s.detach().reshape(-1, V)
+        t = out_t.detach().reshape(-1, V)
+        s = s if s.is_contiguous() else s.contiguous()
+        t = t if t.is_contiguous() else t.contiguous()
+        rows = int(s.shape[0])
+        mask_ptr = None
+        if row_mask is not None:
+            m = row_mask.detach().reshape(-1)
+            if m.numel() != rows:
+                raise ValueError(f"row mask has {m.numel()} entries for {rows} rows")
+            if m.dtype != torch.bool:
+                m = m != 0
+            m = m.contiguous().view(torch.uint8)
+            mask_ptr = m.data_ptr()
+        lib = _lib.lib()
+        dev = s.device
+        ws = torch.empty(lib.ts_mse_workspace_bytes(rows, V), dtype=torch.uint8, device=dev)
+        loss = torch.empty((), dtype=torch.float32, device=dev)
+        grad = torch.empty_like(s) if ctx.needs_input_grad[0] else None
+        with torch.cuda.device(dev):
+            status = lib.ts_mse_fwd_bwd(s.data_ptr(), t.data_ptr(), mask_ptr, rows, V, V, V, float(weight),
+                                        1 if per_element else 0, 0, ws.data_ptr(), loss.data_ptr(),
+                                        None if grad is None else grad.data_ptr(), V, _lib.dtype_code(s.dtype),
+                                        _lib.current_stream_ptr(dev))
+        _lib.check(status, "ts_mse_fwd_bwd")
+        ctx.grad, ctx.shape, ctx.dims = grad, out_s.shape, (rows, V)
+        ctx.backward_done = False
+        return loss
+
+    @staticmethod
+    def backward(ctx, grad_output: Tensor):
+        if ctx.grad is None:
+            return (None,) * 5
+        _once(ctx)
+        return (_scale_saved_grad(ctx.grad, grad_output, *ctx.dims).view(ctx.shape),) + (None,) * 4
+
+
+def logits_mse_loss(out_s: Tensor, out_t: Tensor, row_mask: Optional[Tensor] = None, weight: float = 1.0,
+                    per_element: bool = True) -> Tensor:
+    """Squared error between student and teacher logits.  ``per_element=True``
+    is ``F.mse_loss(out_s, out_t)`` (benchmarks/soft_target/kd_losses/logits.py:17-20);
+    ``per_element=False`` with a ``[bs, seq]`` mask is DistilBERT's
+    ``MSELoss(reduction="sum")(s_slct, t_slct) / s_slct.size(0)``
+    (benchmarks/distilbert/distiller.py:751-755)."""
+    return _LogitsMSEFn.apply(out_s, out_t, row_mask, float(weight), bool(per_element))
+
+
+class Logits(nn.Module):
+    """Drop-in for benchmarks/soft_target/kd_losses/logits.py:9-20."""
+
+    def forward(self, out_s: Tensor, out_t: Tensor) -> Tensor:
+        return logits_mse_loss(out_s, out_t)
 
 
 class _CosineFn(torch.autograd.Function):
@@ -336,34 +413,47 @@ def moco_contrastive_loss(online_view_1, online_view_2, target_view_1, target_vi
 
 def soft_target_tspipe_loss(model_out: Tensor, ema_model_out: Tensor, label: Tensor, tspipe_args, args,
                             epoch: int) -> Tensor:
-    """``tspipe_loss`` of benchmarks/soft_target/train_kd.py:439-453 for
-    ``args.kd_mode == 'st'``: hard-label cross entropy plus ``lambda_kd`` times
-    the soft-target KD term, both in one kernel pass."""
-    if getattr(args, "kd_mode", "st") != "st":
-        raise NotImplementedError("only kd_mode='st' runs on the fused kernel (kd_mode='logits' is a plain MSE)")
-    return kd_ce_loss(model_out, ema_model_out.detach(), label, args.T, kd_weight=args.lambda_kd, ce_weight=1.0)
+    """``tspipe_loss`` of benchmarks/soft_target/train_kd.py:439-453: hard-label
+    cross entropy plus ``lambda_kd`` times the KD criterion -- the soft-target
+    KL for ``args.kd_mode == 'st'`` (both in one kernel pass), the logits MSE
+    for ``'logits'``."""
+    mode = getattr(args, "kd_mode", "st")
+    if mode == "st":
+        return kd_ce_loss(model_out, ema_model_out.detach(), label, args.T, kd_weight=args.lambda_kd, ce_weight=1.0)
+    if mode == "logits":
+        return kd_ce_loss(model_out, ema_model_out.detach(), label, 1.0, kd_weight=0.0, ce_weight=1.0,
+                          mse_weight=args.lambda_kd, mse_per_element=True)
+    raise AssertionError(f"kd_mode {mode!r}: the reference knows 'st' and 'logits'")
 
 
 def distil_loss_fn(student_outputs, teacher_outputs, labels, tspipe_args, params, epoch: int) -> Tensor:
     """``TSPipeDistiller.loss_fn`` of benchmarks/distilbert/distiller.py:711-772:
-    ``alpha_ce`` x masked KD, ``alpha_mlm`` x masked-LM cross entropy
-    (ignore_index -100) -- both in one pass over the logits -- and ``alpha_cos``
-    x cosine embedding loss on the last hidden states.  ``params`` carries
+    ``alpha_ce`` x masked KD, ``alpha_mlm`` x masked-LM cross entropy or
+    ``alpha_clm`` x causal-LM cross entropy (ignore_index -100) -- both in one
+    pass over the logits -- ``alpha_mse`` x squared error of the selected
+    logits, and ``alpha_cos`` x cosine embedding loss on the last hidden states.  ``params`` carries
     ``alpha_ce, alpha_mlm, alpha_clm, alpha_mse, alpha_cos, temperature,
     restrict_ce_to_mask`` like the reference's LossComputeParam."""
     s_logits, t_logits = student_outputs["logits"], teacher_outputs["logits"]
     lm_labels, attention_mask = labels
-    if getattr(params, "alpha_clm", 0.0) > 0.0:
-        raise NotImplementedError("the causal-LM term (alpha_clm) is not on the fused path")
-    if getattr(params, "alpha_mse", 0.0) > 0.0:
-        raise NotImplementedError("the logits-MSE term (alpha_mse) is not on the fused path")
-    mask = (lm_labels > -1) if params.restrict_ce_to_mask else attention_mask
     alpha_mlm = float(getattr(params, "alpha_mlm", 0.0))
+    alpha_clm = float(getattr(params, "alpha_clm", 0.0))
+    alpha_mse = float(getattr(params, "alpha_mse", 0.0))
+    if alpha_mlm > 0.0 and alpha_clm > 0.0:
+        # the reference's own sanity check forbids it (benchmarks/distilbert/train.py:50)
+        raise NotImplementedError("alpha_mlm and alpha_clm are mutually exclusive")
+    mask = (lm_labels > -1) if params.restrict_ce_to_mask else attention_mask
+    ce_labels, ce_weight = None, 0.0
     if alpha_mlm > 0.0:
-        loss = kd_ce_loss(s_logits, t_logits, lm_labels, params.temperature, kd_weight=params.alpha_ce,
-                          ce_weight=alpha_mlm, row_mask=mask, ignore_index=-100)
-    else:
-        loss = distil_ce_loss(s_logits, t_logits, mask, params.temperature, params.alpha_ce)
+        ce_labels, ce_weight = lm_labels, alpha_mlm
+    elif alpha_clm > 0.0:
+        # logits at position p are scored against the label at p+1; the last
+        # position of every sequence has no target (distiller.py:745-749)
+        ce_labels = torch.full_like(lm_labels, -100)
+        ce_labels[..., :-1] = lm_labels[..., 1:]
+        ce_weight = alpha_clm
+    loss = kd_ce_loss(s_logits, t_logits, ce_labels, params.temperature, kd_weight=params.alpha_ce,
+                      ce_weight=ce_weight, row_mask=mask, ignore_index=-100, mse_weight=alpha_mse)
     if getattr(params, "alpha_cos", 0.0) > 0.0:
         s_hid = student_outputs["hidden_states"][-1]
         t_hid = teacher_outputs["hidden_states"][-1]
