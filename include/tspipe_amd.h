@@ -181,6 +181,24 @@ int ts_kdce_fwd_bwd(const void* s, const void* t, const uint8_t* row_mask, const
                     float inv_T, float kd_scale, float ce_weight, void* workspace, float* loss_out,
                     void* grad, int64_t ld_g, int dtype, ts_stream_t stream);
 
+/* The same loss on logits that were never concatenated: the student and teacher
+ * outputs of up to 8 micro-batches stay where the pipeline produced them
+ * (tspipe/gpu_task.py:147,170-171,188-191 concatenates them with torch.cat
+ * before calling loss_fn; this entry point makes both copies unnecessary) and
+ * the gradient is written straight into one buffer per piece.
+ *   s_pieces, t_pieces, grad_pieces: host arrays of n_pieces device pointers,
+ *     piece p being a contiguous [piece_rows[p], V] matrix; grad_pieces may be
+ *     NULL (or hold NULLs) for loss only;
+ *   row_mask, labels: device arrays over the rows of all pieces in order
+ *     (sum of piece_rows entries), as for ts_kdce_fwd_bwd; either may be NULL.
+ * workspace: ts_kd_workspace_bytes(sum of piece_rows, V, dtype).  More than 8
+ * pieces: TS_ERR_RANGE (gather first, or call once per group of pieces). */
+int ts_kdce_pieces_fwd_bwd(const void* const* s_pieces, const void* const* t_pieces,
+                           void* const* grad_pieces, const int64_t* piece_rows, int n_pieces,
+                           const uint8_t* row_mask, const int64_t* labels, int64_t ignore_index,
+                           int64_t V, float inv_T, float kd_scale, float ce_weight,
+                           void* workspace, float* loss_out, int dtype, ts_stream_t stream);
+
 /* grad *= *g for the rows the loss touched; returns at once on the device
  * when *g == 1 (the only value TSPipe's torch.autograd.backward(loss) feeds,
  * tspipe/gpu_task.py:207-212).  g_dev: one float in device memory. */

@@ -402,6 +402,87 @@ def test_logits_mse_and_kd_mode_logits(device, rows, V, dtype):
     assert ((sd3.grad.cpu().double() - gw).abs() <= tol * peak + slack).all()
 
 
+@pytest.mark.parametrize("rows,V,dtype,with_ce", [((64, 64, 64, 64), 100, torch.float32, True),
+                                                  ((5, 1, 9, 2, 7, 3, 4, 6), 1000, torch.float32, False),
+                                                  ((8, 8, 8, 5), 30522, torch.bfloat16, True),
+                                                  ((3,), 6000, torch.bfloat16, False)])
+def test_kd_pieces_equal_gathered(device, rows, V, dtype, with_ce):
+    # micro-batch outputs that are never concatenated: same loss and gradient
+    # as the kernel on the gathered tensors, bit for bit (same arithmetic, only
+    # the row addresses differ; the shapes here keep every row at the same
+    # 16-byte phase in both layouts, so even the summation order is the same),
+    # and within the usual bar of the oracle
+    g = seeded(250 + V)
+    s_p = [(torch.randn(r, V, generator=g) * 2).to(dtype) for r in rows]
+    t_p = [(torch.randn(r, V, generator=g) * 2).to(dtype) for r in rows]
+    total = sum(rows)
+    mask = torch.rand(total, generator=g) < 0.5
+    labels = None
+    if with_ce:
+        labels = torch.randint(0, V, (total,), generator=g)
+        labels[torch.rand(total, generator=g) < 0.4] = -100
+    sd = [p.to(device).requires_grad_() for p in s_p]
+    td = [p.to(device) for p in t_p]
+    lab_d = None if labels is None else labels.to(device)
+    loss = ta.kd_ce_loss_pieces(sd, td, lab_d, 2.0, kd_weight=0.5, ce_weight=1.5, row_mask=mask.to(device))
+    loss.backward()
+    s_cat = torch.cat([p.to(device) for p in s_p]).requires_grad_()
+    ref = ta.kd_ce_loss(s_cat, torch.cat(td), lab_d, 2.0, kd_weight=0.5, ce_weight=1.5, row_mask=mask.to(device))
+    ref.backward()
+    assert loss.item() == ref.item()
+    assert torch.equal(torch.cat([p.grad for p in sd]), s_cat.grad)
+
+    def oracle(a, b):
+        out = ts_oracle.distil_ce(a, b, mask, 2.0, 0.5)
+        if labels is not None:
+            out = out + 1.5 * torch.nn.CrossEntropyLoss(ignore_index=-100)(a, labels)
+        return out
+    want, (gw,) = _oracle_grad(oracle, torch.cat(s_p), others=(torch.cat(t_p),))
+    tol = 1e-5 if dtype == torch.float32 else 1e-3
+    assert rel_err(loss.item(), want) < tol
+    got = torch.cat([p.grad for p in sd]).cpu().double()
+    slack = gw.abs() * (2.0 ** -8 if dtype != torch.float32 else 0.0)
+    assert ((got - gw).abs() <= tol * gw.abs().max().item() + slack).all()
+
+
+def test_distil_loss_fn_pieces_matches_gathered_plugin(device):
+    from argparse import Namespace
+    g = seeded(260)
+    chunks, bs, seq, V, H = 4, 2, 16, 30522, 32
+    s = [(torch.randn(bs, seq, V, generator=g) * 2).to(torch.bfloat16).to(device).requires_grad_() for _ in range(chunks)]
+    t = [(torch.randn(bs, seq, V, generator=g) * 2).to(torch.bfloat16).to(device) for _ in range(chunks)]
+    sh = [torch.randn(bs, seq, H, generator=g).to(torch.bfloat16).to(device).requires_grad_() for _ in range(chunks)]
+    th = [torch.randn(bs, seq, H, generator=g).to(torch.bfloat16).to(device) for _ in range(chunks)]
+    lm = torch.full((chunks * bs, seq), -100, dtype=torch.long)
+    pick = torch.rand(chunks * bs, seq, generator=g) < 0.15
+    lm[pick] = torch.randint(0, V, (int(pick.sum()),), generator=g)
+    att = torch.rand(chunks * bs, seq, generator=g) < 0.8
+    params = Namespace(alpha_ce=0.5, alpha_mlm=2.0, alpha_clm=0.0, alpha_mse=0.0, alpha_cos=1.0, temperature=2.0,
+                       restrict_ce_to_mask=True)
+    labels = (lm.to(device), att.to(device))
+    loss = ta.distil_loss_fn_pieces([{"logits": a, "hidden_states": (b,)} for a, b in zip(s, sh)],
+                                    [{"logits": a, "hidden_states": (b,)} for a, b in zip(t, th)], labels, None, params, 0)
+    loss.backward()
+    s_cat = torch.cat([p.detach() for p in s]).requires_grad_()
+    sh_cat = torch.cat([p.detach() for p in sh]).requires_grad_()
+    ref = ta.distil_loss_fn({"logits": s_cat, "hidden_states": (sh_cat,)},
+                            {"logits": torch.cat(t), "hidden_states": (torch.cat(th),)}, labels, None, params, 0)
+    ref.backward()
+    assert loss.item() == ref.item()
+    assert torch.equal(torch.cat([p.grad for p in s]), s_cat.grad)
+    assert torch.equal(torch.cat([p.grad for p in sh]), sh_cat.grad)
+
+
+def test_kd_pieces_argument_errors(device):
+    s = [torch.randn(4, 10, device=device) for _ in range(9)]
+    with pytest.raises(Exception):
+        ta.kd_ce_loss_pieces(s, s, None, 2.0)  # more than 8 pieces
+    with pytest.raises(ValueError):
+        ta.kd_ce_loss_pieces(s[:2], s[:3], None, 2.0)
+    with pytest.raises(ValueError):
+        ta.kd_ce_loss_pieces(s[:2], s[:2], None, 2.0, row_mask=torch.ones(7, dtype=torch.bool, device=device))
+
+
 def test_kd_masked_cfg3_full_size_properties(device):
     # [32, 128, 30522] bf16, 15 % token mask, gathered from 4 micro-batches: too large for the
     # fp64 oracle, so checked through properties that do not depend on the size

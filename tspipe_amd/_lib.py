@@ -37,6 +37,8 @@ SIGNATURES = {
                               c_float, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_void_p]),
     "ts_kdce_fwd_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64,
                                 c_float, c_float, c_float, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_void_p]),
+    "ts_kdce_pieces_fwd_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int64, c_int64,
+                                       c_float, c_float, c_float, c_void_p, c_void_p, c_int, c_void_p]),
     "ts_cosine_workspace_bytes": (c_size_t, [c_int64]),
     "ts_cosine_fwd_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_float, c_void_p, c_void_p,
                                   c_void_p, c_int, c_void_p]),

@@ -105,6 +105,12 @@ __device__ __forceinline__ void store16(T* p, const Vec16<T>& v) {
 }
 
 // Everything a row kernel needs; passed by value.
+// The logits may come as up to kKdMaxPieces row blocks (micro-batch outputs
+// that were never concatenated): piece p holds rows piece_row0[p] ..
+// piece_row0[p+1]-1 of the batch, contiguous with the common leading
+// dimensions.  n_pieces == 0 means the single matrices s / t / grad.
+constexpr int kKdMaxPieces = 8;
+
 struct KdArgs {
   const void* s;
   const void* t;
@@ -119,7 +125,51 @@ struct KdArgs {
   float* row_kd;      // per-row KD loss terms (0 for unselected rows)
   float* row_ce;      // per-row CE loss terms
   void* grad;         // may be null
+  int n_pieces;
+  int64_t piece_row0[kKdMaxPieces];
+  const void* s_piece[kKdMaxPieces];
+  const void* t_piece[kKdMaxPieces];
+  void* g_piece[kKdMaxPieces];  // all null or all set
 };
+
+// Row pointers.  The piece is found with a chain of selects rather than an
+// indexed load, because a wavefront may hold several rows.
+template <typename T>
+struct KdRowPtrs {
+  const T* s;
+  const T* t;
+  T* g;
+};
+
+template <typename T>
+__device__ __forceinline__ KdRowPtrs<T> kd_row_ptrs(const KdArgs& a, int64_t row) {
+  KdRowPtrs<T> r;
+  if (a.n_pieces == 0) {
+    r.s = reinterpret_cast<const T*>(a.s) + row * a.ld_s;
+    r.t = reinterpret_cast<const T*>(a.t) + row * a.ld_t;
+    r.g = a.grad ? reinterpret_cast<T*>(a.grad) + row * a.ld_g : nullptr;
+    return r;
+  }
+  const void* sb = a.s_piece[0];
+  const void* tb = a.t_piece[0];
+  void* gb = a.g_piece[0];
+  int64_t r0 = 0;
+#pragma unroll
+  for (int i = 1; i < kKdMaxPieces; ++i) {
+    const bool ge = i < a.n_pieces && row >= a.piece_row0[i];
+    sb = ge ? a.s_piece[i] : sb;
+    tb = ge ? a.t_piece[i] : tb;
+    gb = ge ? a.g_piece[i] : gb;
+    r0 = ge ? a.piece_row0[i] : r0;
+  }
+  const int64_t local = row - r0;
+  r.s = reinterpret_cast<const T*>(sb) + local * a.ld_s;
+  r.t = reinterpret_cast<const T*>(tb) + local * a.ld_t;
+  r.g = gb ? reinterpret_cast<T*>(gb) + local * a.ld_g : nullptr;
+  return r;
+}
+
+__device__ __forceinline__ bool kd_has_grad(const KdArgs& a) { return a.n_pieces ? a.g_piece[0] != nullptr : a.grad != nullptr; }
 
 struct RowJob {
   bool kd, ce;
@@ -228,9 +278,10 @@ __global__ __launch_bounds__(BLOCK) void kd_rows_kernel(const KdArgs a) {
   // exits below are uniform; smaller groups never reach a __syncthreads and
   // only shuffle among their own lanes.
   if (row >= a.n_rows) return;
-  const T* srow = reinterpret_cast<const T*>(a.s) + row * a.ld_s;
-  const T* trow = reinterpret_cast<const T*>(a.t) + row * a.ld_t;
-  T* grow = a.grad ? reinterpret_cast<T*>(a.grad) + row * a.ld_g : nullptr;
+  const KdRowPtrs<T> rp = kd_row_ptrs<T>(a, row);
+  const T* srow = rp.s;
+  const T* trow = rp.t;
+  T* grow = rp.g;
   const RowJob job = row_job(a, row);
   const int64_t V = a.V;
 
@@ -357,8 +408,8 @@ __global__ __launch_bounds__(kPartBlock) void kd_wide_pass1_kernel(const KdArgs 
       a.row_kd[row] = 0.f;
       if (CE) a.row_ce[row] = 0.f;
     }
-    if (!a.grad) return;
-    T* grow = reinterpret_cast<T*>(a.grad) + row * a.ld_g;
+    if (!kd_has_grad(a)) return;
+    T* grow = kd_row_ptrs<T>(a, row).g;
     const uint32_t mis = (uint32_t)((uintptr_t)grow & 15u);
     int64_t head = (int64_t)(((16u - mis) & 15u) / sizeof(T));
     if (head > V) head = V;
@@ -379,8 +430,9 @@ __global__ __launch_bounds__(kPartBlock) void kd_wide_pass1_kernel(const KdArgs 
     return;
   }
 
-  const T* srow = reinterpret_cast<const T*>(a.s) + row * a.ld_s;
-  const T* trow = reinterpret_cast<const T*>(a.t) + row * a.ld_t;
+  const KdRowPtrs<T> rp = kd_row_ptrs<T>(a, row);
+  const T* srow = rp.s;
+  const T* trow = rp.t;
   // the row is cut by the alignment of s and t alone; pass 2 cuts it the same way
   const RowGeom g = row_geom<T>(srow, trow, nullptr, V);
   Vec16<T> rt[kPartPerThread], rs[kPartPerThread];
@@ -484,9 +536,10 @@ __global__ __launch_bounds__(kPartBlock) void kd_wide_pass2_kernel(const KdArgs 
     const int64_t row = sel_rows ? (int64_t)sel_rows[item / parts] : item / parts;
     const int part = (int)(item % parts);
     const int64_t v0 = (int64_t)part * kPartVecs;
-    const T* srow = reinterpret_cast<const T*>(a.s) + row * a.ld_s;
-    const T* trow = reinterpret_cast<const T*>(a.t) + row * a.ld_t;
-    T* grow = a.grad ? reinterpret_cast<T*>(a.grad) + row * a.ld_g : nullptr;
+    const KdRowPtrs<T> rp = kd_row_ptrs<T>(a, row);
+    const T* srow = rp.s;
+    const T* trow = rp.t;
+    T* grow = rp.g;
     const RowJob job = row_job(a, row);
     const RowGeom g = row_geom<T>(srow, trow, nullptr, V);
     const bool gvec = grow && (((uintptr_t)grow & 15u) == ((uintptr_t)srow & 15u));
@@ -755,6 +808,63 @@ int ts_kdce_fwd_bwd(const void* s, const void* t, const uint8_t* row_mask, const
   a.counts = nullptr;
   a.row_kd = a.row_ce = nullptr;
   a.grad = grad;
+  a.n_pieces = 0;
+  for (int i = 0; i < ts::kKdMaxPieces; ++i) {
+    a.piece_row0[i] = 0;
+    a.s_piece[i] = a.t_piece[i] = nullptr;
+    a.g_piece[i] = nullptr;
+  }
+  hipStream_t st = (hipStream_t)stream;
+  switch (dtype) {
+    case TS_F32: return ts::launch_kd<float>(a, kd_scale, workspace, loss_out, st);
+    case TS_BF16: return ts::launch_kd<ts::bf16_t>(a, kd_scale, workspace, loss_out, st);
+    default: return ts::launch_kd<ts::f16_t>(a, kd_scale, workspace, loss_out, st);
+  }
+}
+
+int ts_kdce_pieces_fwd_bwd(const void* const* s_pieces, const void* const* t_pieces, void* const* grad_pieces,
+                           const int64_t* piece_rows, int n_pieces, const uint8_t* row_mask, const int64_t* labels,
+                           int64_t ignore_index, int64_t V, float inv_T, float kd_scale, float ce_weight,
+                           void* workspace, float* loss_out, int dtype, ts_stream_t stream) {
+  if (!s_pieces || !t_pieces || !piece_rows || !workspace || !loss_out) return TS_ERR_ARG;
+  if (n_pieces < 1 || n_pieces > ts::kKdMaxPieces) return TS_ERR_RANGE;
+  if (V <= 0 || !(inv_T > 0.f)) return TS_ERR_ARG;
+  if (dtype != TS_F32 && dtype != TS_BF16 && dtype != TS_F16) return TS_ERR_ARG;
+  const uintptr_t esz = (dtype == TS_F32) ? 4 : 2;
+  ts::KdArgs a;
+  a.s = a.t = nullptr;
+  a.grad = nullptr;
+  int64_t rows = 0;
+  const bool want_grad = grad_pieces && grad_pieces[0];
+  for (int i = 0; i < ts::kKdMaxPieces; ++i) {
+    a.piece_row0[i] = rows;
+    a.s_piece[i] = a.t_piece[i] = nullptr;
+    a.g_piece[i] = nullptr;
+    if (i >= n_pieces) continue;
+    if (piece_rows[i] <= 0 || !s_pieces[i] || !t_pieces[i]) return TS_ERR_ARG;
+    if (want_grad != (grad_pieces && grad_pieces[i] != nullptr)) return TS_ERR_ARG;
+    void* g = want_grad ? grad_pieces[i] : nullptr;
+    if (((uintptr_t)s_pieces[i] | (uintptr_t)t_pieces[i] | (uintptr_t)g) & (esz - 1)) return TS_ERR_ALIGN;
+    a.s_piece[i] = s_pieces[i];
+    a.t_piece[i] = t_pieces[i];
+    a.g_piece[i] = g;
+    rows += piece_rows[i];
+  }
+  if (rows > (1 << 24)) return TS_ERR_RANGE;
+  if ((uintptr_t)labels & 7u) return TS_ERR_ALIGN;
+  if ((uintptr_t)workspace & 31u) return TS_ERR_ALIGN;
+  a.n_pieces = n_pieces;
+  a.mask = row_mask;
+  a.labels = labels;
+  a.ignore_index = ignore_index;
+  a.n_rows = rows;
+  a.V = V;
+  a.ld_s = a.ld_t = a.ld_g = V;
+  a.k = inv_T * ts::kLog2e;
+  a.kd_gscale = kd_scale * inv_T;
+  a.ce_weight = ce_weight;
+  a.counts = nullptr;
+  a.row_kd = a.row_ce = nullptr;
   hipStream_t st = (hipStream_t)stream;
   switch (dtype) {
     case TS_F32: return ts::launch_kd<float>(a, kd_scale, workspace, loss_out, st);

@@ -171,6 +171,90 @@ def kd_ce_loss(out_s: Tensor, out_t: Tensor, labels: Optional[Tensor], T: float,
                                  float(mse_weight), bool(mse_per_element))
 
 
+class _KDPiecesFn(torch.autograd.Function):
+    """The KD (+ CE) loss on micro-batch outputs that were never concatenated:
+    the kernels read every piece where it lies and write one gradient buffer
+    per student piece."""
+
+    @staticmethod
+    def forward(ctx, n: int, row_mask: Optional[Tensor], labels: Optional[Tensor], T: float, weight: float,
+                ce_weight: float, ignore_index: int, *pieces: Tensor):
+        import ctypes
+        s_pieces, t_pieces = pieces[:n], pieces[n:]
+        _require_cuda(row_mask, labels, *pieces)
+        V = int(s_pieces[0].shape[-1])
+        dtype, dev = s_pieces[0].dtype, s_pieces[0].device
+        s_flat, t_flat, rows = [], [], []
+        for sp, tp in zip(s_pieces, t_pieces):
+            if sp.shape != tp.shape or sp.dtype != dtype or tp.dtype != dtype or int(sp.shape[-1]) != V:
+                raise ValueError("student/teacher pieces must agree in shape, dtype and class count")
+            s2, t2 = sp.detach().reshape(-1, V), tp.detach().reshape(-1, V)
+            s_flat.append(s2 if s2.is_contiguous() else s2.contiguous())
+            t_flat.append(t2 if t2.is_contiguous() else t2.contiguous())
+            rows.append(int(s2.shape[0]))
+        total = sum(rows)
+        mask_ptr = label_ptr = None
+        if row_mask is not None:
+            m = row_mask.detach().reshape(-1)
+            if m.numel() != total:
+                raise ValueError(f"row mask has {m.numel()} entries for {total} rows")
+            if m.dtype != torch.bool:
+                m = m != 0
+            m = m.contiguous().view(torch.uint8)
+            mask_ptr = m.data_ptr()
+        if labels is not None:
+            lab = labels.detach().reshape(-1)
+            if lab.numel() != total:
+                raise ValueError(f"{lab.numel()} labels for {total} rows")
+            lab = (lab if lab.dtype == torch.int64 else lab.to(torch.int64)).contiguous()
+            label_ptr = lab.data_ptr()
+        need = [ctx.needs_input_grad[7 + i] for i in range(n)]
+        grads = [torch.empty_like(s2) for s2 in s_flat] if any(need) else None
+        lib = _lib.lib()
+        code = _lib.dtype_code(dtype)
+        ws = torch.empty(lib.ts_kd_workspace_bytes(total, V, code), dtype=torch.uint8, device=dev)
+        loss = torch.empty((), dtype=torch.float32, device=dev)
+        ptrs = lambda ts: (ctypes.c_void_p * n)(*[t.data_ptr() for t in ts])
+        with torch.cuda.device(dev):
+            status = lib.ts_kdce_pieces_fwd_bwd(ptrs(s_flat), ptrs(t_flat), None if grads is None else ptrs(grads),
+                                                (ctypes.c_int64 * n)(*rows), n, mask_ptr, label_ptr, int(ignore_index),
+                                                V, 1.0 / T, T * T * weight, float(ce_weight), ws.data_ptr(),
+                                                loss.data_ptr(), code, _lib.current_stream_ptr(dev))
+        _lib.check(status, "ts_kdce_pieces_fwd_bwd")
+        ctx.grads, ctx.need, ctx.n = grads, need, n
+        ctx.shapes = [sp.shape for sp in s_pieces]
+        ctx.dims = [(r, V) for r in rows]
+        ctx.backward_done = False
+        return loss
+
+    @staticmethod
+    def backward(ctx, grad_output: Tensor):
+        none7 = (None,) * 7
+        if ctx.grads is None:
+            return none7 + (None,) * (2 * ctx.n)
+        _once(ctx)
+        outs = []
+        for g, need, shape, dims in zip(ctx.grads, ctx.need, ctx.shapes, ctx.dims):
+            outs.append(_scale_saved_grad(g, grad_output, *dims).view(shape) if need else None)
+        return none7 + tuple(outs) + (None,) * ctx.n
+
+
+def kd_ce_loss_pieces(s_pieces, t_pieces, labels: Optional[Tensor], T: float, kd_weight: float = 1.0,
+                      ce_weight: float = 1.0, row_mask: Optional[Tensor] = None, ignore_index: int = -100) -> Tensor:
+    """``kd_ce_loss`` on lists of micro-batch outputs (split along dim 0) that
+    were never concatenated: same value as
+    ``kd_ce_loss(torch.cat(s_pieces), torch.cat(t_pieces), ...)`` without either
+    copy (the pipeline's gather at tspipe/gpu_task.py:147,170-171,188-191), and
+    the gradient arrives per piece.  ``labels`` and ``row_mask`` cover the whole
+    batch.  Up to 8 pieces per call."""
+    s_pieces, t_pieces = list(s_pieces), list(t_pieces)
+    if len(s_pieces) != len(t_pieces) or not s_pieces:
+        raise ValueError("need as many teacher pieces as student pieces, at least one")
+    n = len(s_pieces)
+    return _KDPiecesFn.apply(n, row_mask, labels, float(T), float(kd_weight),
+                             float(ce_weight) if labels is not None else 0.0, int(ignore_index), *s_pieces, *t_pieces)
+
+
 class _LogitsMSEFn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, out_s: Tensor, out_t: Tensor, row_mask: Optional[Tensor], weight: float, per_element: bool):
@@ -459,3 +543,38 @@ def distil_loss_fn(student_outputs, teacher_outputs, labels, tspipe_args, params
         t_hid = teacher_outputs["hidden_states"][-1]
         loss = loss + cosine_embedding_loss(s_hid, t_hid, attention_mask, params.alpha_cos)
     return loss
+
+
+def distil_loss_fn_pieces(student_pieces, teacher_pieces, labels, tspipe_args, params, epoch: int) -> Tensor:
+    """``distil_loss_fn`` for a pipeline that hands over the per-micro-batch
+    output dicts instead of gathering them first (tspipe/gpu_task.py:147,
+    170-171, 188-191 is where the reference concatenates).  The logits, by far
+    the largest tensors, are read in place by ``kd_ce_loss_pieces``; the hidden
+    states of the cosine term are small and go through ``gather``.  ``labels``
+    is the whole batch's ``(lm_labels, attention_mask)`` as in ``distil_loss_fn``.
+    The ``alpha_mse`` term has no piece-wise kernel: use ``distil_loss_fn``."""
+    from .batch_ops import Batch, gather
+    lm_labels, attention_mask = labels
+    alpha_mlm = float(getattr(params, "alpha_mlm", 0.0))
+    alpha_clm = float(getattr(params, "alpha_clm", 0.0))
+    if float(getattr(params, "alpha_mse", 0.0)) > 0.0:
+        raise NotImplementedError("alpha_mse needs the gathered logits: call distil_loss_fn")
+    if alpha_mlm > 0.0 and alpha_clm > 0.0:
+        raise NotImplementedError("alpha_mlm and alpha_clm are mutually exclusive")
+    mask = (lm_labels > -1) if params.restrict_ce_to_mask else attention_mask
+    ce_labels, ce_weight = None, 0.0
+    if alpha_mlm > 0.0:
+        ce_labels, ce_weight = lm_labels, alpha_mlm
+    elif alpha_clm > 0.0:
+        ce_labels = torch.full_like(lm_labels, -100)
+        ce_labels[..., :-1] = lm_labels[..., 1:]
+        ce_weight = alpha_clm
+    loss = kd_ce_loss_pieces([p["logits"] for p in student_pieces], [p["logits"] for p in teacher_pieces], ce_labels,
+                             params.temperature, kd_weight=params.alpha_ce, ce_weight=ce_weight, row_mask=mask,
+                             ignore_index=-100)
+    if getattr(params, "alpha_cos", 0.0) > 0.0:
+        s_hid = gather([Batch(p["hidden_states"][-1]) for p in student_pieces])
+        t_hid = gather([Batch(p["hidden_states"][-1]) for p in teacher_pieces])
+        loss = loss + cosine_embedding_loss(s_hid, t_hid, attention_mask, params.alpha_cos)
+    return loss
+
