@@ -168,3 +168,24 @@ def test_product_refuses_host_tensors():
         ta.DeferredBatchNorm(3)(torch.zeros(2, 3, 4))
     with pytest.raises(ValueError):
         ta.DeferredBatchNorm(3)(torch.zeros(2, 3))  # fewer than 3 dims: the reference's own check
+
+
+def test_bind_params_repoints_without_copy():
+    import tspipe_amd as ta
+    model = torch.nn.Sequential(torch.nn.Linear(4, 3), torch.nn.Linear(3, 2))
+    params = list(model.parameters())
+    ids = [id(p) for p in params]
+    version = [torch.randn_like(p) for p in params]
+    ta.bind_params_(model.parameters(), version)
+    assert [id(p) for p in model.parameters()] == ids          # same Parameter objects
+    for p, v in zip(model.parameters(), version):
+        assert p.data_ptr() == v.data_ptr() and p.requires_grad  # aliasing the version, still trainable leaves
+        assert torch.equal(p, v)
+    x = torch.randn(5, 4)
+    want = torch.nn.functional.linear(torch.nn.functional.linear(x, version[0], version[1]), version[2], version[3])
+    assert torch.equal(model(x), want)
+    with pytest.raises(ValueError):
+        ta.bind_params_(model.parameters(), version[:-1])
+    with pytest.raises(ValueError):
+        ta.bind_params_(model.parameters(), [v.double() for v in version])
+

@@ -337,3 +337,27 @@ def copy_params_(dst_params: Iterable[torch.Tensor], src_params: Iterable[torch.
         return
     with torch.cuda.device(dsts[0].device):
         _tables.copy_segments([s for s, _ in live], [d for _, d in live])
+
+
+@torch.no_grad()
+def bind_params_(params: Iterable[torch.Tensor], version: Iterable[torch.Tensor]) -> None:
+    """Makes a stored parameter version the live one without moving a byte:
+    every parameter is re-pointed at the version's tensor (``p.data = new``),
+    where tspipe/gpu_task.py:721-723 copies it (``p.copy_(new)``, one launch per
+    tensor).  The ``nn.Parameter`` objects, and so the module and any state
+    keyed by them, stay the same.
+
+    The live parameters then *alias* the stored version, so this is for
+    parameters nobody updates in place: the momentum teacher, whose every new
+    version is a fresh list from ``update_target_fn``.  The student's optimizer
+    steps in place and needs ``copy_params_``."""
+    ps, vs = list(params), list(version)
+    if len(ps) != len(vs):
+        raise ValueError(f"{len(ps)} parameters but {len(vs)} tensors in the version")
+    for p, v in zip(ps, vs):
+        if p.shape != v.shape or p.dtype != v.dtype or p.device != v.device:
+            raise ValueError(f"version tensor {tuple(v.shape)}/{v.dtype}/{v.device} does not fit parameter "
+                             f"{tuple(p.shape)}/{p.dtype}/{p.device}")
+    for p, v in zip(ps, vs):
+        p.data = v.detach()
+
