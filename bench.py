@@ -128,12 +128,28 @@ def run_step_benchmark(steps, warmup, dev):
     avg_ema_ms = sum(ema_ms) / len(ema_ms)
     algo_bytes = 12 * n_params
     achieved = algo_bytes / (avg_ema_ms * 1e-3) / 1e9
+    # the same launches with nothing else on the GPU (the figure above shares
+    # HBM and the CUs with the loss kernels of the other stream)
+    _lib.prepare_timing_events(dev, 30)
+    torch.cuda.synchronize()
+    ema_mod.kernel_events = alone = []
+    with torch.cuda.stream(s_ema):
+        for _ in range(30):
+            state["teacher"] = ta.calculate_updated_momentum_encoder(0.99, student, state["teacher"])
+    torch.cuda.synchronize()
+    ema_mod.kernel_events = None
+    alone_ms = sum(_event_ms(alone)) / len(alone)
+    alone_gbs = algo_bytes / (alone_ms * 1e-3) / 1e9
     return {
         "elapsed": elapsed, "n_params": n_params, "loss": float(state["loss"].item()),
         "roofline": {"bound": "hbm", "kernel": "ema_multi_kernel", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": EMA_VITB_TRAFFIC_BYTES, "algorithmic_bytes_per_launch": algo_bytes,
-                     "avg_kernel_ms": round(avg_ema_ms, 4), "launches_timed": len(ema_ms)},
+                     "avg_kernel_ms": round(avg_ema_ms, 4), "launches_timed": len(ema_ms),
+                     "note": "inside the timed region the kernel shares the GPU with the InfoNCE stream; 'alone' is "
+                             "the same launch with the other stream idle",
+                     "alone": {"achieved": round(alone_gbs, 1), "frac": round(alone_gbs / HBM_PEAK_GBS, 4),
+                               "avg_kernel_ms": round(alone_ms, 4), "launches_timed": len(alone)}},
     }
 
 

@@ -182,9 +182,11 @@ _pool_lock = threading.Lock()
 
 def release_pool() -> None:
     """Drops every cached output arena (memory returns to torch's allocator
-    once the caller's own references are gone)."""
+    once the caller's own references are gone) and the calling thread's
+    cached chunk tables."""
     with _pool_lock:
         _pool.clear()
+    _tables.clear_table_cache()
 
 
 def _acquire_arena(teachers: Sequence[torch.Tensor], shapes) -> _Arena:
