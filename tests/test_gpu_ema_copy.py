@@ -225,3 +225,31 @@ def test_clone_and_update_fused(device, shapes):
     new_t2 = ta.momentum_update(0.996, clones2, t_dev)
     assert all(bits_equal(a, b) for a, b in zip(new_t, new_t2))
     ema_mod.release_pool()
+
+
+def test_generic_gather_of_a_nested_structure_is_one_launch(device):
+    # DistilBERT-like micro-batch outputs: a dict with logits and a tuple of hidden states
+    from tspipe_amd import _tables
+    g = seeded(31)
+    full = {"logits": torch.randn(12, 7, 33, generator=g).to(torch.bfloat16),
+            "hidden_states": tuple(torch.randn(12, 7, 16, generator=g) for _ in range(3)),
+            "note": "x"}
+    pieces = ta.generic_scatter({k: (v.to(device) if torch.is_tensor(v) else
+                                     tuple(h.to(device) for h in v) if isinstance(v, tuple) else v)
+                                 for k, v in full.items()}, 4)
+    _tables.kernel_events = []
+    try:
+        back = ta.generic_gather(pieces)
+        launches = len(_tables.kernel_events)
+    finally:
+        _tables.kernel_events = None
+    assert launches == 1
+    want = ts_oracle.generic_object_gather(*ts_oracle.generic_object_scatter(full, 4))
+    assert bits_equal(back["logits"].cpu(), want["logits"])
+    assert all(bits_equal(a.cpu(), b) for a, b in zip(back["hidden_states"], want["hidden_states"]))
+    assert back["note"] == "x" and type(back) is dict
+    # the structure checks still come first, before anything is launched
+    bad = [p.value for p in pieces]
+    bad[1] = dict(bad[1], note="y")
+    with pytest.raises(ValueError):
+        ta.generic_object_gather(*bad)

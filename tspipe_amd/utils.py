@@ -67,9 +67,24 @@ def generic_object_scatter(obj: Any, chunks: int) -> Any:
     return split(obj)
 
 
+class _Pending:
+    """Stand-in for a tensor leaf whose concatenation is still to be launched."""
+    __slots__ = ("index",)
+
+    def __init__(self, index: int):
+        self.index = index
+
+
 def generic_object_gather(*objs: Any) -> Any:
-    """Merges structures produced by ``generic_object_scatter`` (utils.py:256-292)."""
-    from .batch_ops import concat_dim0
+    """Merges structures produced by ``generic_object_scatter`` (utils.py:256-292).
+
+    The structure is walked first (all type, key and value checks happen
+    there, in the reference's order), the tensor leaves are only collected;
+    then every leaf of the whole structure is concatenated by ONE copy launch
+    and the results are put in place."""
+    from . import batch_ops
+
+    groups = []
 
     def keys_agree(first, others):
         for other in others:
@@ -92,12 +107,29 @@ def generic_object_gather(*objs: Any) -> Any:
                       for group in zip(*(x.items() for x in items)))
             return OrderedDict(merged) if isinstance(head, OrderedDict) else dict(merged)
         if isinstance(head, Tensor):
-            return concat_dim0(items)
+            groups.append(items)
+            return _Pending(len(groups) - 1)
         if any(head != x for x in items):
             raise ValueError(f"Value of given objects must match: {items}")
         return head
 
+    def resolve(node, done):
+        if isinstance(node, _Pending):
+            return done[node.index]
+        if isinstance(node, list):
+            return [resolve(x, done) for x in node]
+        if isinstance(node, tuple):
+            return tuple(resolve(x, done) for x in node)
+        if isinstance(node, dict):
+            return type(node)((k, resolve(v, done)) for k, v in node.items())
+        return node
+
+    def finish(tree):
+        if not groups:
+            return tree
+        return resolve(tree, batch_ops.concat_groups(groups))
+
     if all(isinstance(o, TSPipeModelOutput) for o in objs):
-        return TSPipeModelOutput(data=merge(*(o.data for o in objs)),
+        return TSPipeModelOutput(data=finish(merge(*(o.data for o in objs))),
                                  lst_require_grad_tensor_path=objs[0].lst_require_grad_tensor_path)
-    return merge(*objs)
+    return finish(merge(*objs))
