@@ -253,3 +253,40 @@ def test_generic_gather_of_a_nested_structure_is_one_launch(device):
     bad[1] = dict(bad[1], note="y")
     with pytest.raises(ValueError):
         ta.generic_object_gather(*bad)
+
+
+def test_ema_and_gather_from_two_threads(device):
+    # TSPipe drives the plug-ins from one worker thread per partition
+    # (tspipe/gpu_worker.py); each thread has its own stream, table ring and
+    # table cache, the output arenas are shared under a lock.
+    import threading
+    shapes = [(64, 3, 7, 7), (64,), (128, 64, 3, 3), (1000, 512), (1000,)]
+    results, errors = {}, []
+
+    def worker(idx):
+        try:
+            torch.cuda.set_device(device)
+            s, t = param_lists(shapes, seed=40 + idx)
+            want = t
+            for _ in range(12):
+                want = ts_oracle.ema_update(0.99, s, want)
+            stream = torch.cuda.Stream(device)
+            with torch.cuda.stream(stream):
+                sd, td = [x.to(device) for x in s], [x.to(device) for x in t]
+                got = td
+                for _ in range(12):
+                    got = ta.calculate_target_network_parameters(0.99, sd, got)
+                cat = ta.gather([ta.Batch(x.reshape(-1, 1)) for x in got])
+            stream.synchronize()
+            results[idx] = (all(bits_equal(a.cpu(), b) for a, b in zip(got, want)),
+                            bits_equal(cat.cpu(), torch.cat([w.reshape(-1, 1) for w in want])))
+        except Exception as e:  # pragma: no cover - reported below
+            errors.append(repr(e))
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(2)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join(timeout=100)
+    assert not errors, errors
+    assert results == {0: (True, True), 1: (True, True)}
