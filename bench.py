@@ -293,12 +293,12 @@ def run_kernel_table(dev):
                                               loss_p.data_ptr(), _lib.TS_BF16, stream), "ts_kdce_pieces_fwd_bwd")
     out["kd_masked_4_pieces_8x128x30522_bf16"] = entry(
         3 * n_sel * row_b + (4096 - n_sel) * row_b, _time_stream(f_pieces, 30),
-        "same loss read from the 4 micro-batch outputs in place: replaces 2 gathers (2 x ~77 us) + the call above", 4)
+        "same loss read from the 4 micro-batch outputs in place: replaces 2 gathers (2 x ~77 us) + the call below", 3)
     del pieces_s, pieces_t, flat_s, flat_t, grads, ws_p
     f = kd_call(s_full, t_full, mask, 2.0, torch.empty_like(s_full))
     out["kd_masked_32x128x30522_bf16"] = entry(3 * n_sel * row_b + (4096 - n_sel) * row_b, _time_stream(f, 30),
                                                f"n_sel={n_sel}; bytes = read s,t + write grad for selected rows, "
-                                               f"zero-fill of the other rows", 4)
+                                               f"zero-fill of the other rows", 3)
     del s_full, t_full, f
 
     # InfoNCE (cfg4), single pair

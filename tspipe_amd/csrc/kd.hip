@@ -390,14 +390,27 @@ struct PartStat {  // 32 bytes
   float mt, zt, at, ms, zs, z1, pad0, pad1;
 };
 
+template <int NT>
+__device__ __forceinline__ void kd_count_block(const KdArgs& a, int* __restrict__ counts, int* __restrict__ sel_rows);
+
+// With count_out set, workgroup 0 does the row counting and compaction that
+// pass 2 and the final reduction need (nothing in pass 1 reads them), and the
+// (row, part) items start at workgroup 1.
 template <typename T, bool CE>
 __global__ __launch_bounds__(kPartBlock) void kd_wide_pass1_kernel(const KdArgs a, int parts,
-                                                                   PartStat* __restrict__ part_stats) {
+                                                                   PartStat* __restrict__ part_stats,
+                                                                   int* __restrict__ count_out,
+                                                                   int* __restrict__ sel_rows_out) {
   constexpr int VEC = Vec16<T>::N;
   __shared__ TStat lds_t[kPartBlock / kWave];
   __shared__ SStat lds_s[kPartBlock / kWave];
-  const int64_t row = blockIdx.x / parts;
-  const int part = (int)(blockIdx.x % parts);
+  if (count_out && blockIdx.x == 0) {
+    kd_count_block<kPartBlock>(a, count_out, sel_rows_out);
+    return;
+  }
+  const int64_t item = (int64_t)blockIdx.x - (count_out ? 1 : 0);
+  const int64_t row = item / parts;
+  const int part = (int)(item % parts);
   const int tid = threadIdx.x;
   const int64_t v0 = (int64_t)part * kPartVecs;
   const int64_t V = a.V;
@@ -602,13 +615,14 @@ inline int64_t kd_parts(int64_t V) {
 // counts[0] = rows with the KD term, counts[1] = rows with the CE term,
 // counts[2] = rows with either; sel_rows (optional) = indices of the latter in
 // ascending order.  One workgroup; thread i owns the i-th contiguous slice.
-__global__ __launch_bounds__(1024) void kd_count_kernel(const KdArgs a, int* __restrict__ counts,
-                                                        int* __restrict__ sel_rows) {
-  __shared__ int scan[1024];
-  __shared__ int tot_kd[1024 / kWave], tot_ce[1024 / kWave];
+template <int NT>
+__device__ __forceinline__ void kd_count_block(const KdArgs& a, int* __restrict__ counts,
+                                               int* __restrict__ sel_rows) {
+  __shared__ int scan[NT];
+  __shared__ int tot_kd[NT / kWave], tot_ce[NT / kWave];
   const int tid = threadIdx.x;
   const int64_t n = a.n_rows;
-  const int64_t per = (n + 1023) / 1024;
+  const int64_t per = (n + NT - 1) / NT;
   const int64_t lo = tid * per, hi = (lo + per < n) ? lo + per : n;
   int c_any = 0, c_kd = 0, c_ce = 0;
   for (int64_t i = lo; i < hi; ++i) {
@@ -625,8 +639,8 @@ __global__ __launch_bounds__(1024) void kd_count_kernel(const KdArgs a, int* __r
   }
   scan[tid] = c_any;
   __syncthreads();
-  // inclusive Hillis-Steele scan over the 1024 per-thread counts
-  for (int off = 1; off < 1024; off <<= 1) {
+  // inclusive Hillis-Steele scan over the per-thread counts
+  for (int off = 1; off < NT; off <<= 1) {
     const int add = (tid >= off) ? scan[tid - off] : 0;
     __syncthreads();
     scan[tid] += add;
@@ -634,13 +648,13 @@ __global__ __launch_bounds__(1024) void kd_count_kernel(const KdArgs a, int* __r
   }
   if (tid == 0) {
     int k = 0, c = 0;
-    for (int i = 0; i < 1024 / kWave; ++i) {
+    for (int i = 0; i < NT / kWave; ++i) {
       k += tot_kd[i];
       c += tot_ce[i];
     }
     counts[0] = k;
     counts[1] = c;
-    counts[2] = scan[1023];
+    counts[2] = scan[NT - 1];
   }
   if (sel_rows) {
     int pos = scan[tid] - c_any;
@@ -649,6 +663,11 @@ __global__ __launch_bounds__(1024) void kd_count_kernel(const KdArgs a, int* __r
       if (j.kd || j.ce) sel_rows[pos++] = (int)i;
     }
   }
+}
+
+__global__ __launch_bounds__(1024) void kd_count_kernel(const KdArgs a, int* __restrict__ counts,
+                                                        int* __restrict__ sel_rows) {
+  kd_count_block<1024>(a, counts, sel_rows);
 }
 
 // loss = kd_scale * sum(row_kd) / counts[0] + ce_weight * sum(row_ce) / counts[1], fixed summation order.
@@ -716,7 +735,9 @@ int launch_kd_t(KdArgs a, float kd_scale, void* ws, float* loss_out, hipStream_t
   a.row_ce = w.row_ce;
   const bool compact = parts && counted;
   int rc = TS_OK;
-  if (counted) {
+  const int64_t vecs_ = (a.V + Vec16<T>::N - 1) / Vec16<T>::N + 1;
+  const bool wide = a.n_rows > 0 && parts > 0 && vecs_ > 64 * 4;
+  if (counted && !wide) {
     hipLaunchKernelGGL(kd_count_kernel, dim3(1), dim3(1024), 0, stream, a, w.counts,
                        compact ? w.sel_rows : (int*)nullptr);
     rc = check_launch();
@@ -744,8 +765,9 @@ int launch_kd_t(KdArgs a, float kd_scale, void* ws, float* loss_out, hipStream_t
   } else {
     const int64_t items = a.n_rows * parts;
     if (items > 0x7fffffffLL) return TS_ERR_RANGE;
-    hipLaunchKernelGGL((kd_wide_pass1_kernel<T, CE>), dim3((unsigned)items), dim3(kPartBlock), 0, stream, a,
-                       (int)parts, w.part_stats);
+    hipLaunchKernelGGL((kd_wide_pass1_kernel<T, CE>), dim3((unsigned)(items + (counted ? 1 : 0))), dim3(kPartBlock),
+                       0, stream, a, (int)parts, w.part_stats, counted ? w.counts : (int*)nullptr,
+                       (counted && compact) ? w.sel_rows : (int*)nullptr);
     rc = check_launch();
     if (rc) return rc;
     const int64_t grid2 = items < kPass2MaxGrid ? items : kPass2MaxGrid;
