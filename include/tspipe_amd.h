@@ -309,6 +309,19 @@ int ts_bn_apply(const float* x, float* y, const float* mean, const float* invstd
                 const float* gamma, const float* beta, int64_t N, int64_t C, int64_t HW,
                 int is_var, float eps, ts_stream_t stream);
 
+/* Training forward of one micro-batch in two launches instead of three:
+ * ts_bn_stats + ts_bn_apply(training) with the bookkeeping of the statistics
+ * folded into the normalising kernel (tspipe/batchnorm.py:45-59 and 111-120
+ * together).  Same results as the two calls, bit for bit.
+ *   ws: 4*C floats, zero before the first call, owned by the layer: two
+ *       halves used alternately.  parity (0/1) selects the half this call
+ *       reduces into; it must alternate from call to call on the same ws
+ *       (the call clears the half the previous call used).
+ *   sum, sum_squares, ub_mean, ub_invstd: as for ts_bn_stats (any may be NULL). */
+int ts_bn_forward_train(const float* x, float* y, const float* gamma, const float* beta, int64_t N,
+                        int64_t C, int64_t HW, float* sum, float* sum_squares, float* ub_mean,
+                        float* ub_invstd, float* ws, int parity, float eps, ts_stream_t stream);
+
 /* Backward of the normalisation (what autograd derives for F.batch_norm):
  * dgamma = sum dy*xhat, dbeta = sum dy, and
  *   training != 0 (batch statistics, batchnorm.py:111-120):

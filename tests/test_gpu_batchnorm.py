@@ -16,6 +16,17 @@ from oracle import ts_oracle
 pytestmark = pytest.mark.gpu
 
 
+
+def _check_workspace(bn):
+    # the shared reduction area (backward, stand-alone statistics) is left
+    # clean; of the two halves the training forward alternates between, the
+    # one the NEXT call will reduce into is zero
+    c = bn.num_features
+    ws = bn._ws.cpu()
+    assert (ws[:2 * c] == 0).all()
+    nxt = 2 * c + bn._parity * 2 * c
+    assert (ws[nxt:nxt + 2 * c] == 0).all()
+
 def _rel(a, b):
     a, b = a.detach().cpu().double(), b.detach().cpu().double()
     return ((a - b).abs() / b.abs().clamp_min(1e-30)).max().item()
@@ -51,7 +62,7 @@ def test_deferred_bn_matches_oracle(device, shape, chunks):
         assert _rel(bn.running_mean, ora.running_mean) < 1e-6 or (ora.running_mean == 0).all()
         assert _rel(bn.running_var, ora.running_var) < 1e-6
         assert int(bn.num_batches_tracked) == int(ora.num_batches_tracked)
-    assert (bn._ws == 0).all()  # reduction workspace is left clean
+    _check_workspace(bn)
 
 
 def test_deferred_bn_cfg5_shape(device):
@@ -123,7 +134,7 @@ def test_deferred_bn_backward(device):
     assert max_rel_to_peak(xd.grad, x64.grad) < 1e-5
     assert max_rel_to_peak(bn.weight.grad, w64.grad) < 1e-5
     assert max_rel_to_peak(bn.bias.grad, b64.grad) < 1e-5
-    assert (bn._ws == 0).all()
+    _check_workspace(bn)
 
 
 def test_deferred_bn_eval_mode_and_momentum_none(device):
@@ -167,3 +178,37 @@ def test_deferred_bn_module_contract(device):
     conv = conv.to(device)
     out = conv(torch.randn(2, 3, 8, 8, device=device))
     assert out.shape == (2, 4, 6, 6)
+
+
+def test_fused_training_forward_equals_the_two_calls(device):
+    # ts_bn_forward_train against ts_bn_stats + ts_bn_apply through the C ABI: bit for bit,
+    # over several calls so that both workspace halves are used and cleared
+    from tspipe_amd import _lib
+    lib = _lib.lib()
+    st = torch.cuda.current_stream(device).cuda_stream
+    N, C, H, W = 6, 10, 9, 7
+    g = seeded(77)
+    z = lambda n: torch.zeros(n, device=device)  # noqa: E731
+    gamma, beta = torch.rand(C, generator=g).to(device) + 0.5, torch.randn(C, generator=g).to(device)
+    ws2, ws4 = z(2 * C), z(4 * C)
+    sum_a, sq_a, sum_b, sq_b = z(C), z(C), z(C), z(C)
+    for call in range(5):
+        x = (torch.randn(N, C, H, W, generator=g) * 1.5 + 0.5).to(device)
+        ya, yb = torch.empty_like(x), torch.empty_like(x)
+        mean_a, inv_a, mean_b, inv_b = z(C), z(C), z(C), z(C)
+        _lib.check(lib.ts_bn_stats(x.data_ptr(), N, C, H * W, ws2.data_ptr(), sum_a.data_ptr(), sq_a.data_ptr(),
+                                   mean_a.data_ptr(), inv_a.data_ptr(), 1e-5, st), "ts_bn_stats")
+        _lib.check(lib.ts_bn_apply(x.data_ptr(), ya.data_ptr(), mean_a.data_ptr(), inv_a.data_ptr(), gamma.data_ptr(),
+                                   beta.data_ptr(), N, C, H * W, 0, 1e-5, st), "ts_bn_apply")
+        _lib.check(lib.ts_bn_forward_train(x.data_ptr(), yb.data_ptr(), gamma.data_ptr(), beta.data_ptr(), N, C, H * W,
+                                           sum_b.data_ptr(), sq_b.data_ptr(), mean_b.data_ptr(), inv_b.data_ptr(),
+                                           ws4.data_ptr(), call % 2, 1e-5, st), "ts_bn_forward_train")
+        torch.cuda.synchronize()
+        assert torch.equal(ya, yb)
+        assert torch.equal(mean_a, mean_b) and torch.equal(inv_a, inv_b)
+        assert torch.equal(sum_a, sum_b) and torch.equal(sq_a, sq_b)
+        half = ws4.view(2, 2 * C)
+        assert (half[1 - call % 2] == 0).all() and (half[call % 2] != 0).any()
+    assert lib.ts_bn_forward_train(x.data_ptr(), yb.data_ptr(), None, None, N, C, H * W, None, None, None, None,
+                                   ws4.data_ptr(), 2, 1e-5, st) == -1
+

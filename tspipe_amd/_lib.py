@@ -57,6 +57,8 @@ SIGNATURES = {
                              c_double, c_void_p]),
     "ts_bn_apply": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64,
                             c_int64, c_int, c_float, c_void_p]),
+    "ts_bn_forward_train": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p,
+                                    c_void_p, c_void_p, c_void_p, c_int, c_float, c_void_p]),
     "ts_bn_backward": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p]),
 }

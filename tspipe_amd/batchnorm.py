@@ -91,6 +91,38 @@ class _NormalizeFn(torch.autograd.Function):
                 None, None, None, None, None)
 
 
+class _TrainForwardFn(torch.autograd.Function):
+    """Training forward of one micro-batch: statistics, their bookkeeping in
+    the layer's accumulators and the normalisation in two launches
+    (``ts_bn_forward_train``); backward as for ``_NormalizeFn``."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias, layer: "DeferredBatchNorm"):
+        n, c, hw = _dims(x)
+        y = torch.empty_like(x)
+        mean = torch.empty(c, dtype=torch.float32, device=x.device)
+        invstd = torch.empty(c, dtype=torch.float32, device=x.device)
+        ws = layer._workspace(x)
+        parity = layer._parity
+        layer._parity = 1 - parity
+        with torch.cuda.device(x.device):
+            status = _lib.lib().ts_bn_forward_train(
+                x.data_ptr(), y.data_ptr(), _ptr(weight), _ptr(bias), n, c, hw, layer.sum.data_ptr(),
+                layer.sum_squares.data_ptr(), mean.data_ptr(), invstd.data_ptr(), ws.data_ptr() + 8 * c, parity,
+                float(layer.eps), _lib.current_stream_ptr(x.device))
+        _lib.check(status, "ts_bn_forward_train")
+        ctx.save_for_backward(x, weight, mean, invstd)
+        ctx.ws = ws
+        ctx.training = True
+        ctx.eps = float(layer.eps)
+        ctx.has_bias = bias is not None
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        return _NormalizeFn.backward(ctx, dy)[:3] + (None,)
+
+
 class DeferredBatchNorm(_BatchNorm):
     """A BatchNorm layer that tracks several micro-batches before it updates
     its running statistics (tspipe/batchnorm.py:17-120)."""
@@ -103,9 +135,12 @@ class DeferredBatchNorm(_BatchNorm):
         super().__init__(num_features, eps, momentum, affine, track_running_stats=True)
         self.register_buffer("sum", torch.zeros_like(self.running_mean))
         self.register_buffer("sum_squares", torch.zeros_like(self.running_var))
-        # reduction workspace of the kernels (zero between calls); not part of
-        # the state dict
-        self.register_buffer("_ws", torch.zeros(2 * num_features), persistent=False)
+        # reduction workspace of the kernels, not part of the state dict: 2C
+        # floats that are zero between calls (backward, stand-alone statistics)
+        # and two halves of 2C floats that the training forward alternates
+        # between (``_parity`` says which one the next call reduces into)
+        self.register_buffer("_ws", torch.zeros(6 * num_features), persistent=False)
+        self._parity = 0
         self.counter = 0
         self.tracked = 0
         self.chunks = chunks
@@ -115,8 +150,9 @@ class DeferredBatchNorm(_BatchNorm):
             raise ValueError("expected at least 3D input (got %dD input)" % input.dim())
 
     def _workspace(self, x: Tensor) -> Tensor:
-        if self._ws.device != x.device or self._ws.numel() != 2 * self.num_features:
-            self._ws = torch.zeros(2 * self.num_features, dtype=torch.float32, device=x.device)
+        if self._ws.device != x.device or self._ws.numel() != 6 * self.num_features:
+            self._ws = torch.zeros(6 * self.num_features, dtype=torch.float32, device=x.device)
+            self._parity = 0
         return self._ws
 
     def _stats(self, x: Tensor, accumulate: bool):
@@ -172,11 +208,15 @@ class DeferredBatchNorm(_BatchNorm):
             return _NormalizeFn.apply(x, weight, bias, self.running_mean, self.running_var,
                                       self._workspace(x), False, float(self.eps))
 
-        if self._track(x):
+        # statistics of this micro-batch into the accumulators
+        # (tspipe/batchnorm.py:45-59) and its normalisation (111-120), fused;
+        # the commit (61-85) follows once ``chunks`` micro-batches are in
+        y = _TrainForwardFn.apply(x, weight, bias, self)
+        self.counter += input.size().numel() // input.size(1)
+        self.tracked += 1
+        if self.tracked == self.chunks:
             self._commit()
-        mean, invstd = self._last_stats
-        self._last_stats = None
-        return _NormalizeFn.apply(x, weight, bias, mean, invstd, self._workspace(x), True, float(self.eps))
+        return y
 
     @classmethod
     def convert_deferred_batch_norm(cls, module: TModule, chunks: int = 1) -> TModule:

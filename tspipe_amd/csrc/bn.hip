@@ -181,20 +181,12 @@ __global__ __launch_bounds__(256) void bn_commit_kernel(float* __restrict__ sum,
 
 __global__ void bn_bump_counter_kernel(int64_t* nbt) { *nbt += 1; }
 
-__global__ __launch_bounds__(kBnBlock) void bn_apply_kernel(const float* __restrict__ x, float* __restrict__ y,
-                                                            const float* __restrict__ mean,
-                                                            const float* __restrict__ invstd_or_var,
-                                                            const float* __restrict__ gamma,
-                                                            const float* __restrict__ beta, int64_t N,
-                                                            int64_t C, int64_t HW, int64_t slab, int is_var,
-                                                            float eps) {
-  const int64_t c = blockIdx.y;
+// y = (x - mu) * a + b over this workgroup's slab of channel c
+__device__ __forceinline__ void bn_apply_slab(const float* __restrict__ x, float* __restrict__ y, int64_t N,
+                                              int64_t C, int64_t HW, int64_t slab, int64_t c, float mu, float a,
+                                              float b) {
   const int64_t n0 = (int64_t)blockIdx.x * slab;
   const int64_t n1 = (n0 + slab < N) ? n0 + slab : N;
-  const float mu = mean[c];
-  const float istd = is_var ? 1.f / sqrtf(invstd_or_var[c] + eps) : invstd_or_var[c];
-  const float a = gamma ? istd * gamma[c] : istd;
-  const float b = beta ? beta[c] : 0.f;
   const int tid = threadIdx.x;
   for (int64_t n = n0; n < n1; ++n) {
     const int64_t off = (n * C + c) * HW;
@@ -236,6 +228,55 @@ __global__ __launch_bounds__(kBnBlock) void bn_apply_kernel(const float* __restr
     const int64_t it = sp.tail0 + tid;
     if (it < HW) py[it] = (px[it] - mu) * a + b;
   }
+}
+
+__global__ __launch_bounds__(kBnBlock) void bn_apply_kernel(const float* __restrict__ x, float* __restrict__ y,
+                                                            const float* __restrict__ mean,
+                                                            const float* __restrict__ invstd_or_var,
+                                                            const float* __restrict__ gamma,
+                                                            const float* __restrict__ beta, int64_t N,
+                                                            int64_t C, int64_t HW, int64_t slab, int is_var,
+                                                            float eps) {
+  const int64_t c = blockIdx.y;
+  const float mu = mean[c];
+  const float istd = is_var ? 1.f / sqrtf(invstd_or_var[c] + eps) : invstd_or_var[c];
+  const float a = gamma ? istd * gamma[c] : istd;
+  const float b = beta ? beta[c] : 0.f;
+  bn_apply_slab(x, y, N, C, HW, slab, c, mu, a, b);
+}
+
+// Training forward, second launch: normalises with the micro-batch statistics
+// that bn_stats_kernel left in `ws_in` (every workgroup derives mean and
+// 1/std of its channel from the two sums itself), and the first workgroup of
+// each channel does what bn_stats_finalize_kernel does -- running sums,
+// saved statistics -- except that it clears the OTHER workspace half: this
+// one is still being read by the channel's other workgroups, the other one
+// was consumed by the previous call.
+__global__ __launch_bounds__(kBnBlock) void bn_apply_train_kernel(const float* __restrict__ x, float* __restrict__ y,
+                                                                  const float* __restrict__ gamma,
+                                                                  const float* __restrict__ beta, int64_t N,
+                                                                  int64_t C, int64_t HW, int64_t slab, float cnt,
+                                                                  float eps, const float* __restrict__ ws_in,
+                                                                  float* __restrict__ ws_clear, float* sum,
+                                                                  float* sum_squares, float* ub_mean,
+                                                                  float* ub_invstd) {
+  const int64_t c = blockIdx.y;
+  const float S = ws_in[c], Q = ws_in[C + c];
+  const float k = x[c * HW];
+  const float dm = S / cnt;  // mean - k
+  const float mu = k + dm;
+  const float istd = 1.f / sqrtf(fmaxf(Q / cnt - dm * dm, 0.f) + eps);
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    if (sum) sum[c] += S + cnt * k;
+    if (sum_squares) sum_squares[c] += Q + 2.f * k * S + cnt * k * k;
+    if (ub_mean) ub_mean[c] = mu;
+    if (ub_invstd) ub_invstd[c] = istd;
+    ws_clear[c] = 0.f;
+    ws_clear[C + c] = 0.f;
+  }
+  const float a = gamma ? istd * gamma[c] : istd;
+  const float b = beta ? beta[c] : 0.f;
+  bn_apply_slab(x, y, N, C, HW, slab, c, mu, a, b);
 }
 
 // Backward, level 1: per-channel sum(dy) and sum(dy * xhat) into ws.
@@ -409,6 +450,26 @@ int ts_bn_apply(const float* x, float* y, const float* mean, const float* invstd
   dim3 grid((unsigned)((N + slab - 1) / slab), (unsigned)C);
   hipLaunchKernelGGL(ts::bn_apply_kernel, grid, dim3(ts::kBnBlock), 0, (hipStream_t)stream, x, y, mean,
                      invstd_or_var, gamma, beta, N, C, HW, slab, is_var, eps);
+  return ts::check_launch();
+}
+
+int ts_bn_forward_train(const float* x, float* y, const float* gamma, const float* beta, int64_t N, int64_t C,
+                        int64_t HW, float* sum, float* sum_squares, float* ub_mean, float* ub_invstd, float* ws,
+                        int parity, float eps, ts_stream_t stream) {
+  if (!x || !y || !ws || (parity != 0 && parity != 1)) return TS_ERR_ARG;
+  int rc = ts::bn_check_dims(N, C, HW);
+  if (rc) return rc;
+  if (((uintptr_t)x | (uintptr_t)y) & 3u) return TS_ERR_ALIGN;
+  const int64_t slab = ts::bn_slab(N, HW);
+  dim3 grid((unsigned)((N + slab - 1) / slab), (unsigned)C);
+  hipStream_t st = (hipStream_t)stream;
+  float* ws_now = ws + (int64_t)parity * 2 * C;
+  float* ws_other = ws + (int64_t)(1 - parity) * 2 * C;
+  hipLaunchKernelGGL(ts::bn_stats_kernel, grid, dim3(ts::kBnBlock), 0, st, x, N, C, HW, slab, ws_now);
+  rc = ts::check_launch();
+  if (rc) return rc;
+  hipLaunchKernelGGL(ts::bn_apply_train_kernel, grid, dim3(ts::kBnBlock), 0, st, x, y, gamma, beta, N, C, HW, slab,
+                     (float)((double)N * (double)HW), eps, ws_now, ws_other, sum, sum_squares, ub_mean, ub_invstd);
   return ts::check_launch();
 }
 
