@@ -69,6 +69,25 @@ def build_host(verbose: bool = False) -> str:
     return final
 
 
+CONSUMER_SRC = os.path.join(os.path.dirname(HERE), "tests", "cabi", "consumer.cpp")
+CONSUMER_BIN = os.path.join(os.path.dirname(HERE), "tests", "cabi", "build", "consumer")
+
+
+def build_consumer(verbose: bool = False) -> str:
+    """Builds the stand-alone C++ consumer of the C ABI (tests/cabi): host code
+    only, linked against the library with an rpath, no Python or torch."""
+    os.makedirs(os.path.dirname(CONSUMER_BIN), exist_ok=True)
+    cmd = [HIPCC, "-O2", "-std=c++17", "-Wall", "--offload-arch=gfx950", CONSUMER_SRC, "-o", CONSUMER_BIN,
+           "-L" + HERE, "-ltspipe_amd", "-Wl,-rpath,$ORIGIN/../../../tspipe_amd"]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"building the C-ABI consumer failed:\n{res.stderr}")
+    if verbose:
+        print(f"built {CONSUMER_BIN}")
+    return CONSUMER_BIN
+
+
 if __name__ == "__main__":
     build()
     build_host()
+    build_consumer()
