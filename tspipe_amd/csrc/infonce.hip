@@ -482,17 +482,46 @@ __global__ __launch_bounds__(kNceBlock) void nce_combine_kernel(NceArgs args, in
   const int64_t row = tile32 * 32 + col;
   const bool live = row < n;
 
-  float l = 0.f, A = 0.f;
-  for (int s = 0; s < splits; ++s) {
-    l += lpart[(int64_t)s * npad + row];
-    A += apart[(int64_t)s * npad + row];
+  // The kernel is bound by memory latency, not by arithmetic: every load whose
+  // address is known up front is issued before the first use of any of them
+  // (the row sums, the k and q values of this lane, the first four splits of
+  // the partial O^T).
+  const int64_t qk_row = live ? row : 0;  // padded rows read row 0 and discard it
+  T kv[4][4], qv[4][4];
+  if (dq) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int f0 = 32 * fb + 8 * g + 4 * h;  // this lane holds features f0 .. f0+3 of its row
+      __builtin_memcpy(kv[g], k + qk_row * C + f0, sizeof(kv[g]));
+      __builtin_memcpy(qv[g], q + qk_row * C + f0, sizeof(qv[g]));
+    }
   }
   const float d = diag[row];
+  const float rq_i = rq[row], rk_i = rk[row];
+  float l = 0.f, A = 0.f;
+  {
+    int s = 0;
+    for (; s + 4 <= splits; s += 4) {
+      float lv[4], av[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        lv[u] = lpart[(int64_t)(s + u) * npad + row];
+        av[u] = apart[(int64_t)(s + u) * npad + row];
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        l += lv[u];
+        A += av[u];
+      }
+    }
+    for (; s < splits; ++s) {
+      l += lpart[(int64_t)s * npad + row];
+      A += apart[(int64_t)s * npad + row];
+    }
+  }
   if (fb == 0 && h == 0) row_loss[row] = live ? kNceLn2 * (scale2 + log2f(l) - d) : 0.f;
   if (!dq) return;
 
-  // all loads of four splits are issued before the first add: the kernel is
-  // bound by memory latency, not by arithmetic
   float o[16];
 #pragma unroll
   for (int i = 0; i < 16; ++i) o[i] = 0.f;
@@ -523,21 +552,18 @@ __global__ __launch_bounds__(kNceBlock) void nce_combine_kernel(NceArgs args, in
   }
   if (!live) return;
   const float inv_l = 1.f / l;
-  const float rq_i = rq[row], rk_i = rk[row];
   const float gn = 2.f / (float)n;
   // below eps the norm is the constant eps and normalize() is linear: no projection
   const bool clamped = rq_i >= 1.f / kNormEps;
   const float dot = clamped ? 0.f : gn * (A * inv_l - d) / scale2;
 #pragma unroll
   for (int g = 0; g < 4; ++g) {
-    const int f0 = 32 * fb + 8 * g + 4 * h;  // this lane holds features f0 .. f0+3 of its row
-    T kv[4], qv[4], out[4];
-    __builtin_memcpy(kv, k + row * C + f0, sizeof(kv));
-    __builtin_memcpy(qv, q + row * C + f0, sizeof(qv));
+    const int f0 = 32 * fb + 8 * g + 4 * h;
+    T out[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const float dqh = gn * (o[4 * g + j] * inv_l - to_f32(kv[j]) * rk_i);
-      out[j] = from_f32<T>((dqh - to_f32(qv[j]) * rq_i * dot) * rq_i);
+      const float dqh = gn * (o[4 * g + j] * inv_l - to_f32(kv[g][j]) * rk_i);
+      out[j] = from_f32<T>((dqh - to_f32(qv[g][j]) * rq_i * dot) * rq_i);
     }
     __builtin_memcpy(dq + row * C + f0, out, sizeof(out));
   }
