@@ -152,24 +152,34 @@ __global__ __launch_bounds__(kNceBlock) void nce_prep_kernel(NceArgs args, int64
   const int sub = lane / P::LPR, li = lane % P::LPR;  // row within the pass, lane within the row
   const int64_t row0 = (int64_t)blockIdx.x * P::ROWS;
 
-  for (int r = w * P::RPP + sub; r < P::ROWS; r += 4 * P::RPP) {
+  // the loads of all of this wavefront's rows go out before any is used
+  constexpr int NP = P::ROWS / (4 * P::RPP);  // passes (rows per lane group)
+  static_assert(NP >= 1 && NP * 4 * P::RPP == P::ROWS, "rows divide evenly among the wavefronts");
+  u32x4 rawq[NP], rawk[NP];
+#pragma unroll
+  for (int pass = 0; pass < NP; ++pass) {
+    const int64_t row = row0 + w * P::RPP + sub + pass * 4 * P::RPP;
+    rawq[pass] = rawk[pass] = u32x4{0u, 0u, 0u, 0u};  // zero rows beyond n (0.0 in every dtype)
+    if (row < n) {
+      rawq[pass] = *reinterpret_cast<const u32x4*>(q + row * C + li * P::VEC);
+      rawk[pass] = *reinterpret_cast<const u32x4*>(k + row * C + li * P::VEC);
+    }
+  }
+#pragma unroll
+  for (int pass = 0; pass < NP; ++pass) {
+    const int r = w * P::RPP + sub + pass * 4 * P::RPP;
     const int64_t row = row0 + r;
     const bool live = row < n;
     float qv[P::VEC], kv[P::VEC];
-    if (live) {
-      u32x4 rawq = *reinterpret_cast<const u32x4*>(q + row * C + li * P::VEC);
-      u32x4 rawk = *reinterpret_cast<const u32x4*>(k + row * C + li * P::VEC);
+    {
       T tq[P::VEC], tk[P::VEC];
-      __builtin_memcpy(tq, &rawq, 16);
-      __builtin_memcpy(tk, &rawk, 16);
+      __builtin_memcpy(tq, &rawq[pass], 16);
+      __builtin_memcpy(tk, &rawk[pass], 16);
 #pragma unroll
       for (int e = 0; e < P::VEC; ++e) {
         qv[e] = to_f32(tq[e]);
         kv[e] = to_f32(tk[e]);
       }
-    } else {
-#pragma unroll
-      for (int e = 0; e < P::VEC; ++e) qv[e] = kv[e] = 0.f;
     }
     float sqq = 0.f, skk = 0.f;
 #pragma unroll
