@@ -305,6 +305,110 @@ __global__ __launch_bounds__(BLOCK) void kd_rows_kernel(const KdArgs a) {
     }
   }
 
+  if (g.head == 0 && g.tail0 == V) {
+    // Whole row in 16-byte vectors (the usual case): the registers hold
+    // everything, so the maxima come first, then every exponential is taken
+    // once and kept, and the gradient is a multiplication away.
+    float xt[KREG][VEC], xs[KREG][VEC], x1[CE ? KREG : 1][CE ? VEC : 1];
+    float mt = kNegBig, ms = kNegBig;
+#pragma unroll
+    for (int j = 0; j < KREG; ++j) {
+      const bool live = gtid + (int64_t)j * GROUP < g.nvec;
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) {
+        xt[j][i] = live ? to_f32(rt[j].v[i]) : kNegBig;
+        xs[j][i] = live ? to_f32(rs[j].v[i]) : kNegBig;
+        mt = fmaxf(mt, xt[j][i]);
+        ms = fmaxf(ms, xs[j][i]);
+      }
+    }
+#pragma unroll
+    for (int off = (GROUP < kWave ? GROUP : kWave) / 2; off > 0; off >>= 1) {
+      mt = fmaxf(mt, __shfl_xor(mt, off, kWave));
+      ms = fmaxf(ms, __shfl_xor(ms, off, kWave));
+    }
+    const int w = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    if (NW > 1) {
+      if (lane == 0) {
+        lds_t[w].m = mt;
+        lds_s[w].m = ms;
+      }
+      __syncthreads();
+#pragma unroll
+      for (int i = 0; i < NW; ++i) {
+        mt = fmaxf(mt, lds_t[i].m);
+        ms = fmaxf(ms, lds_s[i].m);
+      }
+    }
+    const float mtk = mt * a.k, msk = ms * a.k, ms1 = ms * kLog2e;
+    float zt = 0.f, at = 0.f, zs = 0.f, z1 = 0.f;
+#pragma unroll
+    for (int j = 0; j < KREG; ++j) {
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) {
+        const float tv = xt[j][i], sv = xs[j][i];
+        const float et = fast_exp2(fmaf(tv, a.k, -mtk));
+        const float es = fast_exp2(fmaf(sv, a.k, -msk));
+        zt += et;
+        zs += es;
+        at = fmaf(et, tv - sv, at);
+        xt[j][i] = et;
+        xs[j][i] = es;
+        if (CE) {
+          const float e1 = fast_exp2(fmaf(sv, kLog2e, -ms1));
+          z1 += e1;
+          x1[j][i] = e1;
+        }
+      }
+    }
+#pragma unroll
+    for (int off = (GROUP < kWave ? GROUP : kWave) / 2; off > 0; off >>= 1) {
+      zt += __shfl_xor(zt, off, kWave);
+      zs += __shfl_xor(zs, off, kWave);
+      at += __shfl_xor(at, off, kWave);
+      if (CE) z1 += __shfl_xor(z1, off, kWave);
+    }
+    if (NW > 1) {
+      // .m of both arrays is still being read by slower wavefronts; the sums
+      // go into the other fields
+      if (lane == 0) {
+        lds_t[w].z = zt;
+        lds_t[w].a = at;
+        lds_s[w].z = zs;
+        lds_s[w].z1 = z1;
+      }
+      __syncthreads();
+      zt = at = zs = z1 = 0.f;
+#pragma unroll
+      for (int i = 0; i < NW; ++i) {
+        zt += lds_t[i].z;
+        at += lds_t[i].a;
+        zs += lds_s[i].z;
+        z1 += lds_s[i].z1;
+      }
+    }
+    const RowFinal f =
+        finish_row<T, CE>(a, job, row, TStat{mt, zt, at}, SStat{ms, zs, z1}, srow, gtid == 0);
+    if (!grow) return;
+    const float ct = f.g_kd / zt, cs = f.g_kd / zs, c1 = CE ? f.g_ce / z1 : 0.f;
+#pragma unroll
+    for (int j = 0; j < KREG; ++j) {
+      const int64_t v = gtid + (int64_t)j * GROUP;
+      if (v < g.nvec) {
+        Vec16<T> o;
+        const int64_t e0 = v * VEC;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+          float gv = xs[j][i] * cs - xt[j][i] * ct;
+          if (CE) gv += fmaf(x1[j][i], c1, e0 + i == job.label ? -f.g_ce : 0.f);
+          o.v[i] = from_f32<T>(gv);
+        }
+        store16(grow + e0, o);
+      }
+    }
+    return;
+  }
+
   TStat st = tstat_init();
   SStat ss = sstat_init();
   {
