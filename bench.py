@@ -27,6 +27,7 @@ import json
 import os
 import statistics
 import sys
+import threading
 import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
@@ -94,17 +95,51 @@ def run_step_benchmark(steps, warmup, dev):
     s_loss.wait_stream(torch.cuda.current_stream(dev))
     state = {"teacher": teacher, "loss": None}
 
-    def step():
+    # One host thread per stream, as TSPipe's workers are: the loss thread
+    # spends most of a step waiting for autograd's device thread (GIL released),
+    # and the EMA thread's launches fit into those waits.
+    def ema_worker(n, events):
         with torch.cuda.stream(s_ema):
-            state["teacher"] = ta.calculate_updated_momentum_encoder(0.99, student, state["teacher"])
-        with torch.cuda.stream(s_loss):
-            q.grad = None
-            loss = ta.infonce_loss(q, k, 0.2)
-            loss.backward()
-            state["loss"] = loss
+            state["ema_span"] = span = (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+            span[0].record()
+            for i in range(n):
+                ema_mod.kernel_events = events if (events is not None and i % TIMED_EVERY == 0) else None
+                state["teacher"] = ta.calculate_updated_momentum_encoder(0.99, student, state["teacher"])
+            span[1].record()
+        ema_mod.kernel_events = None
+        state["ema_enqueued"] = time.perf_counter()
 
-    for _ in range(warmup):
-        step()
+    def loss_worker(n, _events):
+        with torch.cuda.stream(s_loss):
+            state["loss_span"] = span = (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+            span[0].record()
+            for _ in range(n):
+                q.grad = None
+                loss = ta.infonce_loss(q, k, 0.2)
+                loss.backward()
+                state["loss"] = loss
+            span[1].record()
+        state["loss_enqueued"] = time.perf_counter()
+
+    def run_steps(n, events):
+        failures = []
+
+        def guarded(fn):
+            def body():
+                try:
+                    fn(n, events)
+                except BaseException as exc:  # re-raised on the main thread below
+                    failures.append(exc)
+            return body
+        workers = [threading.Thread(target=guarded(f)) for f in (ema_worker, loss_worker)]
+        for w in workers:
+            w.start()
+        for w in workers:
+            w.join()
+        if failures:
+            raise failures[0]
+
+    run_steps(warmup, None)
     torch.cuda.synchronize()
     # Every TIMED_EVERY-th EMA launch of the timed region stamps its own begin
     # and end into a pair of HIP events (a timed launch costs the host ~25 us
@@ -116,13 +151,15 @@ def run_step_benchmark(steps, warmup, dev):
     gc.collect()
     gc.disable()  # as timeit does: no collector pause inside the timed region
     t0 = time.perf_counter()
-    for i in range(steps):
-        ema_mod.kernel_events = events if i % TIMED_EVERY == 0 else None
-        step()
+    run_steps(steps, events)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     gc.enable()
-    ema_mod.kernel_events = None
+    host_ms = {"ema_thread_enqueue_ms_per_step": round((state["ema_enqueued"] - t0) / steps * 1e3, 4),
+               "loss_thread_enqueue_ms_per_step": round((state["loss_enqueued"] - t0) / steps * 1e3, 4),
+               # first to last command of each stream, by HIP events on that stream
+               "ema_stream_ms_per_step": round(state["ema_span"][0].elapsed_time(state["ema_span"][1]) / steps, 4),
+               "loss_stream_ms_per_step": round(state["loss_span"][0].elapsed_time(state["loss_span"][1]) / steps, 4)}
     ema_ms = _event_ms(events)
     assert len(ema_ms) == n_timed
     avg_ema_ms = sum(ema_ms) / len(ema_ms)
@@ -141,7 +178,7 @@ def run_step_benchmark(steps, warmup, dev):
     alone_ms = sum(_event_ms(alone)) / len(alone)
     alone_gbs = algo_bytes / (alone_ms * 1e-3) / 1e9
     return {
-        "elapsed": elapsed, "n_params": n_params, "loss": float(state["loss"].item()),
+        "elapsed": elapsed, "n_params": n_params, "loss": float(state["loss"].item()), "host": host_ms,
         "roofline": {"bound": "hbm", "kernel": "ema_multi_kernel", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": EMA_VITB_TRAFFIC_BYTES, "algorithmic_bytes_per_launch": algo_bytes,
@@ -439,6 +476,7 @@ def main():
                    "ema_tensors": 152, "ema_params": res["n_params"], "infonce_n": 4096, "infonce_c": 256},
         "roofline": res["roofline"],
         "loss": res["loss"],
+        "host": res["host"],
     }
     if not args.no_kernels:
         line["kernels"] = run_kernel_table(dev)

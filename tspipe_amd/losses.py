@@ -401,11 +401,14 @@ class _BYOLFn(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_output: Tensor):
         _once(ctx)
+        # the context lets go of the buffers, so autograd can adopt them as .grad instead of copying
+        g1, g2 = ctx.g1, ctx.g2
+        ctx.g1 = ctx.g2 = None
         out1 = out2 = None
-        if ctx.g1 is not None:
-            out1 = _scale_saved_grad(ctx.g1, grad_output, *ctx.dims)
-        if ctx.g2 is not None:
-            out2 = _scale_saved_grad(ctx.g2, grad_output, *ctx.dims)
+        if g1 is not None:
+            out1 = _scale_saved_grad(g1, grad_output, *ctx.dims)
+        if g2 is not None:
+            out2 = _scale_saved_grad(g2, grad_output, *ctx.dims)
         return out1, None, out2, None
 
 
@@ -458,11 +461,14 @@ class _InfoNCEFn(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_output: Tensor):
         _once(ctx)
+        # the context lets go of the buffers, so autograd can adopt them as .grad instead of copying
+        g1, g2 = ctx.g1, ctx.g2
+        ctx.g1 = ctx.g2 = None
         out1 = out2 = None
-        if ctx.g1 is not None:
-            out1 = _scale_saved_grad(ctx.g1, grad_output, *ctx.dims)
-        if ctx.g2 is not None:
-            out2 = _scale_saved_grad(ctx.g2, grad_output, *ctx.dims)
+        if g1 is not None:
+            out1 = _scale_saved_grad(g1, grad_output, *ctx.dims)
+        if g2 is not None:
+            out2 = _scale_saved_grad(g2, grad_output, *ctx.dims)
         return out1, None, out2, None, None
 
 
