@@ -28,7 +28,8 @@
 //            images go from global memory straight into LDS (no registers),
 //            three tiles ahead.  Writes per-split partial l and O^T in
 //            register-native order.
-//   combine  per 32-row q tile: adds the splits, forms loss rows and dq.
+//   combine  per 32-row q tile: adds the splits and forms dq; its first
+//            workgroup adds up the loss from the split row sums.
 //
 // Tile image (C features, KK = C/16, FB = C/32; 1 KB fragments, lane L =
 // 32h + col reads bytes 16L..16L+15 of a fragment as one MFMA A operand):
@@ -60,8 +61,8 @@ int launch_sum_scale(const float* v, int64_t n, float scale, float denom, float*
 
 __host__ __device__ inline int64_t nce_round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
 
-// Workspace carve-up (all offsets multiples of 256 bytes): a head with the
-// loss rows of every pair, [pairs][npad] floats, then one region per pair.
+// Workspace carve-up (all offsets multiples of 256 bytes): a small head, then
+// one region per pair.
 struct NceLayout {
   int64_t npad;
   int splits;
@@ -76,7 +77,7 @@ struct NcePair {
   const void* k;
   void* dq;
   const uint16_t* qsrc;  // bf16 queries the MFMA reads: q itself or the rounded copy
-  float *rq, *rk, *diag, *lpart, *apart, *opart, *row_loss;
+  float *rq, *rk, *diag, *lpart, *apart, *opart;
   uint8_t* kimg;
   uint16_t* qb;
 };
@@ -100,7 +101,7 @@ inline NceLayout nce_layout(int64_t n, int64_t c, int n_pairs, bool fp32_in) {
   NceLayout L;
   L.npad = nce_round_up(n > 0 ? n : 1, kQTile);
   L.splits = nce_splits(L.npad, n_pairs);
-  L.head_bytes = nce_align((size_t)n_pairs * L.npad * 4);
+  L.head_bytes = 256;  // scratch for the empty-batch case
   size_t o = 0;
   L.off_rq = o;       o += nce_align(L.npad * 4);
   L.off_rk = o;       o += nce_align(L.npad * 4);
@@ -468,9 +469,82 @@ __global__ __launch_bounds__(kNceBlock) void nce_main_kernel(NceArgs args, int64
 // element-wise, because <qh_i, dqh_i> follows from the row sums:
 //   <qh_i, sum_j P_ij kh_j> = (tau/log2e) A_i / l_i,  <qh_i, kh_i> = (tau/log2e) diag_i
 // ---------------------------------------------------------------------------
+// The scalar loss, by one workgroup straight from the split row sums:
+//   loss = loss_scale / n * sum over pairs and rows of ln2 (x_max + log2 l_i - diag_i).
+// Re-deriving l_i here instead of reading the other workgroups' results keeps
+// the reduction inside this launch; the order of every addition is fixed.
+__device__ __forceinline__ void nce_loss_block(const NceArgs& args, int pairs, int64_t n, int64_t npad, int splits,
+                                               float scale2, float loss_scale, float* __restrict__ loss_out) {
+  __shared__ float red[kNceBlock / kWave];
+  const int tid = threadIdx.x;
+  constexpr int U = 4;   // row quads per thread and trip
+  constexpr int SC = 4;  // splits per batch of loads
+  const int64_t quads = npad / 4;
+  float acc = 0.f;
+  for (int p = 0; p < pairs; ++p) {
+    const float* __restrict__ lpart = args.p[p].lpart;
+    const float* __restrict__ diag = args.p[p].diag;
+    for (int64_t q0 = tid; q0 < quads; q0 += (int64_t)U * kNceBlock) {
+      // Loads of a batch are all issued before the first is used; a quad or a
+      // split beyond the end re-reads a valid address and is added as zero, so
+      // no branch separates the loads.
+      int64_t quad[U];
+      float keep_q[U];
+      f32x4 l[U], d[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int64_t want = q0 + (int64_t)u * kNceBlock;
+        keep_q[u] = want < quads ? 1.f : 0.f;
+        quad[u] = want < quads ? want : q0;
+        l[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+        d[u] = *reinterpret_cast<const f32x4*>(diag + 4 * quad[u]);
+      }
+      for (int s0 = 0; s0 < splits; s0 += SC) {
+        f32x4 v[SC][U];
+        float keep_s[SC];
+#pragma unroll
+        for (int c = 0; c < SC; ++c) {
+          keep_s[c] = s0 + c < splits ? 1.f : 0.f;
+          const int sp = s0 + c < splits ? s0 + c : s0;
+#pragma unroll
+          for (int u = 0; u < U; ++u) v[c][u] = *reinterpret_cast<const f32x4*>(lpart + (int64_t)sp * npad + 4 * quad[u]);
+        }
+#pragma unroll
+        for (int c = 0; c < SC; ++c)
+#pragma unroll
+          for (int u = 0; u < U; ++u) l[u] += v[c][u] * keep_s[c];
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const bool live = keep_q[u] != 0.f && 4 * quad[u] + j < n;
+          const float term = kNceLn2 * (scale2 + log2f(l[u][j]) - d[u][j]);
+          acc += live ? term : 0.f;
+        }
+      }
+    }
+  }
+  acc = wave_sum(acc);
+  if (tid % kWave == 0) red[tid / kWave] = acc;
+  __syncthreads();
+  if (tid == 0) {
+    float total = 0.f;
+#pragma unroll
+    for (int w = 0; w < kNceBlock / kWave; ++w) total += red[w];
+    *loss_out = total * loss_scale / (float)n;
+  }
+}
+
 template <typename T, int C>
 __global__ __launch_bounds__(kNceBlock) void nce_combine_kernel(NceArgs args, int64_t n, int64_t npad, int splits,
-                                                                float scale2) {
+                                                                float scale2, float loss_scale,
+                                                                float* __restrict__ loss_out) {
+  // workgroup 0 of the first pair computes the loss; the (q tile, feature block) items start at workgroup 1
+  if (blockIdx.x == 0) {
+    if (blockIdx.z == 0) nce_loss_block(args, (int)gridDim.z, n, npad, splits, scale2, loss_scale, loss_out);
+    return;
+  }
   const NcePair& pr = args.p[blockIdx.z];
   const T* __restrict__ q = (const T*)pr.q;
   const T* __restrict__ k = (const T*)pr.k;
@@ -480,12 +554,11 @@ __global__ __launch_bounds__(kNceBlock) void nce_combine_kernel(NceArgs args, in
   const float* __restrict__ lpart = pr.lpart;
   const float* __restrict__ apart = pr.apart;
   const float* __restrict__ opart = pr.opart;
-  float* __restrict__ row_loss = pr.row_loss;
   T* __restrict__ dq = (T*)pr.dq;
   constexpr int FB = C / 32;
   const int lane = threadIdx.x % kWave, w = threadIdx.x / kWave;
   const int col = lane % 32, h = lane / 32;
-  const int64_t item = (int64_t)blockIdx.x * (kNceBlock / kWave) + w;
+  const int64_t item = (int64_t)(blockIdx.x - 1) * (kNceBlock / kWave) + w;
   const int64_t tile32 = item / FB;
   const int fb = (int)(item % FB);
   if (tile32 >= npad / 32) return;
@@ -529,7 +602,6 @@ __global__ __launch_bounds__(kNceBlock) void nce_combine_kernel(NceArgs args, in
       A += apart[(int64_t)s * npad + row];
     }
   }
-  if (fb == 0 && h == 0) row_loss[row] = live ? kNceLn2 * (scale2 + log2f(l) - d) : 0.f;
   if (!dq) return;
 
   float o[16];
@@ -580,7 +652,8 @@ __global__ __launch_bounds__(kNceBlock) void nce_combine_kernel(NceArgs args, in
 }
 
 template <typename T, int C>
-int nce_run(const NceArgs& args, int pairs, int64_t n, float tau, const NceLayout& L, hipStream_t stream) {
+int nce_run(const NceArgs& args, int pairs, int64_t n, float tau, const NceLayout& L, float* loss_out,
+            hipStream_t stream) {
   const float scale2 = kNceLog2e / tau;
   const unsigned z = (unsigned)pairs;
   hipLaunchKernelGGL((nce_prep_kernel<T, C>), dim3((unsigned)(L.npad / kKTile), 1, z), dim3(kNceBlock), 0, stream, args,
@@ -592,18 +665,18 @@ int nce_run(const NceArgs& args, int pairs, int64_t n, float tau, const NceLayou
   rc = check_launch();
   if (rc) return rc;
   const int64_t items = L.npad / 32 * (C / 32);  // a multiple of 4: npad is a multiple of 128
-  hipLaunchKernelGGL((nce_combine_kernel<T, C>), dim3((unsigned)(items / 4), 1, z), dim3(kNceBlock), 0, stream, args,
-                     n, L.npad, L.splits, scale2);
+  hipLaunchKernelGGL((nce_combine_kernel<T, C>), dim3((unsigned)(items / 4 + 1), 1, z), dim3(kNceBlock), 0, stream,
+                     args, n, L.npad, L.splits, scale2, 2.f * tau, loss_out);
   return check_launch();
 }
 
 template <typename T>
 int nce_dispatch_c(const NceArgs& args, int pairs, int64_t n, int64_t c, float tau, const NceLayout& L,
-                   hipStream_t stream) {
+                   float* loss_out, hipStream_t stream) {
   switch (c) {
-    case 64: return nce_run<T, 64>(args, pairs, n, tau, L, stream);
-    case 128: return nce_run<T, 128>(args, pairs, n, tau, L, stream);
-    case 256: return nce_run<T, 256>(args, pairs, n, tau, L, stream);
+    case 64: return nce_run<T, 64>(args, pairs, n, tau, L, loss_out, stream);
+    case 128: return nce_run<T, 128>(args, pairs, n, tau, L, loss_out, stream);
+    case 256: return nce_run<T, 256>(args, pairs, n, tau, L, loss_out, stream);
     default: return TS_ERR_ARG;
   }
 }
@@ -641,7 +714,6 @@ int ts_infonce_fwd_bwd(const void* q1, const void* k1, const void* q2, const voi
   }
   const ts::NceLayout L = ts::nce_layout(n, c, pairs, true);
   char* ws = (char*)workspace;
-  float* row_loss = (float*)ws;
   ts::NceArgs args;
   for (int p = 0; p < 2; ++p) {
     const int src = p < pairs ? p : 0;  // an unused second slot mirrors the first
@@ -659,13 +731,10 @@ int ts_infonce_fwd_bwd(const void* q1, const void* k1, const void* q2, const voi
     P.kimg = (uint8_t*)(wsp + L.off_kimg);
     P.qb = dtype == TS_F32 ? (uint16_t*)(wsp + L.off_qb) : nullptr;
     P.qsrc = dtype == TS_F32 ? P.qb : (const uint16_t*)P.q;
-    P.row_loss = row_loss + (size_t)src * L.npad;
   }
-  const int rc = (dtype == TS_F32) ? ts::nce_dispatch_c<float>(args, pairs, n, c, tau, L, st)
-                                   : ts::nce_dispatch_c<ts::bf16_t>(args, pairs, n, c, tau, L, st);
-  if (rc) return rc;
-  // loss = 2 tau / n * sum over all pairs' rows (padding rows hold zero)
-  return ts::launch_sum_scale(row_loss, (int64_t)pairs * L.npad, 2.f * tau, (float)n, loss_out, st);
+  // loss = 2 tau / n * sum over all pairs' rows, written by the combine launch
+  return (dtype == TS_F32) ? ts::nce_dispatch_c<float>(args, pairs, n, c, tau, L, loss_out, st)
+                           : ts::nce_dispatch_c<ts::bf16_t>(args, pairs, n, c, tau, L, loss_out, st);
 }
 
 }  // extern "C"
