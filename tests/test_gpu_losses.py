@@ -42,7 +42,8 @@ def test_kd_cfg2_fp32(device):
     assert max_rel_to_peak(sd.grad, s32.grad) < 1e-5
 
 
-@pytest.mark.parametrize("rows,V", [(1, 1), (3, 5), (7, 63), (5, 64), (4, 65), (9, 1000), (2, 2049), (3, 4099)])
+@pytest.mark.parametrize("rows,V", [(1, 1), (3, 5), (7, 63), (5, 64), (4, 65), (9, 1000), (2, 2049), (3, 4099),
+                                    (5, 8191), (2, 16380), (2, 16381)])
 def test_kd_shapes_fp32(device, rows, V):
     g = seeded(100 + V)
     s = torch.randn(rows, V, generator=g) * 3
@@ -53,6 +54,42 @@ def test_kd_shapes_fp32(device, rows, V):
     loss.backward()
     assert rel_err(loss.item(), want) < 2e-5 or abs(loss.item() - want) < 1e-7
     assert max_rel_to_peak(sd.grad, gw) < 2e-5 or gw.abs().max() < 1e-12
+
+
+@pytest.mark.parametrize("rows,V", [(5, 4097), (4, 9001), (3, 30522), (2, 32760), (2, 32761)])
+def test_kd_long_rows_bf16_unmasked(device, rows, V):
+    # rows of 8 K to 32 K bf16 logits without a mask: one launch with the row pair in registers
+    # (up to 32760 elements, here also with rows that start off a 16-byte boundary), two passes beyond
+    g = seeded(300 + V)
+    s = (torch.randn(rows, V, generator=g) * 2).to(torch.bfloat16)
+    t = (torch.randn(rows, V, generator=g) * 2).to(torch.bfloat16)
+    want, (gw,) = _oracle_grad(lambda a, b: ts_oracle.kd_soft_target(a, b, 2.0), s, others=(t,))
+    sd = s.to(device).requires_grad_()
+    loss = ta.kd_soft_target_loss(sd, t.to(device), 2.0)
+    loss.backward()
+    assert rel_err(loss.item(), want) < 1e-3
+    err = (sd.grad.cpu().double() - gw).abs()
+    assert (err <= 1e-3 * gw.abs().max() + gw.abs() * 2.0 ** -8).all()
+
+
+def test_kd_long_rows_operands_aligned_differently(device):
+    # student and teacher rows at different offsets from a 16-byte boundary: same results
+    # as for aligned operands (the kernels fall back to element-wise access where they must)
+    g = seeded(41)
+    rows, V = 3, 6000
+    s = torch.randn(rows, V, generator=g) * 3
+    t = torch.randn(rows, V, generator=g) * 3
+    ref_s = s.to(device).requires_grad_()
+    ref = ta.kd_soft_target_loss(ref_s, t.to(device), 3.0)
+    ref.backward()
+    pad = torch.zeros(rows * V + 1, device=device)
+    pad[1:] = s.to(device).reshape(-1)
+    shifted = pad[1:].view(rows, V).detach().requires_grad_()  # data pointer 4 bytes past a 16-byte boundary
+    assert shifted.data_ptr() % 16 == 4 and shifted.is_contiguous()
+    got = ta.kd_soft_target_loss(shifted, t.to(device), 3.0)
+    got.backward()
+    assert rel_err(got.item(), ref.item()) < 1e-6
+    assert max_rel_to_peak(shifted.grad, ref_s.grad.cpu()) < 1e-6
 
 
 def test_kd_identities(device):

@@ -305,12 +305,29 @@ __global__ __launch_bounds__(BLOCK) void kd_rows_kernel(const KdArgs a) {
     }
   }
 
-  if (g.head == 0 && g.tail0 == V) {
-    // Whole row in 16-byte vectors (the usual case): the registers hold
-    // everything, so the maxima come first, then every exponential is taken
-    // once and kept, and the gradient is a multiplication away.
-    float xt[KREG][VEC], xs[KREG][VEC], x1[CE ? KREG : 1][CE ? VEC : 1];
-    float mt = kNegBig, ms = kNegBig;
+  // Rows whose operands share one alignment (the usual case): all but a few
+  // end elements are 16-byte vectors held in registers, and each of those end
+  // elements gets a lane of its own.  The maxima come first, then every
+  // exponential is taken once and kept, and the gradient is a multiplication
+  // away.  (With the CE term on long rows the temperature-1 exponentials are
+  // recomputed instead of kept: registers.)
+  constexpr bool kKeepCe = CE && KREG * VEC <= 32;
+  // the long-row instantiation is only launched on rows of this kind (checked on the host)
+  constexpr bool kAlignedOnly = KREG * GROUP > 1024;
+  const int64_t ntail = V - g.tail0;
+  if (kAlignedOnly || (g.head < VEC && ntail < VEC)) {
+    const bool has_h = gtid < g.head, has_t = gtid < ntail;
+    float eh_t = kNegBig, eh_s = kNegBig, el_t = kNegBig, el_s = kNegBig;  // end elements: head, last
+    if (has_h) {
+      eh_t = to_f32(trow[gtid]);
+      eh_s = to_f32(srow[gtid]);
+    }
+    if (has_t) {
+      el_t = to_f32(trow[g.tail0 + gtid]);
+      el_s = to_f32(srow[g.tail0 + gtid]);
+    }
+    float xt[KREG][VEC], xs[KREG][VEC], x1[kKeepCe ? KREG : 1][kKeepCe ? VEC : 1];
+    float mt = fmaxf(eh_t, el_t), ms = fmaxf(eh_s, el_s);
 #pragma unroll
     for (int j = 0; j < KREG; ++j) {
       const bool live = gtid + (int64_t)j * GROUP < g.nvec;
@@ -342,25 +359,28 @@ __global__ __launch_bounds__(BLOCK) void kd_rows_kernel(const KdArgs a) {
     }
     const float mtk = mt * a.k, msk = ms * a.k, ms1 = ms * kLog2e;
     float zt = 0.f, at = 0.f, zs = 0.f, z1 = 0.f;
-#pragma unroll
-    for (int j = 0; j < KREG; ++j) {
-#pragma unroll
-      for (int i = 0; i < VEC; ++i) {
-        const float tv = xt[j][i], sv = xs[j][i];
-        const float et = fast_exp2(fmaf(tv, a.k, -mtk));
-        const float es = fast_exp2(fmaf(sv, a.k, -msk));
-        zt += et;
-        zs += es;
-        at = fmaf(et, tv - sv, at);
-        xt[j][i] = et;
-        xs[j][i] = es;
-        if (CE) {
-          const float e1 = fast_exp2(fmaf(sv, kLog2e, -ms1));
-          z1 += e1;
-          x1[j][i] = e1;
-        }
+    // one (teacher, student) pair: exponentials into the operands' own registers
+    auto take = [&](float& tv, float& sv, float* e1_keep) {
+      const float et = fast_exp2(fmaf(tv, a.k, -mtk));
+      const float es = fast_exp2(fmaf(sv, a.k, -msk));
+      zt += et;
+      zs += es;
+      at = fmaf(et, tv - sv, at);
+      if (CE) {
+        const float e1 = fast_exp2(fmaf(sv, kLog2e, -ms1));
+        z1 += e1;
+        if (e1_keep) *e1_keep = e1;
       }
-    }
+      tv = et;
+      sv = es;
+    };
+    float eh_1 = 0.f, el_1 = 0.f;
+    take(eh_t, eh_s, &eh_1);
+    take(el_t, el_s, &el_1);
+#pragma unroll
+    for (int j = 0; j < KREG; ++j)
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) take(xt[j][i], xs[j][i], kKeepCe ? &x1[j][i] : nullptr);
 #pragma unroll
     for (int off = (GROUP < kWave ? GROUP : kWave) / 2; off > 0; off >>= 1) {
       zt += __shfl_xor(zt, off, kWave);
@@ -390,18 +410,27 @@ __global__ __launch_bounds__(BLOCK) void kd_rows_kernel(const KdArgs a) {
     const RowFinal f =
         finish_row<T, CE>(a, job, row, TStat{mt, zt, at}, SStat{ms, zs, z1}, srow, gtid == 0);
     if (!grow) return;
-    const float ct = f.g_kd / zt, cs = f.g_kd / zs, c1 = CE ? f.g_ce / z1 : 0.f;
+    // probabilities first and the weight last, as the general path does: a
+    // weight folded into the reciprocals would be amplified by the cancellation in q - p
+    const float rt_ = 1.f / zt, rs_ = 1.f / zs, r1_ = CE ? 1.f / z1 : 0.f;
+    auto grad_of = [&](float et, float es, float e1, int64_t col) {
+      float gv = f.g_kd * fmaf(es, rs_, -(et * rt_));
+      if (CE) gv = fmaf(f.g_ce, fmaf(e1, r1_, col == job.label ? -1.f : 0.f), gv);
+      return from_f32<T>(gv);
+    };
+    if (has_h) grow[gtid] = grad_of(eh_t, eh_s, eh_1, gtid);
+    if (has_t) grow[g.tail0 + gtid] = grad_of(el_t, el_s, el_1, g.tail0 + gtid);
 #pragma unroll
     for (int j = 0; j < KREG; ++j) {
       const int64_t v = gtid + (int64_t)j * GROUP;
       if (v < g.nvec) {
         Vec16<T> o;
-        const int64_t e0 = v * VEC;
+        const int64_t e0 = g.head + v * VEC;
 #pragma unroll
         for (int i = 0; i < VEC; ++i) {
-          float gv = xs[j][i] * cs - xt[j][i] * ct;
-          if (CE) gv += fmaf(x1[j][i], c1, e0 + i == job.label ? -f.g_ce : 0.f);
-          o.v[i] = from_f32<T>(gv);
+          float e1 = 0.f;
+          if (CE) e1 = kKeepCe ? x1[j][i] : fast_exp2(fmaf(to_f32(rs[j].v[i]), kLog2e, -ms1));
+          o.v[i] = grad_of(xt[j][i], xs[j][i], e1, e0 + i);
         }
         store16(grow + e0, o);
       }
@@ -409,6 +438,7 @@ __global__ __launch_bounds__(BLOCK) void kd_rows_kernel(const KdArgs a) {
     return;
   }
 
+  if constexpr (!kAlignedOnly) {
   TStat st = tstat_init();
   SStat ss = sstat_init();
   {
@@ -471,6 +501,7 @@ __global__ __launch_bounds__(BLOCK) void kd_rows_kernel(const KdArgs a) {
       store16(grow + e0, o);
     }
   }
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -497,6 +528,38 @@ struct PartStat {  // 32 bytes
 template <int NT>
 __device__ __forceinline__ void kd_count_block(const KdArgs& a, int* __restrict__ counts, int* __restrict__ sel_rows);
 
+// A row without a loss term: zero loss entries, and this part of its gradient row zero-filled.
+template <typename T, bool CE>
+__device__ __forceinline__ void kd_zero_part(const KdArgs& a, int64_t row, int part, int parts) {
+  constexpr int VEC = Vec16<T>::N;
+  const int tid = threadIdx.x;
+  const int64_t V = a.V;
+  const int64_t v0 = (int64_t)part * kPartVecs;
+  if (part == 0 && tid == 0) {
+    a.row_kd[row] = 0.f;
+    if (CE) a.row_ce[row] = 0.f;
+  }
+  if (!kd_has_grad(a)) return;
+  T* grow = kd_row_ptrs<T>(a, row).g;
+  const uint32_t mis = (uint32_t)((uintptr_t)grow & 15u);
+  int64_t head = (int64_t)(((16u - mis) & 15u) / sizeof(T));
+  if (head > V) head = V;
+  const int64_t nvec = (V - head) / VEC, tail0 = head + nvec * VEC;
+  const T zero = from_f32<T>(0.f);
+  Vec16<T> z;
+#pragma unroll
+  for (int i = 0; i < VEC; ++i) z.v[i] = zero;
+  if (part == 0)
+    for (int64_t i = tid; i < head; i += kPartBlock) grow[i] = zero;
+  if (part == parts - 1)
+    for (int64_t i = tail0 + tid; i < V; i += kPartBlock) grow[i] = zero;
+#pragma unroll
+  for (int j = 0; j < kPartPerThread; ++j) {
+    const int64_t v = v0 + tid + j * kPartBlock;
+    if (v < nvec) store16(grow + head + v * VEC, z);
+  }
+}
+
 // With count_out set, workgroup 0 does the row counting and compaction that
 // pass 2 and the final reduction need (nothing in pass 1 reads them), and the
 // (row, part) items start at workgroup 1.
@@ -521,29 +584,7 @@ __global__ __launch_bounds__(kPartBlock) void kd_wide_pass1_kernel(const KdArgs 
   const RowJob job = row_job(a, row);
 
   if (!job.kd && !job.ce) {
-    if (part == 0 && tid == 0) {
-      a.row_kd[row] = 0.f;
-      if (CE) a.row_ce[row] = 0.f;
-    }
-    if (!kd_has_grad(a)) return;
-    T* grow = kd_row_ptrs<T>(a, row).g;
-    const uint32_t mis = (uint32_t)((uintptr_t)grow & 15u);
-    int64_t head = (int64_t)(((16u - mis) & 15u) / sizeof(T));
-    if (head > V) head = V;
-    const int64_t nvec = (V - head) / VEC, tail0 = head + nvec * VEC;
-    const T zero = from_f32<T>(0.f);
-    Vec16<T> z;
-#pragma unroll
-    for (int i = 0; i < VEC; ++i) z.v[i] = zero;
-    if (part == 0)
-      for (int64_t i = tid; i < head; i += kPartBlock) grow[i] = zero;
-    if (part == parts - 1)
-      for (int64_t i = tail0 + tid; i < V; i += kPartBlock) grow[i] = zero;
-#pragma unroll
-    for (int j = 0; j < kPartPerThread; ++j) {
-      const int64_t v = v0 + tid + j * kPartBlock;
-      if (v < nvec) store16(grow + head + v * VEC, z);
-    }
+    kd_zero_part<T, CE>(a, row, part, parts);
     return;
   }
 
@@ -829,6 +870,21 @@ inline KdWorkspace kd_carve(void* ws, int64_t n_rows) {
   return w;
 }
 
+// True when in every row s, t and the gradient sit at the same offset from a
+// 16-byte boundary, so that one split into end elements and vectors fits all three.
+template <typename T>
+inline bool kd_rows_aligned_alike(const KdArgs& a) {
+  auto alike = [](const void* x, const void* y) { return (((uintptr_t)x ^ (uintptr_t)y) & 15u) == 0; };
+  const int64_t sz = (int64_t)sizeof(T);
+  if (((a.ld_s - a.ld_t) * sz) & 15) return false;
+  const bool has_g = a.n_pieces ? a.g_piece[0] != nullptr : a.grad != nullptr;
+  if (has_g && (((a.ld_s - a.ld_g) * sz) & 15)) return false;
+  if (a.n_pieces == 0) return alike(a.s, a.t) && (!has_g || alike(a.s, a.grad));
+  for (int p = 0; p < a.n_pieces; ++p)
+    if (!alike(a.s_piece[p], a.t_piece[p]) || (has_g && !alike(a.s_piece[p], a.g_piece[p]))) return false;
+  return true;
+}
+
 template <typename T, bool CE>
 int launch_kd_t(KdArgs a, float kd_scale, void* ws, float* loss_out, hipStream_t stream) {
   const KdWorkspace w = kd_carve(ws, a.n_rows);
@@ -840,7 +896,12 @@ int launch_kd_t(KdArgs a, float kd_scale, void* ws, float* loss_out, hipStream_t
   const bool compact = parts && counted;
   int rc = TS_OK;
   const int64_t vecs_ = (a.V + Vec16<T>::N - 1) / Vec16<T>::N + 1;
-  const bool wide = a.n_rows > 0 && parts > 0 && vecs_ > 64 * 4;
+  // Long rows without a mask or labels, operands aligned alike: one launch, the
+  // row pair held in the registers of a 512-thread workgroup.  Under a mask
+  // the two-pass form below stays: it overlaps the zero-fill of the rows
+  // without a term with the arithmetic of the others.
+  const bool one_launch = a.n_rows > 0 && parts > 0 && !counted && vecs_ <= 512 * 8 && kd_rows_aligned_alike<T>(a);
+  const bool wide = a.n_rows > 0 && parts > 0 && !one_launch;
   if (counted && !wide) {
     hipLaunchKernelGGL(kd_count_kernel, dim3(1), dim3(1024), 0, stream, a, w.counts,
                        compact ? w.sel_rows : (int*)nullptr);
@@ -866,6 +927,8 @@ int launch_kd_t(KdArgs a, float kd_scale, void* ws, float* loss_out, hipStream_t
     TS_KD_LAUNCH(256, 64, 4);
   } else if (parts == 0) {
     TS_KD_LAUNCH(256, 256, 4);
+  } else if (one_launch) {
+    TS_KD_LAUNCH(512, 512, 8);
   } else {
     const int64_t items = a.n_rows * parts;
     if (items > 0x7fffffffLL) return TS_ERR_RANGE;
