@@ -338,22 +338,35 @@ def run_kernel_table(dev):
                                                f"zero-fill of the other rows", 3)
     del s_full, t_full, f
 
-    # InfoNCE (cfg4), single pair
-    q = torch.nn.functional.normalize(torch.randn(4096, 256, generator=g), dim=1).to(torch.bfloat16).to(dev)
-    k = torch.nn.functional.normalize(torch.randn(4096, 256, generator=g), dim=1).to(torch.bfloat16).to(dev)
-    ws = torch.empty(lib.ts_infonce_workspace_bytes(4096, 256, 1), dtype=torch.uint8, device=dev)
-    loss, dq = torch.empty((), device=dev), torch.empty_like(q)
+    # InfoNCE: cfg4 (single pair), the symmetric two-pair call of MoCo-v3's contrastive_loss, and a
+    # batch four times as large, where the fixed costs of the three launches weigh less
+    def nce_entry(n, pairs, iters, note=None):
+        mk = lambda: torch.nn.functional.normalize(torch.randn(n, 256, generator=g), dim=1).to(torch.bfloat16).to(dev)
+        q1, k1 = mk(), mk()
+        q2, k2 = (mk(), mk()) if pairs == 2 else (None, None)
+        ws = torch.empty(lib.ts_infonce_workspace_bytes(n, 256, pairs), dtype=torch.uint8, device=dev)
+        loss, d1 = torch.empty((), device=dev), torch.empty_like(q1)
+        d2 = torch.empty_like(q1) if pairs == 2 else None
+        ptr = lambda t: None if t is None else t.data_ptr()
 
-    def f():
-        _lib.check(lib.ts_infonce_fwd_bwd(q.data_ptr(), k.data_ptr(), None, None, 4096, 256, 0.2, ws.data_ptr(),
-                                          loss.data_ptr(), dq.data_ptr(), None, _lib.TS_BF16, stream), "ts_infonce_fwd_bwd")
-    ms = _time_stream(f, 50)
-    flops = 2 * 2 * 4096 * 4096 * 256
-    out["infonce_4096x256_bf16"] = {"ms": round(ms, 4), "TFLOP/s": round(flops / (ms * 1e-3) / 1e12, 1),
-                                    "frac_mfma_bf16_peak": round(flops / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
-                                    "algorithmic_flop": flops, "kernel_launches": 3}
+        def f():
+            _lib.check(lib.ts_infonce_fwd_bwd(ptr(q1), ptr(k1), ptr(q2), ptr(k2), n, 256, 0.2, ws.data_ptr(),
+                                              loss.data_ptr(), ptr(d1), ptr(d2), _lib.TS_BF16, stream),
+                       "ts_infonce_fwd_bwd")
+        ms = _time_stream(f, iters)
+        flops = pairs * 2 * 2 * n * n * 256
+        e = {"ms": round(ms, 4), "TFLOP/s": round(flops / (ms * 1e-3) / 1e12, 1),
+             "frac_mfma_bf16_peak": round(flops / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+             "algorithmic_flop": flops, "kernel_launches": 3}
+        if note:
+            e["note"] = note
+        return e
+    out["infonce_4096x256_bf16"] = nce_entry(4096, 1, 50)
+    out["infonce_2_pairs_4096x256_bf16"] = nce_entry(4096, 2, 50, "both directions of the symmetric loss in one call")
+    out["infonce_16384x256_bf16"] = nce_entry(16384, 1, 20, "not a BASELINE config: the same kernels at 16x the work")
 
     # BYOL loss (latency only)
+    loss = torch.empty((), device=dev)
     o = [torch.randn(256, 128, generator=g).to(dev) for _ in range(4)]
     g1, g2 = torch.empty_like(o[0]), torch.empty_like(o[1])
     wsb = torch.empty(512, device=dev)
