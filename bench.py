@@ -363,7 +363,7 @@ def run_kernel_table(dev):
         return e
     out["infonce_4096x256_bf16"] = nce_entry(4096, 1, 50)
     out["infonce_2_pairs_4096x256_bf16"] = nce_entry(4096, 2, 50, "both directions of the symmetric loss in one call")
-    out["infonce_16384x256_bf16"] = nce_entry(16384, 1, 20, "not a BASELINE config: the same kernels at 16x the work")
+    out["infonce_16384x256_bf16"] = nce_entry(16384, 1, 20, "not one of the benchmark configurations: the same kernels at 16x the work")
 
     # BYOL loss (latency only)
     loss = torch.empty((), device=dev)
