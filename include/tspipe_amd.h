@@ -263,8 +263,9 @@ int ts_cosine_fwd_bwd(const void* x, const void* y, const uint8_t* row_mask, int
 /*   loss = CrossEntropy(logits, arange(N)) * 2 tau   (mean over rows)       */
 /*   dq   = d loss / d q  (k is the detached teacher output)                 */
 /* Up to two (q,k) pairs are summed into one loss (main.py:162); q2,k2,dq2   */
-/* may be NULL.  q*, k*: [n, c] contiguous bf16 (TS_BF16) or fp32 (TS_F32,   */
-/* rounded to bf16 for the MFMA contraction); c a multiple of 32, <= 256.    */
+/* may be NULL.  q*, k*: [n, c] contiguous bf16 (TS_BF16), or fp32 / fp16     */
+/* (TS_F32 / TS_F16, rounded to bf16 for the MFMA contraction; dq comes back */
+/* in the input type); c = 64, 128 or 256.                                   */
 /* workspace: ts_infonce_workspace_bytes(n, c, n_pairs) bytes, 256-aligned.  */
 /* ------------------------------------------------------------------------ */
 

@@ -152,7 +152,7 @@ def test_device_entry_points_validate_before_launching():
     assert lib.ts_infonce_fwd_bwd(p, p, None, None, 16, 100, 0.2, p, p, None, None, 1, None) == -1   # c not 64/128/256
     assert lib.ts_infonce_fwd_bwd(p, p, None, None, 16, 64, 0.001, 0x1000, p, None, None, 1, None) == -5  # tau too small
     assert lib.ts_infonce_fwd_bwd(p, p, None, None, 16, 64, 0.2, 0x1010, p, None, None, 1, None) == -4   # workspace alignment
-    assert lib.ts_infonce_fwd_bwd(p, p, None, None, 16, 64, 0.2, 0x1000, p, None, None, 2, None) == -1   # fp16 unsupported
+    assert lib.ts_infonce_fwd_bwd(p, p, None, None, 16, 64, 0.2, 0x1000, p, None, None, 7, None) == -1   # dtype
     assert lib.ts_bn_stats(None, 2, 3, 4, p, None, None, None, None, 1e-5, None) == -1
     assert lib.ts_bn_stats(p, 2, 70000, 4, p, None, None, None, None, 1e-5, None) == -5
     assert lib.ts_bn_stats(p, 2, 3, 4, p, p, None, None, None, 1e-5, None) == -1                 # sum without sum_squares

@@ -246,6 +246,20 @@ def test_infonce_unnormalised_inputs_and_pair(device):
     assert dots < 2e-2 * d1.grad.float().abs().max().item() * d1.detach().float().norm(dim=1).max().item()
 
 
+@pytest.mark.parametrize("n,c", [(512, 256), (130, 64)])
+def test_infonce_fp16_inputs(device, n, c):
+    # fp16 embeddings (autocast): q and the normalised k are rounded to bf16 for the
+    # contraction, as for fp32 inputs, so the tolerance is the bf16 one; dq is stored in fp16
+    q, k = _nce_inputs(n, c, 17, torch.float16)
+    want, (gw,) = _oracle_grad(lambda a, b: ts_oracle.infonce(a, b, 0.2), q, others=(k,))
+    qd = q.to(device).requires_grad_()
+    loss = ta.infonce_loss(qd, k.to(device), 0.2)
+    loss.backward()
+    assert qd.grad.dtype == torch.float16
+    assert rel_err(loss.item(), want) < 2e-3
+    assert max_rel_to_peak(qd.grad, gw) < 1e-2
+
+
 def test_infonce_fp32_inputs_and_identities(device):
     q, k = _nce_inputs(256, 128, 9, torch.float32)
     want, (gw,) = _oracle_grad(lambda a, b: ts_oracle.infonce(a, b, 0.5), q, others=(k,))

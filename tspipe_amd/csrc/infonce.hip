@@ -21,7 +21,7 @@
 //            normalised and rounded to bf16, are written as "tile images":
 //            for every 32 keys the exact bytes, in the exact order, that the
 //            main kernel's MFMA operand reads want to find in LDS (below).
-//            fp32 queries are also rounded to a bf16 copy here.
+//            fp32 and fp16 queries are also rounded to a bf16 copy here.
 //   main     grid (key split, q tile of 128 rows); 4 wavefronts, each owning
 //            32 q rows; per 32-key tile: S^T = Kh Q^T (MFMA 32x32x16),
 //            P = 2^(S*scale - x_max), l += P, O^T += Kh^T P (MFMA).  Tile
@@ -699,7 +699,7 @@ int ts_infonce_fwd_bwd(const void* q1, const void* k1, const void* q2, const voi
   if ((q2 == nullptr) != (k2 == nullptr)) return TS_ERR_ARG;
   if (n < 0 || !(tau > 0.f)) return TS_ERR_ARG;
   if (c != 64 && c != 128 && c != 256) return TS_ERR_ARG;
-  if (dtype != TS_F32 && dtype != TS_BF16) return TS_ERR_ARG;
+  if (dtype != TS_F32 && dtype != TS_BF16 && dtype != TS_F16) return TS_ERR_ARG;
   // fixed soft-max reference point: 2^(-2 log2(e)/tau) must stay a normal fp32
   if (tau < 0.03f) return TS_ERR_RANGE;
   if (n > (1 << 24)) return TS_ERR_RANGE;
@@ -729,12 +729,14 @@ int ts_infonce_fwd_bwd(const void* q1, const void* k1, const void* q2, const voi
     P.apart = (float*)(wsp + L.off_apart);
     P.opart = (float*)(wsp + L.off_opart);
     P.kimg = (uint8_t*)(wsp + L.off_kimg);
-    P.qb = dtype == TS_F32 ? (uint16_t*)(wsp + L.off_qb) : nullptr;
-    P.qsrc = dtype == TS_F32 ? P.qb : (const uint16_t*)P.q;
+    // fp32 and fp16 queries are rounded to a bf16 copy for the MFMA; bf16 ones are read in place
+    P.qb = dtype != TS_BF16 ? (uint16_t*)(wsp + L.off_qb) : nullptr;
+    P.qsrc = dtype != TS_BF16 ? P.qb : (const uint16_t*)P.q;
   }
   // loss = 2 tau / n * sum over all pairs' rows, written by the combine launch
-  return (dtype == TS_F32) ? ts::nce_dispatch_c<float>(args, pairs, n, c, tau, L, loss_out, st)
-                           : ts::nce_dispatch_c<ts::bf16_t>(args, pairs, n, c, tau, L, loss_out, st);
+  if (dtype == TS_F32) return ts::nce_dispatch_c<float>(args, pairs, n, c, tau, L, loss_out, st);
+  if (dtype == TS_F16) return ts::nce_dispatch_c<ts::f16_t>(args, pairs, n, c, tau, L, loss_out, st);
+  return ts::nce_dispatch_c<ts::bf16_t>(args, pairs, n, c, tau, L, loss_out, st);
 }
 
 }  // extern "C"
