@@ -260,6 +260,26 @@ def test_infonce_fp16_inputs(device, n, c):
     assert max_rel_to_peak(qd.grad, gw) < 1e-2
 
 
+def test_infonce_other_widths_and_argument_errors(device):
+    # widths between the kernels' 64 / 128 / 256 are zero-padded (norms and products unchanged)
+    for n, c in ((100, 96), (65, 200), (40, 24)):
+        q, k = _nce_inputs(n, c, 50 + c, torch.bfloat16)
+        want, (gw,) = _oracle_grad(lambda a, b: ts_oracle.infonce(a, b, 0.2), q, others=(k,))
+        qd = q.to(device).requires_grad_()
+        loss = ta.infonce_loss(qd, k.to(device), 0.2)
+        loss.backward()
+        assert qd.grad.shape == (n, c)
+        assert rel_err(loss.item(), want) < 1e-3
+        err = (qd.grad.cpu().double() - gw).abs()
+        assert (err <= 1e-3 * gw.abs().max() + gw.abs() * 2.0 ** -8).all()
+    q, k = _nce_inputs(8, 320, 1, torch.bfloat16)
+    with pytest.raises(ValueError, match="256 features"):
+        ta.infonce_loss(q.to(device), k.to(device), 0.2)
+    q, k = _nce_inputs(8, 64, 1, torch.bfloat16)
+    with pytest.raises(ValueError, match="temperature"):
+        ta.infonce_loss(q.to(device), k.to(device), 0.01)
+
+
 def test_infonce_fp32_inputs_and_identities(device):
     q, k = _nce_inputs(256, 128, 9, torch.float32)
     want, (gw,) = _oracle_grad(lambda a, b: ts_oracle.infonce(a, b, 0.5), q, others=(k,))

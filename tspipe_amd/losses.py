@@ -437,8 +437,16 @@ class _InfoNCEFn(torch.autograd.Function):
             raise ValueError("InfoNCE expects [batch, features] embeddings")
         if any(t.shape != q1.shape or t.dtype != q1.dtype for t in tensors):
             raise ValueError("InfoNCE inputs must agree in shape and dtype")
-        n, c = int(q1.shape[0]), int(q1.shape[1])
+        n, c_in = int(q1.shape[0]), int(q1.shape[1])
+        if c_in > 256:
+            raise ValueError(f"InfoNCE kernels take embeddings of up to 256 features, got {c_in}")
+        if not tau >= 0.03:
+            raise ValueError(f"InfoNCE kernels need a temperature of at least 0.03, got {tau}")
+        # the kernels come in widths 64, 128 and 256; zero features change neither norms nor products
+        c = 64 if c_in <= 64 else 128 if c_in <= 128 else 256
         prep = [t.detach() if t.is_contiguous() else t.detach().contiguous() for t in tensors]
+        if c != c_in:
+            prep = [torch.nn.functional.pad(t, (0, c - c_in)) for t in prep]
         dev = q1.device
         lib = _lib.lib()
         pairs = 2 if q2 is not None else 1
@@ -454,7 +462,7 @@ class _InfoNCEFn(torch.autograd.Function):
                 None if g1 is None else g1.data_ptr(), None if g2 is None else g2.data_ptr(),
                 _lib.dtype_code(q1.dtype), _lib.current_stream_ptr(dev))
         _lib.check(status, "ts_infonce_fwd_bwd")
-        ctx.g1, ctx.g2, ctx.dims = g1, g2, (n, c)
+        ctx.g1, ctx.g2, ctx.dims, ctx.c_in = g1, g2, (n, c), c_in
         ctx.backward_done = False
         return loss
 
@@ -467,8 +475,10 @@ class _InfoNCEFn(torch.autograd.Function):
         out1 = out2 = None
         if g1 is not None:
             out1 = _scale_saved_grad(g1, grad_output, *ctx.dims)
+            out1 = out1 if ctx.c_in == ctx.dims[1] else out1[:, :ctx.c_in]
         if g2 is not None:
             out2 = _scale_saved_grad(g2, grad_output, *ctx.dims)
+            out2 = out2 if ctx.c_in == ctx.dims[1] else out2[:, :ctx.c_in]
         return out1, None, out2, None, None
 
 
