@@ -410,10 +410,11 @@ def run_kernel_table(dev):
 
     def bwd():
         _lib.check(lib.ts_bn_backward(x.data_ptr(), dy.data_ptr(), mean_b.data_ptr(), inv_b.data_ptr(), gamma.data_ptr(),
-                                      dx.data_ptr(), dgam.data_ptr(), dbet.data_ptr(), wsn.data_ptr(), 32, 256, 3136, 1,
-                                      stream), "ts_bn_backward")
+                                      dx.data_ptr(), dgam.data_ptr(), dbet.data_ptr(), ws4.data_ptr(), par["p"], 32, 256,
+                                      3136, 1, stream), "ts_bn_backward")
+        par["p"] ^= 1
     out["bn_backward_32x256x56x56_f32"] = entry(x.numel() * 20, _time_stream(bwd, 30),
-                                                "bytes = read x,dy twice + write dx", 3)
+                                                "bytes = read x,dy twice + write dx", 2)
     return out
 
 

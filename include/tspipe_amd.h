@@ -329,10 +329,13 @@ int ts_bn_forward_train(const float* x, float* y, const float* gamma, const floa
  *     dx = gamma*invstd*(dy - dbeta/cnt - xhat*dgamma/cnt)
  *   training == 0 (fixed running statistics, batchnorm.py:88-99):
  *     dx = gamma*invstd*dy
- * ws: 2*C floats zero on entry, zero again on return.  dgamma/dbeta: [C]
+ * Two launches: the reduction, then dx, whose workgroups read the two sums
+ * themselves.  ws, parity: as for ts_bn_forward_train (4*C floats, zero before
+ * the first use, two halves used alternately; a layer's forward and backward
+ * calls may share one ws and one alternating parity).  dgamma/dbeta: [C]
  * outputs (required); gamma may be NULL (treated as 1). */
 int ts_bn_backward(const float* x, const float* dy, const float* ub_mean, const float* ub_invstd,
-                   const float* gamma, float* dx, float* dgamma, float* dbeta, float* ws,
+                   const float* gamma, float* dx, float* dgamma, float* dbeta, float* ws, int parity,
                    int64_t N, int64_t C, int64_t HW, int training, ts_stream_t stream);
 
 #ifdef __cplusplus

@@ -158,7 +158,8 @@ def test_device_entry_points_validate_before_launching():
     assert lib.ts_bn_stats(p, 2, 3, 4, p, p, None, None, None, 1e-5, None) == -1                 # sum without sum_squares
     assert lib.ts_bn_commit(p, p, p, p, None, 8, 100.0, -1.0, None) == -1                        # momentum=None needs the counter
     assert lib.ts_bn_apply(p, None, p, p, None, None, 2, 3, 4, 0, 1e-5, None) == -1
-    assert lib.ts_bn_backward(p, p, p, p, None, p, p, None, p, 2, 3, 4, 1, None) == -1
+    assert lib.ts_bn_backward(p, p, p, p, None, p, p, None, p, 0, 2, 3, 4, 1, None) == -1
+    assert lib.ts_bn_backward(p, p, p, p, None, p, p, p, p, 2, 2, 3, 4, 1, None) == -1   # parity
     assert lib.ts_scale_rows(p, 4, 10, 9, p, 0, None) == -1
     assert lib.ts_kd_workspace_bytes(0, 100, 0) == 32 and lib.ts_kd_workspace_bytes(5, 100, 0) == 32 + 3 * 32
     assert lib.ts_kd_workspace_bytes(4096, 30522, 1) == 32 + 3 * 4096 * 4 + 4096 * 4 * 32  # 4 parts per wide row

@@ -18,8 +18,8 @@ pytestmark = pytest.mark.gpu
 
 
 def _check_workspace(bn):
-    # the shared reduction area (backward, stand-alone statistics) is left
-    # clean; of the two halves the training forward alternates between, the
+    # the area of the stand-alone statistics pass is left clean; of the two
+    # halves that the training forward and the backward alternate between, the
     # one the NEXT call will reduce into is zero
     c = bn.num_features
     ws = bn._ws.cpu()
@@ -134,6 +134,36 @@ def test_deferred_bn_backward(device):
     assert max_rel_to_peak(xd.grad, x64.grad) < 1e-5
     assert max_rel_to_peak(bn.weight.grad, w64.grad) < 1e-5
     assert max_rel_to_peak(bn.bias.grad, b64.grad) < 1e-5
+    _check_workspace(bn)
+
+
+def test_deferred_bn_interleaved_forwards_and_backwards(device):
+    # a pipeline runs several micro-batches forward before the first backward, and backward
+    # in another order: the layer's forward and backward calls share one alternating workspace
+    g = seeded(77)
+    C, shape = 12, (5, 12, 8, 6)
+    bn = ta.DeferredBatchNorm(C, chunks=3).to(device)
+    with torch.no_grad():
+        bn.weight.copy_(torch.rand(C, generator=g) + 0.5)
+        bn.bias.copy_(torch.randn(C, generator=g) * 0.1)
+    xs = [_make(shape, 80 + i) for i in range(3)]
+    dys = [torch.randn(shape, generator=g) for _ in range(3)]
+    xd = [x.to(device).requires_grad_() for x in xs]
+    ys = [bn(x) for x in xd]                      # forward 0, 1, 2
+    for i in (2, 0):                              # backward 2, 0
+        ys[i].backward(dys[i].to(device))
+    extra = bn(_make(shape, 90).to(device))       # another forward in between
+    ys[1].backward(dys[1].to(device))             # backward 1
+    torch.cuda.synchronize()
+    w64 = bn.weight.detach().cpu().double().requires_grad_()
+    b64 = bn.bias.detach().cpu().double().requires_grad_()
+    for i in range(3):
+        x64 = xs[i].double().requires_grad_()
+        F.batch_norm(x64, None, None, w64, b64, True, 0.0, 1e-5).backward(dys[i].double())
+        assert max_rel_to_peak(xd[i].grad, x64.grad) < 1e-5
+    assert max_rel_to_peak(bn.weight.grad, w64.grad) < 1e-5
+    assert max_rel_to_peak(bn.bias.grad, b64.grad) < 1e-5
+    assert extra.shape == shape
     _check_workspace(bn)
 
 

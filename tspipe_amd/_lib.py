@@ -60,7 +60,7 @@ SIGNATURES = {
     "ts_bn_forward_train": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p,
                                     c_void_p, c_void_p, c_void_p, c_int, c_float, c_void_p]),
     "ts_bn_backward": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                               c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p]),
+                               c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_int, c_void_p]),
 }
 
 

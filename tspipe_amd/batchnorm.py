@@ -57,7 +57,7 @@ class _NormalizeFn(torch.autograd.Function):
     (``spread`` holds variances, ``eps`` is added on the fly)."""
 
     @staticmethod
-    def forward(ctx, x, weight, bias, mean, spread, ws, training: bool, eps: float):
+    def forward(ctx, x, weight, bias, mean, spread, layer: "DeferredBatchNorm", training: bool, eps: float):
         n, c, hw = _dims(x)
         y = torch.empty_like(x)
         with torch.cuda.device(x.device):
@@ -66,7 +66,7 @@ class _NormalizeFn(torch.autograd.Function):
                                             _lib.current_stream_ptr(x.device))
         _lib.check(status, "ts_bn_apply")
         ctx.save_for_backward(x, weight, mean, spread)
-        ctx.ws = ws
+        ctx.layer = layer
         ctx.training = training
         ctx.eps = eps
         ctx.has_bias = bias is not None
@@ -81,10 +81,14 @@ class _NormalizeFn(torch.autograd.Function):
         dx = torch.empty_like(x)
         dgamma = torch.empty(c, dtype=torch.float32, device=x.device)
         dbeta = torch.empty(c, dtype=torch.float32, device=x.device)
+        layer = ctx.layer
+        ws = layer._workspace(x)
+        parity = layer._parity  # shared with the training forward: the calls of a layer alternate
+        layer._parity = 1 - parity
         with torch.cuda.device(x.device):
             status = _lib.lib().ts_bn_backward(x.data_ptr(), dy.data_ptr(), mean.data_ptr(), invstd.data_ptr(),
                                                _ptr(weight), dx.data_ptr(), dgamma.data_ptr(), dbeta.data_ptr(),
-                                               ctx.ws.data_ptr(), n, c, hw, 1 if ctx.training else 0,
+                                               ws.data_ptr() + 8 * c, parity, n, c, hw, 1 if ctx.training else 0,
                                                _lib.current_stream_ptr(x.device))
         _lib.check(status, "ts_bn_backward")
         return (dx, dgamma if weight is not None else None, dbeta if ctx.has_bias else None,
@@ -112,7 +116,7 @@ class _TrainForwardFn(torch.autograd.Function):
                 float(layer.eps), _lib.current_stream_ptr(x.device))
         _lib.check(status, "ts_bn_forward_train")
         ctx.save_for_backward(x, weight, mean, invstd)
-        ctx.ws = ws
+        ctx.layer = layer
         ctx.training = True
         ctx.eps = float(layer.eps)
         ctx.has_bias = bias is not None
@@ -136,9 +140,9 @@ class DeferredBatchNorm(_BatchNorm):
         self.register_buffer("sum", torch.zeros_like(self.running_mean))
         self.register_buffer("sum_squares", torch.zeros_like(self.running_var))
         # reduction workspace of the kernels, not part of the state dict: 2C
-        # floats that are zero between calls (backward, stand-alone statistics)
-        # and two halves of 2C floats that the training forward alternates
-        # between (``_parity`` says which one the next call reduces into)
+        # floats that are zero between calls (stand-alone statistics) and two
+        # halves of 2C floats that the training forward and the backward
+        # alternate between (``_parity`` says which one the next call reduces into)
         self.register_buffer("_ws", torch.zeros(6 * num_features), persistent=False)
         self._parity = 0
         self.counter = 0
@@ -206,7 +210,7 @@ class DeferredBatchNorm(_BatchNorm):
         if not self.training:
             # fixed running statistics (tspipe/batchnorm.py:88-99)
             return _NormalizeFn.apply(x, weight, bias, self.running_mean, self.running_var,
-                                      self._workspace(x), False, float(self.eps))
+                                      self, False, float(self.eps))
 
         # statistics of this micro-batch into the accumulators
         # (tspipe/batchnorm.py:45-59) and its normalisation (111-120), fused;

@@ -304,25 +304,20 @@ __global__ __launch_bounds__(kBnBlock) void bn_bwd_reduce_kernel(const float* __
   }
 }
 
-__global__ __launch_bounds__(256) void bn_bwd_finalize_kernel(int64_t C, float* __restrict__ ws,
-                                                              float* __restrict__ dgamma,
-                                                              float* __restrict__ dbeta) {
-  const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (c >= C) return;
-  dbeta[c] = ws[c];
-  dgamma[c] = ws[C + c];
-  ws[c] = 0.f;
-  ws[C + c] = 0.f;
-}
-
 // Backward, level 2: dx = gamma*invstd*(dy - dbeta/cnt - xhat*dgamma/cnt).
+// Every workgroup takes its channel's two sums straight from the reduction
+// workspace; the channel's first workgroup also hands them out as dbeta and
+// dgamma and, because its siblings are still reading them, clears the OTHER
+// of the two alternating workspace halves (the one the previous call used).
 __global__ __launch_bounds__(kBnBlock) void bn_bwd_dx_kernel(const float* __restrict__ x,
                                                              const float* __restrict__ dy,
                                                              const float* __restrict__ mean,
                                                              const float* __restrict__ invstd,
                                                              const float* __restrict__ gamma,
-                                                             const float* __restrict__ dgamma,
-                                                             const float* __restrict__ dbeta,
+                                                             const float* __restrict__ ws_sums,
+                                                             float* __restrict__ ws_clear,
+                                                             float* __restrict__ dgamma,
+                                                             float* __restrict__ dbeta,
                                                              float* __restrict__ dx, int64_t N, int64_t C,
                                                              int64_t HW, int64_t slab, float inv_cnt /* 0: fixed statistics */) {
   const int64_t c = blockIdx.y;
@@ -330,7 +325,14 @@ __global__ __launch_bounds__(kBnBlock) void bn_bwd_dx_kernel(const float* __rest
   const int64_t n1 = (n0 + slab < N) ? n0 + slab : N;
   const float mu = mean[c], istd = invstd[c];
   const float gi = (gamma ? gamma[c] : 1.f) * istd;
-  const float mb = dbeta[c] * inv_cnt, mg = dgamma[c] * inv_cnt;
+  const float sum_dy = ws_sums[c], sum_dyx = ws_sums[C + c];
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    dbeta[c] = sum_dy;
+    dgamma[c] = sum_dyx;
+    ws_clear[c] = 0.f;
+    ws_clear[C + c] = 0.f;
+  }
+  const float mb = sum_dy * inv_cnt, mg = sum_dyx * inv_cnt;
   const int tid = threadIdx.x;
   auto one = [=](float xv, float g) { return gi * (g - mb - ((xv - mu) * istd) * mg); };
   for (int64_t n = n0; n < n1; ++n) {
@@ -474,25 +476,24 @@ int ts_bn_forward_train(const float* x, float* y, const float* gamma, const floa
 }
 
 int ts_bn_backward(const float* x, const float* dy, const float* ub_mean, const float* ub_invstd,
-                   const float* gamma, float* dx, float* dgamma, float* dbeta, float* ws, int64_t N,
-                   int64_t C, int64_t HW, int training, ts_stream_t stream) {
+                   const float* gamma, float* dx, float* dgamma, float* dbeta, float* ws, int parity,
+                   int64_t N, int64_t C, int64_t HW, int training, ts_stream_t stream) {
   if (!x || !dy || !ub_mean || !ub_invstd || !dx || !dgamma || !dbeta || !ws) return TS_ERR_ARG;
+  if (parity != 0 && parity != 1) return TS_ERR_ARG;
   int rc = ts::bn_check_dims(N, C, HW);
   if (rc) return rc;
   if (((uintptr_t)x | (uintptr_t)dy | (uintptr_t)dx) & 3u) return TS_ERR_ALIGN;
   const int64_t slab = ts::bn_slab(N, HW);
   dim3 grid((unsigned)((N + slab - 1) / slab), (unsigned)C);
   hipStream_t st = (hipStream_t)stream;
+  float* ws_now = ws + (int64_t)parity * 2 * C;
+  float* ws_other = ws + (int64_t)(1 - parity) * 2 * C;
   hipLaunchKernelGGL(ts::bn_bwd_reduce_kernel, grid, dim3(ts::kBnBlock), 0, st, x, dy, ub_mean, ub_invstd,
-                     N, C, HW, slab, ws);
-  rc = ts::check_launch();
-  if (rc) return rc;
-  hipLaunchKernelGGL(ts::bn_bwd_finalize_kernel, dim3((unsigned)((C + 255) / 256)), dim3(256), 0, st, C,
-                     ws, dgamma, dbeta);
+                     N, C, HW, slab, ws_now);
   rc = ts::check_launch();
   if (rc) return rc;
   hipLaunchKernelGGL(ts::bn_bwd_dx_kernel, grid, dim3(ts::kBnBlock), 0, st, x, dy, ub_mean, ub_invstd,
-                     gamma, dgamma, dbeta, dx, N, C, HW, slab,
+                     gamma, ws_now, ws_other, dgamma, dbeta, dx, N, C, HW, slab,
                      training ? (float)(1.0 / ((double)N * (double)HW)) : 0.f);
   return ts::check_launch();
 }
