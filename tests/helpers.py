@@ -1,8 +1,5 @@
 """Shared input generators and comparison helpers for the parity tests."""
-import numpy as np
 import torch
-
-from shapes import numel
 
 
 def seeded(seed: int) -> torch.Generator:

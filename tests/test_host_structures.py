@@ -14,7 +14,7 @@ import torch
 
 import tspipe_amd as ta
 from oracle import ts_oracle
-from structure_util import attempt, build, describe, load_cases, run_batch_op
+from structure_util import attempt, build, load_cases, run_batch_op
 from tspipe_amd import batch_ops
 
 CASES = load_cases()

@@ -8,8 +8,7 @@ missing, every operation raises.
 import ctypes
 import os
 import threading
-from ctypes import (POINTER, c_char_p, c_double, c_float, c_int, c_int64, c_size_t, c_uint8,
-                    c_void_p)
+from ctypes import c_char_p, c_double, c_float, c_int, c_int64, c_size_t, c_void_p
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libtspipe_amd.so")

@@ -14,9 +14,8 @@ structure bookkeeping whose quirks are kept:
 * non-tensor leaves are replicated on scatter and must compare equal on gather.
 """
 from collections import OrderedDict
-from typing import Any, Callable, List
+from typing import Any, Callable
 
-import torch
 from torch import Tensor
 
 from .model_wrapper import TSPipeModelOutput
