@@ -18,7 +18,7 @@ from typing import Any, Callable
 
 from torch import Tensor
 
-from .model_wrapper import TSPipeModelOutput
+from ._outputs import TSPipeModelOutput
 
 
 def traverse_tensor_map(obj: Any, fn: Callable[[Tensor], Any]) -> Any:
@@ -38,8 +38,7 @@ def traverse_tensor_map(obj: Any, fn: Callable[[Tensor], Any]) -> Any:
         return o
 
     if isinstance(obj, TSPipeModelOutput):
-        return TSPipeModelOutput(data=walk(obj.data),
-                                 lst_require_grad_tensor_path=obj.lst_require_grad_tensor_path)
+        return obj.with_data(walk(obj.data))
     return walk(obj)
 
 
@@ -61,8 +60,7 @@ def generic_object_scatter(obj: Any, chunks: int) -> Any:
         return [o for _ in range(chunks)]
 
     if isinstance(obj, TSPipeModelOutput):
-        return [TSPipeModelOutput(data=piece, lst_require_grad_tensor_path=obj.lst_require_grad_tensor_path)
-                for piece in split(obj.data)]
+        return [obj.with_data(piece) for piece in split(obj.data)]
     return split(obj)
 
 
@@ -129,6 +127,5 @@ def generic_object_gather(*objs: Any) -> Any:
         return resolve(tree, batch_ops.concat_groups(groups))
 
     if all(isinstance(o, TSPipeModelOutput) for o in objs):
-        return TSPipeModelOutput(data=finish(merge(*(o.data for o in objs))),
-                                 lst_require_grad_tensor_path=objs[0].lst_require_grad_tensor_path)
+        return objs[0].with_data(finish(merge(*(o.data for o in objs))))
     return finish(merge(*objs))
