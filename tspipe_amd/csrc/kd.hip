@@ -266,7 +266,7 @@ __device__ __forceinline__ RowGeom row_geom(const T* srow, const T* trow, const 
 // launcher guarantees ceil(V / VEC) + 1 <= KREG * GROUP.
 // ---------------------------------------------------------------------------
 template <typename T, int BLOCK, int GROUP, int KREG, bool CE>
-__global__ __launch_bounds__(BLOCK) void kd_rows_kernel(const KdArgs a) {
+__global__ __launch_bounds__(BLOCK, (KREG * GROUP > 1024 ? 4 : 1)) void kd_rows_kernel(const KdArgs a) {
   constexpr int VEC = Vec16<T>::N;
   constexpr int NW = GROUP / kWave;  // wavefronts per group (0 for sub-wavefront groups)
   __shared__ TStat lds_t[BLOCK / kWave];
@@ -315,7 +315,129 @@ __global__ __launch_bounds__(BLOCK) void kd_rows_kernel(const KdArgs a) {
   // the long-row instantiation is only launched on rows of this kind (checked on the host)
   constexpr bool kAlignedOnly = KREG * GROUP > 1024;
   const int64_t ntail = V - g.tail0;
-  if (kAlignedOnly || (g.head < VEC && ntail < VEC)) {
+  if constexpr (kAlignedOnly) {
+    // Long rows: the packed row pair stays in registers and is walked three
+    // times (maxima, sums, gradient) with the exponentials retaken, which
+    // keeps the kernel at half the registers of the form below, so that two
+    // workgroups share a CU and one's loads overlap the other's arithmetic.
+    const bool has_h = gtid < g.head, has_t = gtid < ntail;
+    float eh_t = kNegBig, eh_s = kNegBig, el_t = kNegBig, el_s = kNegBig;  // end elements: head, last
+    if (has_h) {
+      eh_t = to_f32(trow[gtid]);
+      eh_s = to_f32(srow[gtid]);
+    }
+    if (has_t) {
+      el_t = to_f32(trow[g.tail0 + gtid]);
+      el_s = to_f32(srow[g.tail0 + gtid]);
+    }
+    // Each walk starts from registers the compiler can assume nothing about;
+    // otherwise it would unpack the row once and keep all the fp32 values.
+    auto fresh = [&](int j) {
+      u32x4 bt, bs;
+      __builtin_memcpy(&bt, &rt[j], 16);
+      __builtin_memcpy(&bs, &rs[j], 16);
+      asm volatile("" : "+v"(bt), "+v"(bs));
+      __builtin_memcpy(&rt[j], &bt, 16);
+      __builtin_memcpy(&rs[j], &bs, 16);
+    };
+    float mt = fmaxf(eh_t, el_t), ms = fmaxf(eh_s, el_s);
+#pragma unroll
+    for (int j = 0; j < KREG; ++j) {
+      if (gtid + j * GROUP < (int)g.nvec) {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+          mt = fmaxf(mt, to_f32(rt[j].v[i]));
+          ms = fmaxf(ms, to_f32(rs[j].v[i]));
+        }
+      }
+      // one vector pair at a time: unpacking all of them ahead would double the registers
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    mt = wave_max(mt);
+    ms = wave_max(ms);
+    const int w = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    if (lane == 0) {
+      lds_t[w].m = mt;
+      lds_s[w].m = ms;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < NW; ++i) {
+      mt = fmaxf(mt, lds_t[i].m);
+      ms = fmaxf(ms, lds_s[i].m);
+    }
+    const float mtk = mt * a.k, msk = ms * a.k, ms1 = ms * kLog2e;
+    float zt = 0.f, at = 0.f, zs = 0.f, z1 = 0.f;
+    auto add = [&](float tv, float sv) {
+      const float et = fast_exp2(fmaf(tv, a.k, -mtk));
+      zt += et;
+      zs += fast_exp2(fmaf(sv, a.k, -msk));
+      at = fmaf(et, tv - sv, at);
+      if (CE) z1 += fast_exp2(fmaf(sv, kLog2e, -ms1));
+    };
+    add(eh_t, eh_s);  // a missing end element contributes 2^(-huge) = 0
+    add(el_t, el_s);
+#pragma unroll
+    for (int j = 0; j < KREG; ++j) {
+      if (gtid + j * GROUP < (int)g.nvec) {
+        fresh(j);
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) add(to_f32(rt[j].v[i]), to_f32(rs[j].v[i]));
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    zt = wave_sum(zt);
+    zs = wave_sum(zs);
+    at = wave_sum(at);
+    if (CE) z1 = wave_sum(z1);
+    // .m of both arrays is still being read by slower wavefronts; the sums go into the other fields
+    if (lane == 0) {
+      lds_t[w].z = zt;
+      lds_t[w].a = at;
+      lds_s[w].z = zs;
+      lds_s[w].z1 = z1;
+    }
+    __syncthreads();
+    zt = at = zs = z1 = 0.f;
+#pragma unroll
+    for (int i = 0; i < NW; ++i) {
+      zt += lds_t[i].z;
+      at += lds_t[i].a;
+      zs += lds_s[i].z;
+      z1 += lds_s[i].z1;
+    }
+    const RowFinal f =
+        finish_row<T, CE>(a, job, row, TStat{mt, zt, at}, SStat{ms, zs, z1}, srow, gtid == 0);
+    if (!grow) return;
+    // probabilities first and the weight last, as everywhere in this file
+    const float rt_ = 1.f / zt, rs_ = 1.f / zs, r1_ = CE ? 1.f / z1 : 0.f;
+    const int label = CE ? (int)job.label : -1;  // a row with the CE term has 0 <= label < V
+    auto grad_of = [&](float tv, float sv, int col) {
+      const float et = fast_exp2(fmaf(tv, a.k, -mtk));
+      const float es = fast_exp2(fmaf(sv, a.k, -msk));
+      float gv = f.g_kd * fmaf(es, rs_, -(et * rt_));
+      if (CE) {
+        const float e1 = fast_exp2(fmaf(sv, kLog2e, -ms1));
+        gv = fmaf(f.g_ce, fmaf(e1, r1_, col == label ? -1.f : 0.f), gv);
+      }
+      return from_f32<T>(gv);
+    };
+    if (has_h) grow[gtid] = grad_of(eh_t, eh_s, gtid);
+    if (has_t) grow[g.tail0 + gtid] = grad_of(el_t, el_s, (int)g.tail0 + gtid);
+#pragma unroll
+    for (int j = 0; j < KREG; ++j) {
+      if (gtid + j * GROUP < (int)g.nvec) {
+        fresh(j);
+        Vec16<T> o;
+        const int e0 = (int)g.head + (gtid + j * GROUP) * VEC;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) o.v[i] = grad_of(to_f32(rt[j].v[i]), to_f32(rs[j].v[i]), e0 + i);
+        store16(grow + e0, o);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    return;
+  } else if (g.head < VEC && ntail < VEC) {
     const bool has_h = gtid < g.head, has_t = gtid < ntail;
     float eh_t = kNegBig, eh_s = kNegBig, el_t = kNegBig, el_s = kNegBig;  // end elements: head, last
     if (has_h) {
