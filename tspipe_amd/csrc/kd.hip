@@ -307,19 +307,16 @@ __global__ __launch_bounds__(BLOCK, (KREG * GROUP > 1024 ? 4 : 1)) void kd_rows_
 
   // Rows whose operands share one alignment (the usual case): all but a few
   // end elements are 16-byte vectors held in registers, and each of those end
-  // elements gets a lane of its own.  The maxima come first, then every
-  // exponential is taken once and kept, and the gradient is a multiplication
-  // away.  (With the CE term on long rows the temperature-1 exponentials are
-  // recomputed instead of kept: registers.)
-  constexpr bool kKeepCe = CE && KREG * VEC <= 32;
+  // elements gets a lane of its own.
   // the long-row instantiation is only launched on rows of this kind (checked on the host)
   constexpr bool kAlignedOnly = KREG * GROUP > 1024;
   const int64_t ntail = V - g.tail0;
-  if constexpr (kAlignedOnly) {
-    // Long rows: the packed row pair stays in registers and is walked three
-    // times (maxima, sums, gradient) with the exponentials retaken, which
-    // keeps the kernel at half the registers of the form below, so that two
-    // workgroups share a CU and one's loads overlap the other's arithmetic.
+  if (kAlignedOnly || (g.head < VEC && ntail < VEC)) {
+    // The packed row pair stays in registers and is walked three times
+    // (maxima, sums, gradient), the exponentials being retaken in the third
+    // walk.  Keeping them instead (two per logit pair fewer) was measured no
+    // faster for short rows and slower for long ones: it doubles the
+    // registers, and occupancy is what hides the load latency here.
     const bool has_h = gtid < g.head, has_t = gtid < ntail;
     float eh_t = kNegBig, eh_s = kNegBig, el_t = kNegBig, el_s = kNegBig;  // end elements: head, last
     if (has_h) {
@@ -353,18 +350,23 @@ __global__ __launch_bounds__(BLOCK, (KREG * GROUP > 1024 ? 4 : 1)) void kd_rows_
       // one vector pair at a time: unpacking all of them ahead would double the registers
       __builtin_amdgcn_sched_barrier(0);
     }
-    mt = wave_max(mt);
-    ms = wave_max(ms);
-    const int w = threadIdx.x / kWave, lane = threadIdx.x % kWave;
-    if (lane == 0) {
-      lds_t[w].m = mt;
-      lds_s[w].m = ms;
-    }
-    __syncthreads();
 #pragma unroll
-    for (int i = 0; i < NW; ++i) {
-      mt = fmaxf(mt, lds_t[i].m);
-      ms = fmaxf(ms, lds_s[i].m);
+    for (int off = (GROUP < kWave ? GROUP : kWave) / 2; off > 0; off >>= 1) {
+      mt = fmaxf(mt, __shfl_xor(mt, off, kWave));
+      ms = fmaxf(ms, __shfl_xor(ms, off, kWave));
+    }
+    const int w = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    if (NW > 1) {
+      if (lane == 0) {
+        lds_t[w].m = mt;
+        lds_s[w].m = ms;
+      }
+      __syncthreads();
+#pragma unroll
+      for (int i = 0; i < NW; ++i) {
+        mt = fmaxf(mt, lds_t[i].m);
+        ms = fmaxf(ms, lds_s[i].m);
+      }
     }
     const float mtk = mt * a.k, msk = ms * a.k, ms1 = ms * kLog2e;
     float zt = 0.f, at = 0.f, zs = 0.f, z1 = 0.f;
@@ -386,25 +388,30 @@ __global__ __launch_bounds__(BLOCK, (KREG * GROUP > 1024 ? 4 : 1)) void kd_rows_
       }
       __builtin_amdgcn_sched_barrier(0);
     }
-    zt = wave_sum(zt);
-    zs = wave_sum(zs);
-    at = wave_sum(at);
-    if (CE) z1 = wave_sum(z1);
-    // .m of both arrays is still being read by slower wavefronts; the sums go into the other fields
-    if (lane == 0) {
-      lds_t[w].z = zt;
-      lds_t[w].a = at;
-      lds_s[w].z = zs;
-      lds_s[w].z1 = z1;
-    }
-    __syncthreads();
-    zt = at = zs = z1 = 0.f;
 #pragma unroll
-    for (int i = 0; i < NW; ++i) {
-      zt += lds_t[i].z;
-      at += lds_t[i].a;
-      zs += lds_s[i].z;
-      z1 += lds_s[i].z1;
+    for (int off = (GROUP < kWave ? GROUP : kWave) / 2; off > 0; off >>= 1) {
+      zt += __shfl_xor(zt, off, kWave);
+      zs += __shfl_xor(zs, off, kWave);
+      at += __shfl_xor(at, off, kWave);
+      if (CE) z1 += __shfl_xor(z1, off, kWave);
+    }
+    if (NW > 1) {
+      // .m of both arrays is still being read by slower wavefronts; the sums go into the other fields
+      if (lane == 0) {
+        lds_t[w].z = zt;
+        lds_t[w].a = at;
+        lds_s[w].z = zs;
+        lds_s[w].z1 = z1;
+      }
+      __syncthreads();
+      zt = at = zs = z1 = 0.f;
+#pragma unroll
+      for (int i = 0; i < NW; ++i) {
+        zt += lds_t[i].z;
+        at += lds_t[i].a;
+        zs += lds_s[i].z;
+        z1 += lds_s[i].z1;
+      }
     }
     const RowFinal f =
         finish_row<T, CE>(a, job, row, TStat{mt, zt, at}, SStat{ms, zs, z1}, srow, gtid == 0);
@@ -435,127 +442,6 @@ __global__ __launch_bounds__(BLOCK, (KREG * GROUP > 1024 ? 4 : 1)) void kd_rows_
         store16(grow + e0, o);
       }
       __builtin_amdgcn_sched_barrier(0);
-    }
-    return;
-  } else if (g.head < VEC && ntail < VEC) {
-    const bool has_h = gtid < g.head, has_t = gtid < ntail;
-    float eh_t = kNegBig, eh_s = kNegBig, el_t = kNegBig, el_s = kNegBig;  // end elements: head, last
-    if (has_h) {
-      eh_t = to_f32(trow[gtid]);
-      eh_s = to_f32(srow[gtid]);
-    }
-    if (has_t) {
-      el_t = to_f32(trow[g.tail0 + gtid]);
-      el_s = to_f32(srow[g.tail0 + gtid]);
-    }
-    float xt[KREG][VEC], xs[KREG][VEC], x1[kKeepCe ? KREG : 1][kKeepCe ? VEC : 1];
-    float mt = fmaxf(eh_t, el_t), ms = fmaxf(eh_s, el_s);
-#pragma unroll
-    for (int j = 0; j < KREG; ++j) {
-      const bool live = gtid + (int64_t)j * GROUP < g.nvec;
-#pragma unroll
-      for (int i = 0; i < VEC; ++i) {
-        xt[j][i] = live ? to_f32(rt[j].v[i]) : kNegBig;
-        xs[j][i] = live ? to_f32(rs[j].v[i]) : kNegBig;
-        mt = fmaxf(mt, xt[j][i]);
-        ms = fmaxf(ms, xs[j][i]);
-      }
-    }
-#pragma unroll
-    for (int off = (GROUP < kWave ? GROUP : kWave) / 2; off > 0; off >>= 1) {
-      mt = fmaxf(mt, __shfl_xor(mt, off, kWave));
-      ms = fmaxf(ms, __shfl_xor(ms, off, kWave));
-    }
-    const int w = threadIdx.x / kWave, lane = threadIdx.x % kWave;
-    if (NW > 1) {
-      if (lane == 0) {
-        lds_t[w].m = mt;
-        lds_s[w].m = ms;
-      }
-      __syncthreads();
-#pragma unroll
-      for (int i = 0; i < NW; ++i) {
-        mt = fmaxf(mt, lds_t[i].m);
-        ms = fmaxf(ms, lds_s[i].m);
-      }
-    }
-    const float mtk = mt * a.k, msk = ms * a.k, ms1 = ms * kLog2e;
-    float zt = 0.f, at = 0.f, zs = 0.f, z1 = 0.f;
-    // one (teacher, student) pair: exponentials into the operands' own registers
-    auto take = [&](float& tv, float& sv, float* e1_keep) {
-      const float et = fast_exp2(fmaf(tv, a.k, -mtk));
-      const float es = fast_exp2(fmaf(sv, a.k, -msk));
-      zt += et;
-      zs += es;
-      at = fmaf(et, tv - sv, at);
-      if (CE) {
-        const float e1 = fast_exp2(fmaf(sv, kLog2e, -ms1));
-        z1 += e1;
-        if (e1_keep) *e1_keep = e1;
-      }
-      tv = et;
-      sv = es;
-    };
-    float eh_1 = 0.f, el_1 = 0.f;
-    take(eh_t, eh_s, &eh_1);
-    take(el_t, el_s, &el_1);
-#pragma unroll
-    for (int j = 0; j < KREG; ++j)
-#pragma unroll
-      for (int i = 0; i < VEC; ++i) take(xt[j][i], xs[j][i], kKeepCe ? &x1[j][i] : nullptr);
-#pragma unroll
-    for (int off = (GROUP < kWave ? GROUP : kWave) / 2; off > 0; off >>= 1) {
-      zt += __shfl_xor(zt, off, kWave);
-      zs += __shfl_xor(zs, off, kWave);
-      at += __shfl_xor(at, off, kWave);
-      if (CE) z1 += __shfl_xor(z1, off, kWave);
-    }
-    if (NW > 1) {
-      // .m of both arrays is still being read by slower wavefronts; the sums
-      // go into the other fields
-      if (lane == 0) {
-        lds_t[w].z = zt;
-        lds_t[w].a = at;
-        lds_s[w].z = zs;
-        lds_s[w].z1 = z1;
-      }
-      __syncthreads();
-      zt = at = zs = z1 = 0.f;
-#pragma unroll
-      for (int i = 0; i < NW; ++i) {
-        zt += lds_t[i].z;
-        at += lds_t[i].a;
-        zs += lds_s[i].z;
-        z1 += lds_s[i].z1;
-      }
-    }
-    const RowFinal f =
-        finish_row<T, CE>(a, job, row, TStat{mt, zt, at}, SStat{ms, zs, z1}, srow, gtid == 0);
-    if (!grow) return;
-    // probabilities first and the weight last, as the general path does: a
-    // weight folded into the reciprocals would be amplified by the cancellation in q - p
-    const float rt_ = 1.f / zt, rs_ = 1.f / zs, r1_ = CE ? 1.f / z1 : 0.f;
-    auto grad_of = [&](float et, float es, float e1, int64_t col) {
-      float gv = f.g_kd * fmaf(es, rs_, -(et * rt_));
-      if (CE) gv = fmaf(f.g_ce, fmaf(e1, r1_, col == job.label ? -1.f : 0.f), gv);
-      return from_f32<T>(gv);
-    };
-    if (has_h) grow[gtid] = grad_of(eh_t, eh_s, eh_1, gtid);
-    if (has_t) grow[g.tail0 + gtid] = grad_of(el_t, el_s, el_1, g.tail0 + gtid);
-#pragma unroll
-    for (int j = 0; j < KREG; ++j) {
-      const int64_t v = gtid + (int64_t)j * GROUP;
-      if (v < g.nvec) {
-        Vec16<T> o;
-        const int64_t e0 = g.head + v * VEC;
-#pragma unroll
-        for (int i = 0; i < VEC; ++i) {
-          float e1 = 0.f;
-          if (CE) e1 = kKeepCe ? x1[j][i] : fast_exp2(fmaf(to_f32(rs[j].v[i]), kLog2e, -ms1));
-          o.v[i] = grad_of(xt[j][i], xs[j][i], e1, e0 + i);
-        }
-        store16(grow + e0, o);
-      }
     }
     return;
   }
