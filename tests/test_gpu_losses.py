@@ -43,7 +43,7 @@ def test_kd_cfg2_fp32(device):
 
 
 @pytest.mark.parametrize("rows,V", [(1, 1), (3, 5), (7, 63), (5, 64), (4, 65), (9, 1000), (2, 2049), (3, 4099),
-                                    (5, 8191), (2, 16380), (2, 16381)])
+                                    (5, 8191), (2, 16380), (2, 16381), (2, 32760), (2, 32761)])
 def test_kd_shapes_fp32(device, rows, V):
     g = seeded(100 + V)
     s = torch.randn(rows, V, generator=g) * 3
@@ -56,10 +56,12 @@ def test_kd_shapes_fp32(device, rows, V):
     assert max_rel_to_peak(sd.grad, gw) < 2e-5 or gw.abs().max() < 1e-12
 
 
-@pytest.mark.parametrize("rows,V", [(5, 4097), (4, 9001), (3, 30522), (2, 32760), (2, 32761)])
+@pytest.mark.parametrize("rows,V", [(5, 4097), (4, 9001), (3, 30522), (2, 32760), (2, 32761), (3, 50257), (2, 65520),
+                                    (2, 65521)])
 def test_kd_long_rows_bf16_unmasked(device, rows, V):
-    # rows of 8 K to 32 K bf16 logits without a mask: one launch with the row pair in registers
-    # (up to 32760 elements, here also with rows that start off a 16-byte boundary), two passes beyond
+    # rows of 8 K to 64 K bf16 logits without a mask: one launch with the row pair in registers
+    # (512 threads per row up to 32760 elements, 1024 up to 65520, here also with rows that start
+    # off a 16-byte boundary), two passes beyond
     g = seeded(300 + V)
     s = (torch.randn(rows, V, generator=g) * 2).to(torch.bfloat16)
     t = (torch.randn(rows, V, generator=g) * 2).to(torch.bfloat16)

@@ -905,10 +905,10 @@ int launch_kd_t(KdArgs a, float kd_scale, void* ws, float* loss_out, hipStream_t
   int rc = TS_OK;
   const int64_t vecs_ = (a.V + Vec16<T>::N - 1) / Vec16<T>::N + 1;
   // Long rows without a mask (every row carries the KD term), operands aligned
-  // alike: one launch, the row pair held in the registers of a 512-thread
-  // workgroup.  Under a mask the two-pass form below stays: it overlaps the
+  // alike: one launch, the row pair held in the registers of a 512- or
+  // 1024-thread workgroup.  Under a mask the two-pass form below stays: it overlaps the
   // zero-fill of the rows without a term with the arithmetic of the others.
-  const bool one_launch = a.n_rows > 0 && parts > 0 && !a.mask && vecs_ <= 512 * 8 && kd_rows_aligned_alike<T>(a);
+  const bool one_launch = a.n_rows > 0 && parts > 0 && !a.mask && vecs_ <= 1024 * 8 && kd_rows_aligned_alike<T>(a);
   const bool wide = a.n_rows > 0 && parts > 0 && !one_launch;
   if (counted && !wide) {
     hipLaunchKernelGGL(kd_count_kernel, dim3(1), dim3(1024), 0, stream, a, w.counts,
@@ -935,8 +935,10 @@ int launch_kd_t(KdArgs a, float kd_scale, void* ws, float* loss_out, hipStream_t
     TS_KD_LAUNCH(256, 64, 4);
   } else if (parts == 0) {
     TS_KD_LAUNCH(256, 256, 4);
-  } else if (one_launch) {
+  } else if (one_launch && vecs <= 512 * 8) {
     TS_KD_LAUNCH(512, 512, 8);
+  } else if (one_launch) {
+    TS_KD_LAUNCH(1024, 1024, 8);
   } else {
     const int64_t items = a.n_rows * parts;
     if (items > 0x7fffffffLL) return TS_ERR_RANGE;
