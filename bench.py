@@ -296,6 +296,14 @@ def run_kernel_table(dev):
         out[name] = entry(3 * rows * 100 * 4, _time_stream(f, 50),
                           "latency-bound: 2 launches of a few us each" if rows == 256 else None, 2)
 
+    # an ImageNet-sized class count (not one of the benchmark configurations): rows long enough to stream
+    s = (torch.randn(32768, 1000, generator=g) * 3).to(dev)
+    t = (torch.randn(32768, 1000, generator=g) * 3).to(dev)
+    f = kd_call(s, t, None, 4.0, torch.empty_like(s))
+    out["kd_32768x1000_f32"] = entry(3 * 32768 * 1000 * 4, _time_stream(f, 30),
+                                     "not one of the benchmark configurations", 2)
+    del s, t, f
+
     # DistilBERT-shaped masked KD (cfg3) after a gather of 4 micro-batches
     pieces_s = [(torch.randn(8, 128, 30522, generator=g) * 2).to(torch.bfloat16).to(dev) for _ in range(4)]
     pieces_t = [(torch.randn(8, 128, 30522, generator=g) * 2).to(torch.bfloat16).to(dev) for _ in range(4)]
