@@ -266,18 +266,24 @@ __device__ __forceinline__ RowGeom row_geom(const T* srow, const T* trow, const 
 // launcher guarantees ceil(V / VEC) + 1 <= KREG * GROUP.
 // ---------------------------------------------------------------------------
 template <typename T, int BLOCK, int GROUP, int KREG, bool CE>
-__global__ __launch_bounds__(BLOCK, (KREG * GROUP > 1024 ? 4 : 1)) void kd_rows_kernel(const KdArgs a) {
+__global__ __launch_bounds__(BLOCK, (KREG * GROUP > 1024 ? 4 : 1)) void kd_rows_kernel(
+    const KdArgs a, const int* __restrict__ sel_rows) {
   constexpr int VEC = Vec16<T>::N;
   constexpr int NW = GROUP / kWave;  // wavefronts per group (0 for sub-wavefront groups)
   __shared__ TStat lds_t[BLOCK / kWave];
   __shared__ SStat lds_s[BLOCK / kWave];
 
   const int gtid = threadIdx.x % GROUP;
-  const int64_t row = (int64_t)blockIdx.x * (BLOCK / GROUP) + threadIdx.x / GROUP;
+  int64_t row = (int64_t)blockIdx.x * (BLOCK / GROUP) + threadIdx.x / GROUP;
   // With GROUP == BLOCK the whole workgroup shares one row, so the early
   // exits below are uniform; smaller groups never reach a __syncthreads and
   // only shuffle among their own lanes.
   if (row >= a.n_rows) return;
+  if (sel_rows) {
+    // the grid walks the compacted list of the rows that carry a loss term
+    if (row >= a.counts[2]) return;
+    row = sel_rows[row];
+  }
   const KdRowPtrs<T> rp = kd_row_ptrs<T>(a, row);
   const T* srow = rp.s;
   const T* trow = rp.t;
@@ -566,6 +572,23 @@ __device__ __forceinline__ void kd_zero_part(const KdArgs& a, int64_t row, int p
     const int64_t v = v0 + tid + j * kPartBlock;
     if (v < nvec) store16(grow + head + v * VEC, z);
   }
+}
+
+// Long rows under a mask: workgroup 0 counts and compacts the rows that carry
+// a term, every other workgroup owns one (row, part) and zero-fills it if the
+// row carries none.  The row kernel then walks the compacted list.
+template <typename T, bool CE>
+__global__ __launch_bounds__(kPartBlock) void kd_zero_rows_kernel(const KdArgs a, int parts,
+                                                                  int* __restrict__ count_out,
+                                                                  int* __restrict__ sel_rows_out) {
+  if (blockIdx.x == 0) {
+    kd_count_block<kPartBlock>(a, count_out, sel_rows_out);
+    return;
+  }
+  const int64_t item = (int64_t)blockIdx.x - 1;
+  const int64_t row = item / parts;
+  const RowJob job = row_job(a, row);
+  if (!job.kd && !job.ce) kd_zero_part<T, CE>(a, row, (int)(item % parts), parts);
 }
 
 // With count_out set, workgroup 0 does the row counting and compaction that
@@ -904,13 +927,23 @@ int launch_kd_t(KdArgs a, float kd_scale, void* ws, float* loss_out, hipStream_t
   const bool compact = parts && counted;
   int rc = TS_OK;
   const int64_t vecs_ = (a.V + Vec16<T>::N - 1) / Vec16<T>::N + 1;
-  // Long rows without a mask (every row carries the KD term), operands aligned
-  // alike: one launch, the row pair held in the registers of a 512- or
-  // 1024-thread workgroup.  Under a mask the two-pass form below stays: it overlaps the
-  // zero-fill of the rows without a term with the arithmetic of the others.
-  const bool one_launch = a.n_rows > 0 && parts > 0 && !a.mask && vecs_ <= 1024 * 8 && kd_rows_aligned_alike<T>(a);
+  // Long rows, operands aligned alike: the row pair held in the registers of a
+  // 512- or 1024-thread workgroup, one launch.  Under a mask the rows without
+  // a term are zero-filled by a launch of their own in front (which also
+  // counts and compacts) and the row kernel walks the compacted list: as fast
+  // as the two passes below when few rows are selected, and much faster when
+  // most are.  The two passes remain for wider or differently aligned rows.
+  const bool one_launch = a.n_rows > 0 && parts > 0 && vecs_ <= 1024 * 8 && kd_rows_aligned_alike<T>(a);
   const bool wide = a.n_rows > 0 && parts > 0 && !one_launch;
-  if (counted && !wide) {
+  const bool zero_first = one_launch && a.mask;
+  if (zero_first) {
+    const int64_t zparts = (vecs_ + kPartVecs - 1) / kPartVecs;
+    if (a.n_rows * zparts > 0x7ffffff0LL) return TS_ERR_RANGE;
+    hipLaunchKernelGGL((kd_zero_rows_kernel<T, CE>), dim3((unsigned)(a.n_rows * zparts + 1)), dim3(kPartBlock), 0,
+                       stream, a, (int)zparts, w.counts, w.sel_rows);
+    rc = check_launch();
+    if (rc) return rc;
+  } else if (counted && !wide) {
     hipLaunchKernelGGL(kd_count_kernel, dim3(1), dim3(1024), 0, stream, a, w.counts,
                        compact ? w.sel_rows : (int*)nullptr);
     rc = check_launch();
@@ -926,7 +959,8 @@ int launch_kd_t(KdArgs a, float kd_scale, void* ws, float* loss_out, hipStream_t
 #define TS_KD_LAUNCH(BLOCK, GROUP, KREG)                                                                     \
   hipLaunchKernelGGL((kd_rows_kernel<T, BLOCK, GROUP, KREG, CE>),                                            \
                      dim3((unsigned)((a.n_rows + (BLOCK / GROUP) - 1) / (BLOCK / GROUP))), dim3(BLOCK), 0,   \
-                     stream, a)
+                     stream, a, sel)
+  const int* sel = nullptr;
   if (vecs <= 16 * 2) {
     TS_KD_LAUNCH(256, 16, 2);
   } else if (vecs <= 32 * 2) {
@@ -936,8 +970,10 @@ int launch_kd_t(KdArgs a, float kd_scale, void* ws, float* loss_out, hipStream_t
   } else if (parts == 0) {
     TS_KD_LAUNCH(256, 256, 4);
   } else if (one_launch && vecs <= 512 * 8) {
+    sel = zero_first ? w.sel_rows : nullptr;
     TS_KD_LAUNCH(512, 512, 8);
   } else if (one_launch) {
+    sel = zero_first ? w.sel_rows : nullptr;
     TS_KD_LAUNCH(1024, 1024, 8);
   } else {
     const int64_t items = a.n_rows * parts;
