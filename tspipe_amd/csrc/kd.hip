@@ -278,12 +278,22 @@ __global__ __launch_bounds__(BLOCK, (KREG * GROUP > 1024 ? 4 : 1)) void kd_rows_
   // With GROUP == BLOCK the whole workgroup shares one row, so the early
   // exits below are uniform; smaller groups never reach a __syncthreads and
   // only shuffle among their own lanes.
-  if (row >= a.n_rows) return;
   if (sel_rows) {
-    // the grid walks the compacted list of the rows that carry a loss term
-    if (row >= a.counts[2]) return;
-    row = sel_rows[row];
+    // Masked long rows (one row per workgroup, grid of 2 n_rows): the first
+    // n_rows workgroups walk the compacted list of the rows that carry a loss
+    // term, so that the long-running ones all start first; the next n_rows
+    // zero-fill the rows that carry none.  (Interleaving the two kinds, singly
+    // or in runs of eight, was measured slower than this order.)
+    if (row >= a.n_rows) {
+      row -= a.n_rows;
+      const RowJob j0 = row_job(a, row);
+      if (j0.kd || j0.ce) return;
+    } else {
+      if (row >= a.counts[2]) return;
+      row = sel_rows[row];
+    }
   }
+  if (row >= a.n_rows) return;
   const KdRowPtrs<T> rp = kd_row_ptrs<T>(a, row);
   const T* srow = rp.s;
   const T* trow = rp.t;
@@ -572,23 +582,6 @@ __device__ __forceinline__ void kd_zero_part(const KdArgs& a, int64_t row, int p
     const int64_t v = v0 + tid + j * kPartBlock;
     if (v < nvec) store16(grow + head + v * VEC, z);
   }
-}
-
-// Long rows under a mask: workgroup 0 counts and compacts the rows that carry
-// a term, every other workgroup owns one (row, part) and zero-fills it if the
-// row carries none.  The row kernel then walks the compacted list.
-template <typename T, bool CE>
-__global__ __launch_bounds__(kPartBlock) void kd_zero_rows_kernel(const KdArgs a, int parts,
-                                                                  int* __restrict__ count_out,
-                                                                  int* __restrict__ sel_rows_out) {
-  if (blockIdx.x == 0) {
-    kd_count_block<kPartBlock>(a, count_out, sel_rows_out);
-    return;
-  }
-  const int64_t item = (int64_t)blockIdx.x - 1;
-  const int64_t row = item / parts;
-  const RowJob job = row_job(a, row);
-  if (!job.kd && !job.ce) kd_zero_part<T, CE>(a, row, (int)(item % parts), parts);
 }
 
 // With count_out set, workgroup 0 does the row counting and compaction that
@@ -935,17 +928,10 @@ int launch_kd_t(KdArgs a, float kd_scale, void* ws, float* loss_out, hipStream_t
   // most are.  The two passes remain for wider or differently aligned rows.
   const bool one_launch = a.n_rows > 0 && parts > 0 && vecs_ <= 1024 * 8 && kd_rows_aligned_alike<T>(a);
   const bool wide = a.n_rows > 0 && parts > 0 && !one_launch;
-  const bool zero_first = one_launch && a.mask;
-  if (zero_first) {
-    const int64_t zparts = (vecs_ + kPartVecs - 1) / kPartVecs;
-    if (a.n_rows * zparts > 0x7ffffff0LL) return TS_ERR_RANGE;
-    hipLaunchKernelGGL((kd_zero_rows_kernel<T, CE>), dim3((unsigned)(a.n_rows * zparts + 1)), dim3(kPartBlock), 0,
-                       stream, a, (int)zparts, w.counts, w.sel_rows);
-    rc = check_launch();
-    if (rc) return rc;
-  } else if (counted && !wide) {
+  const bool compacted = one_launch && a.mask;  // the row kernel walks the compacted list, then zero-fills
+  if (counted && !wide) {
     hipLaunchKernelGGL(kd_count_kernel, dim3(1), dim3(1024), 0, stream, a, w.counts,
-                       compact ? w.sel_rows : (int*)nullptr);
+                       (compact || compacted) ? w.sel_rows : (int*)nullptr);
     rc = check_launch();
     if (rc) return rc;
   }
@@ -959,8 +945,7 @@ int launch_kd_t(KdArgs a, float kd_scale, void* ws, float* loss_out, hipStream_t
 #define TS_KD_LAUNCH(BLOCK, GROUP, KREG)                                                                     \
   hipLaunchKernelGGL((kd_rows_kernel<T, BLOCK, GROUP, KREG, CE>),                                            \
                      dim3((unsigned)((a.n_rows + (BLOCK / GROUP) - 1) / (BLOCK / GROUP))), dim3(BLOCK), 0,   \
-                     stream, a, sel)
-  const int* sel = nullptr;
+                     stream, a, (const int*)nullptr)
   if (vecs <= 16 * 2) {
     TS_KD_LAUNCH(256, 16, 2);
   } else if (vecs <= 32 * 2) {
@@ -969,12 +954,14 @@ int launch_kd_t(KdArgs a, float kd_scale, void* ws, float* loss_out, hipStream_t
     TS_KD_LAUNCH(256, 64, 4);
   } else if (parts == 0) {
     TS_KD_LAUNCH(256, 256, 4);
-  } else if (one_launch && vecs <= 512 * 8) {
-    sel = zero_first ? w.sel_rows : nullptr;
-    TS_KD_LAUNCH(512, 512, 8);
   } else if (one_launch) {
-    sel = zero_first ? w.sel_rows : nullptr;
-    TS_KD_LAUNCH(1024, 1024, 8);
+    if (2 * a.n_rows > 0x7fffffffLL) return TS_ERR_RANGE;
+    const dim3 grid((unsigned)(compacted ? 2 * a.n_rows : a.n_rows));
+    const int* sel = compacted ? w.sel_rows : nullptr;
+    if (vecs <= 512 * 8)
+      hipLaunchKernelGGL((kd_rows_kernel<T, 512, 512, 8, CE>), grid, dim3(512), 0, stream, a, sel);
+    else
+      hipLaunchKernelGGL((kd_rows_kernel<T, 1024, 1024, 8, CE>), grid, dim3(1024), 0, stream, a, sel);
   } else {
     const int64_t items = a.n_rows * parts;
     if (items > 0x7fffffffLL) return TS_ERR_RANGE;
