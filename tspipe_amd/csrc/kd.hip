@@ -2,9 +2,11 @@
 //   KD soft target   KL(softmax(t/T) || softmax(s/T)) over rows selected by a mask,
 //   hard-label CE    cross entropy of softmax(s) against integer labels with an
 //                    ignore index, optionally in the same pass over the rows.
-// A "group" of threads owns a row: 16/32/64 lanes of a wavefront for narrow
-// rows, a 256-thread workgroup for medium ones; wide (vocabulary-sized) rows
-// are cut into parts handled by short-lived workgroups in two launches.
+// A "group" of threads owns a row and holds it in registers: 16/32/64 lanes of
+// a wavefront for narrow rows, a 256-, 512- or 1024-thread workgroup for rows
+// of up to 8192 16-byte vectors (vocabulary-sized rows included); wider rows,
+// and long rows whose operands are aligned differently, are cut into parts
+// handled by short-lived workgroups in two launches.
 // Accumulation is fp32 in the log2 domain (v_exp_f32 / v_log_f32); storage is
 // fp32, bf16 or fp16.
 #include "common.h"
@@ -260,7 +262,7 @@ __device__ __forceinline__ RowGeom row_geom(const T* srow, const T* trow, const 
 }
 
 // ---------------------------------------------------------------------------
-// Narrow and medium rows: one launch.  The row pair is held in registers
+// Rows of up to 8192 vectors: one launch.  The row pair is held in registers
 // between the statistics and the gradient (KREG 16-byte vectors per thread
 // and operand, all loads issued up front), so each logit is read once; the
 // launcher guarantees ceil(V / VEC) + 1 <= KREG * GROUP.
