@@ -179,6 +179,42 @@ def test_kd_mask_special_cases(device):
     assert rel_err(ta.distil_ce_loss(sd, td, att.to(device), 2.0).item(), want) < 1e-5
 
 
+@pytest.mark.parametrize("V,dtype", [(9001, torch.bfloat16), (40000, torch.bfloat16), (5000, torch.float32)])
+def test_kd_mask_special_cases_long_rows(device, V, dtype):
+    # the same special cases on rows long enough for the one-workgroup-per-row kernel, whose grid
+    # under a mask holds the compacted selected rows first and the zero-fill of the others after them
+    g = seeded(300 + V)
+    rows = 7
+    s = (torch.randn(1, rows, V, generator=g) * 2).to(dtype)
+    t = (torch.randn(1, rows, V, generator=g) * 2).to(dtype)
+    sd, td = s.to(device), t.to(device)
+    tol = 1e-5 if dtype == torch.float32 else 1e-3
+    full = torch.ones(1, rows, dtype=torch.bool)
+    a = ta.distil_ce_loss(sd, td, full.to(device), 2.0).item()
+    b = ta.kd_soft_target_loss(sd.view(-1, V), td.view(-1, V), 2.0).item()
+    assert rel_err(a, b) < 1e-6
+    for pick in ([3], [0, 6], [1, 2, 4, 5]):
+        m = torch.zeros(1, rows, dtype=torch.bool)
+        m[0, pick] = True
+        x = sd.clone().requires_grad_()
+        l = ta.distil_ce_loss(x, td, m.to(device), 2.0)
+        l.backward()
+        ref_s = s.double().requires_grad_()
+        want = ts_oracle.distil_ce(ref_s, t.double(), m, 2.0)
+        want.backward()
+        assert rel_err(l.item(), want.item()) < tol
+        gw = ref_s.grad
+        err = (x.grad.cpu().double() - gw).abs()
+        assert (err <= tol * gw.abs().max() + gw.abs() * 2.0 ** -8).all()
+        assert (x.grad[0, [i for i in range(rows) if i not in pick]] == 0).all()
+    none = torch.zeros(1, rows, dtype=torch.bool)
+    x = sd.clone().requires_grad_()
+    l = ta.distil_ce_loss(x, td, none.to(device), 2.0)
+    l.backward()
+    assert torch.isnan(l).item()
+    assert (x.grad == 0).all()
+
+
 def test_byol_fp32(device):
     g = seeded(5)
     o1, o2, t1, t2 = [torch.randn(256, 128, generator=g) for _ in range(4)]
