@@ -22,7 +22,7 @@
 //            for every 32 keys the exact bytes, in the exact order, that the
 //            main kernel's MFMA operand reads want to find in LDS (below).
 //            fp32 and fp16 queries are also rounded to a bf16 copy here.
-//   main     grid (key split, q tile of 128 rows); 4 wavefronts, each owning
+//   main     grid (q tile of 128 rows, key split); 4 wavefronts, each owning
 //            32 q rows; per 32-key tile: S^T = Kh Q^T (MFMA 32x32x16),
 //            P = 2^(S*scale - x_max), l += P, O^T += Kh^T P (MFMA).  Tile
 //            images go from global memory straight into LDS (no registers),
@@ -245,7 +245,7 @@ constexpr int kNceBufs = 4;  // tile images in LDS: two in use (tiles t, t+1), t
 
 template <int C>
 __global__ __launch_bounds__(kNceBlock) void nce_main_kernel(NceArgs args, int64_t n, int64_t npad, int splits,
-                                                             float scale2 /* log2(e)/tau */) {
+                                                             float scale2 /* log2(e)/tau */, int qtile_major) {
   const NcePair& pr = args.p[blockIdx.z];
   const uint16_t* __restrict__ qg = pr.qsrc;
   const uint8_t* __restrict__ kimg = pr.kimg;
@@ -258,11 +258,13 @@ __global__ __launch_bounds__(kNceBlock) void nce_main_kernel(NceArgs args, int64
   __shared__ __attribute__((aligned(16))) uint8_t sm[kNceBufs][TI::BYTES];
   const int tid = threadIdx.x, lane = tid % kWave, w = tid / kWave;
   const int col = lane % 32, h = lane / 32;
-  // Workgroup ids are dealt round-robin to the 8 XCDs.  With the key split as
-  // the fastest index (and 8 splits), every XCD keeps seeing the same eighth
-  // of the key images, which then stays in that XCD's own L2.
-  const int split = blockIdx.x;
-  const int64_t qtile = blockIdx.y;
+  // Workgroup ids are dealt round-robin to the 8 XCDs.  While all key images
+  // fit an XCD's L2 (4 MB at N = 4096), the q tile is the fastest index: the
+  // key splits of a q tile run on one XCD, which streams every image through
+  // its L2 (measured 5 % faster there).  For more keys the split is the
+  // fastest index, so that an XCD keeps seeing the same share of the images.
+  const int split = qtile_major ? blockIdx.y : blockIdx.x;
+  const int64_t qtile = qtile_major ? blockIdx.x : blockIdx.y;
   const int64_t qrow = qtile * kQTile + w * 32 + col;  // the q row this lane is a column of
 
   const int64_t ktiles = npad / kKTile;
@@ -660,8 +662,12 @@ int nce_run(const NceArgs& args, int pairs, int64_t n, float tau, const NceLayou
                      n, L.npad, scale2);
   int rc = check_launch();
   if (rc) return rc;
-  hipLaunchKernelGGL((nce_main_kernel<C>), dim3((unsigned)L.splits, (unsigned)(L.npad / kQTile), z), dim3(kNceBlock),
-                     0, stream, args, n, L.npad, L.splits, scale2);
+  // see the kernel for the choice of the fastest grid index
+  const bool qtile_major = (size_t)L.npad * C * 4 <= ((size_t)4 << 20);
+  const dim3 main_grid = qtile_major ? dim3((unsigned)(L.npad / kQTile), (unsigned)L.splits, z)
+                                     : dim3((unsigned)L.splits, (unsigned)(L.npad / kQTile), z);
+  hipLaunchKernelGGL((nce_main_kernel<C>), main_grid, dim3(kNceBlock), 0, stream, args, n, L.npad, L.splits, scale2,
+                     qtile_major ? 1 : 0);
   rc = check_launch();
   if (rc) return rc;
   const int64_t items = L.npad / 32 * (C / 32);  // a multiple of 4: npad is a multiple of 128
