@@ -12,8 +12,11 @@
  *   - every "dev" pointer is device memory owned by the caller and must stay
  *     alive until the work enqueued on `stream` has run;
  *   - `stream` is a hipStream_t passed as void* (NULL = the null stream);
- *   - calls only enqueue work: no implicit synchronisation, no allocation, no
- *     global mutable state; re-entrant from any thread;
+ *   - calls only enqueue work: no implicit synchronisation and no allocation;
+ *     re-entrant from any thread.  State the library keeps: per thread, the
+ *     HIP error of the last failed launch (ts_last_hip_error) and the event
+ *     pair armed by ts_time_next_launch; per process, the address of the
+ *     fixed scratch array of ts_kd_fwd_bwd_static, looked up once per GPU;
  *   - workspaces are caller-provided; sizes are stated per function;
  *   - "plan" functions are pure host code (no GPU needed): they turn tensor
  *     lists into the chunk tables the kernels walk.
@@ -161,6 +164,21 @@ int ts_kd_fwd_bwd(const void* s, const void* t, const uint8_t* row_mask, int64_t
                   int64_t V, int64_t ld_s, int64_t ld_t, float inv_T, float loss_scale,
                   void* workspace, float* loss_out, void* grad, int64_t ld_g, int dtype,
                   ts_stream_t stream);
+
+/* ts_kd_fwd_bwd for callers that cannot allocate device memory (code under
+ * HIP graph capture, serving loops and harnesses that forbid hipMalloc): no
+ * counterpart in the reference.  Same arguments without the workspace, same
+ * kernels and results; the workspace is a fixed array inside the library
+ * (ts_kd_static_scratch_bytes() bytes, one copy per GPU, held until the
+ * process ends).  Shapes whose ts_kd_workspace_bytes() exceeds that size are
+ * refused with TS_ERR_RANGE.  The call allocates nothing.  Every call on a GPU
+ * uses that GPU's one array: calls that may overlap on the same GPU (two
+ * streams, two threads) race and must be serialised by the caller. */
+size_t ts_kd_static_scratch_bytes(void);
+
+int ts_kd_fwd_bwd_static(const void* s, const void* t, const uint8_t* row_mask, int64_t n_rows,
+                         int64_t V, int64_t ld_s, int64_t ld_t, float inv_T, float loss_scale,
+                         float* loss_out, void* grad, int64_t ld_g, int dtype, ts_stream_t stream);
 
 /* The same pass with the hard-label cross entropy added, the combination the
  * reference's distillation plug-ins compute on the student logits:

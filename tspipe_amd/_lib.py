@@ -34,6 +34,9 @@ SIGNATURES = {
     "ts_kd_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int]),
     "ts_kd_fwd_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_float,
                               c_float, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_void_p]),
+    "ts_kd_static_scratch_bytes": (c_size_t, []),
+    "ts_kd_fwd_bwd_static": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_float,
+                                     c_float, c_void_p, c_void_p, c_int64, c_int, c_void_p]),
     "ts_kdce_fwd_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64,
                                 c_float, c_float, c_float, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_void_p]),
     "ts_kdce_pieces_fwd_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int64, c_int64,

@@ -9,9 +9,44 @@
 // handled by short-lived workgroups in two launches.
 // Accumulation is fp32 in the log2 domain (v_exp_f32 / v_log_f32); storage is
 // fp32, bf16 or fp16.
+#include <mutex>
+
 #include "common.h"
 
 namespace ts {
+
+// Scratch of ts_kd_fwd_bwd_static: one copy per GPU, held until the process
+// ends.  In host code the array's name is only a handle for
+// hipGetSymbolAddress; kernels are handed the address it returns.
+constexpr size_t kKdStaticScratchBytes = (size_t)1 << 20;
+static __device__ __align__(256) unsigned char kd_static_scratch[kKdStaticScratchBytes];
+constexpr int kKdMaxDevices = 64;
+static std::mutex g_kd_scratch_lock;
+static void* g_kd_scratch_ptr[kKdMaxDevices];  // device address of the array, per device ordinal
+
+// Address of the current device's copy of the scratch array (looked up once
+// per device); nullptr with *rc set when the runtime refuses.
+static void* kd_static_scratch_ptr(int* rc) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kKdMaxDevices) {
+    set_last_hip_error((int)e);
+    *rc = e != hipSuccess ? TS_ERR_LAUNCH : TS_ERR_RANGE;
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> hold(g_kd_scratch_lock);
+  if (!g_kd_scratch_ptr[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(kd_static_scratch));
+    if (e != hipSuccess || !p) {
+      set_last_hip_error((int)e);
+      *rc = TS_ERR_LAUNCH;
+      return nullptr;
+    }
+    g_kd_scratch_ptr[dev] = p;
+  }
+  return g_kd_scratch_ptr[dev];
+}
 
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
@@ -27,6 +62,16 @@ struct TStat {
 struct SStat {
   float m, z, z1;
 };
+
+// acc + w * (t - s) for the sum p (t - s) of the KD term.  A teacher logit of
+// -inf (a masked vocabulary entry) has weight w = 2^(-inf) = 0 and must
+// contribute nothing, as F.kl_div's xlogy gives, where 0 * (-inf) would be
+// NaN: the difference is kept finite from below (fmaxf also turns the NaN of
+// -inf - -inf into the bound).  +inf (student -inf under a positive teacher
+// weight) stays: the reference's loss is +inf there too.
+__device__ __forceinline__ float acc_weighted_diff(float w, float t, float s, float acc) {
+  return fmaf(w, fmaxf(t - s, -3.4028234e38f), acc);
+}
 
 __device__ __forceinline__ TStat tstat_init() { return TStat{kNegBig, 0.f, 0.f}; }
 __device__ __forceinline__ SStat sstat_init() { return SStat{kNegBig, 0.f, 0.f}; }
@@ -71,13 +116,17 @@ __device__ __forceinline__ void fold(TStat& st, SStat& ss, const float (&t)[N], 
     mt = fmaxf(mt, t[i]);
     ms = fmaxf(ms, s[i]);
   }
+  // a block of nothing but -inf (masked vocabulary entries) keeps a finite
+  // reference point, so that its terms are 2^(-inf) = 0 and not 2^(inf - inf)
+  mt = fmaxf(mt, kNegBig);
+  ms = fmaxf(ms, kNegBig);
   const float mtk = mt * k, msk = ms * k, ms1 = ms * kLog2e;
   float zt = 0.f, at = 0.f, zs = 0.f, z1 = 0.f;
 #pragma unroll
   for (int i = 0; i < N; ++i) {
     const float et = fast_exp2(fmaf(t[i], k, -mtk));
     zt += et;
-    at = fmaf(et, t[i] - s[i], at);
+    at = acc_weighted_diff(et, t[i], s[i], at);
     zs += fast_exp2(fmaf(s[i], k, -msk));
     if (CE) z1 += fast_exp2(fmaf(s[i], kLog2e, -ms1));
   }
@@ -392,7 +441,7 @@ __global__ __launch_bounds__(BLOCK, (KREG * GROUP > 1024 ? 4 : 1)) void kd_rows_
       const float et = fast_exp2(fmaf(tv, a.k, -mtk));
       zt += et;
       zs += fast_exp2(fmaf(sv, a.k, -msk));
-      at = fmaf(et, tv - sv, at);
+      at = acc_weighted_diff(et, tv, sv, at);
       if (CE) z1 += fast_exp2(fmaf(sv, kLog2e, -ms1));
     };
     add(eh_t, eh_s);  // a missing end element contributes 2^(-huge) = 0
@@ -679,7 +728,7 @@ __global__ __launch_bounds__(kPartBlock) void kd_wide_pass1_kernel(const KdArgs 
       for (int i = 0; i < VEC; ++i) {
         const float et = fast_exp2(fmaf(ft[j][i], a.k, -wmtk));
         zt += et;
-        at = fmaf(et, ft[j][i] - fs[j][i], at);
+        at = acc_weighted_diff(et, ft[j][i], fs[j][i], at);
         zs += fast_exp2(fmaf(fs[j][i], a.k, -wmsk));
         if (CE) z1 += fast_exp2(fmaf(fs[j][i], kLog2e, -wms1));
       }
@@ -1102,6 +1151,22 @@ int ts_kd_fwd_bwd(const void* s, const void* t, const uint8_t* row_mask, int64_t
                   int64_t ld_g, int dtype, ts_stream_t stream) {
   return ts_kdce_fwd_bwd(s, t, row_mask, nullptr, 0, n_rows, V, ld_s, ld_t, inv_T, loss_scale, 0.f, workspace,
                          loss_out, grad, ld_g, dtype, stream);
+}
+
+size_t ts_kd_static_scratch_bytes(void) { return ts::kKdStaticScratchBytes; }
+
+int ts_kd_fwd_bwd_static(const void* s, const void* t, const uint8_t* row_mask, int64_t n_rows, int64_t V,
+                         int64_t ld_s, int64_t ld_t, float inv_T, float loss_scale, float* loss_out, void* grad,
+                         int64_t ld_g, int dtype, ts_stream_t stream) {
+  if (n_rows < 0 || V <= 0) return TS_ERR_ARG;
+  if (dtype != TS_F32 && dtype != TS_BF16 && dtype != TS_F16) return TS_ERR_ARG;
+  // the same kernels on the library's own array instead of a caller's workspace
+  if (ts_kd_workspace_bytes(n_rows, V, dtype) > ts::kKdStaticScratchBytes) return TS_ERR_RANGE;
+  int rc = TS_OK;
+  void* ws = ts::kd_static_scratch_ptr(&rc);
+  if (!ws) return rc;
+  return ts_kdce_fwd_bwd(s, t, row_mask, nullptr, 0, n_rows, V, ld_s, ld_t, inv_T, loss_scale, 0.f, ws, loss_out,
+                         grad, ld_g, dtype, stream);
 }
 
 }  // extern "C"
