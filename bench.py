@@ -32,7 +32,6 @@ import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
-sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 TIMED_EVERY = 4  # one EMA launch in four carries kernel timing events
 HBM_PEAK_GBS = 8000.0       # MI355X published HBM3E bandwidth
@@ -44,7 +43,7 @@ EMA_VITB_TRAFFIC_BYTES = 1035.3e6
 
 
 def _shapes():
-    from shapes import numel, resnet18_shapes, vit_base_shapes
+    from tspipe_amd.shapes import numel, resnet18_shapes, vit_base_shapes
     return numel, resnet18_shapes(), vit_base_shapes()
 
 

@@ -242,3 +242,39 @@ def test_fused_training_forward_equals_the_two_calls(device):
     assert lib.ts_bn_forward_train(x.data_ptr(), yb.data_ptr(), None, None, N, C, H * W, None, None, None, None,
                                    ws4.data_ptr(), 2, 1e-5, st) == -1
 
+
+
+def test_a_refused_call_leaves_the_next_forward_correct(device, monkeypatch):
+    from tspipe_amd import _lib
+    bn = ta.DeferredBatchNorm(6, chunks=8).to(device)
+    xs = [_make((4, 6, 5, 5), 70 + i) for i in range(3)]
+    bn(xs[0].to(device))
+    real = _lib.lib()
+
+    class Refusing:
+        def __getattr__(self, name):
+            return getattr(real, name)
+
+        def ts_bn_forward_train(self, *args):
+            return -4  # TS_ERR_ALIGN, nothing enqueued
+
+    parity = bn._parity
+    monkeypatch.setattr(_lib, "lib", lambda: Refusing())
+    with pytest.raises(_lib.TSPipeAmdError):
+        bn(xs[1].to(device))
+    monkeypatch.undo()
+    assert bn._parity in (0, parity)  # not advanced by the refused call
+    _check_workspace(bn)
+    y = bn(xs[2].to(device))
+    want = F.batch_norm(xs[2].double(), None, None, bn.weight.detach().cpu().double(), bn.bias.detach().cpu().double(),
+                        True, 0.0, 1e-5)
+    assert (y.cpu().double() - want).abs().max() < 2e-5
+    _check_workspace(bn)
+    # a cast of the module takes the workspace along; it comes back as fp32 zeros
+    bn.half()
+    bn.float()
+    assert bn._workspace(xs[0].to(device)).dtype == torch.float32
+    y = bn(xs[0].to(device))
+    want = F.batch_norm(xs[0].double(), None, None, bn.weight.detach().cpu().double(), bn.bias.detach().cpu().double(),
+                        True, 0.0, 1e-5)
+    assert (y.cpu().double() - want).abs().max() < 2e-5

@@ -5,7 +5,7 @@ import torch
 import tspipe_amd as ta
 from helpers import bits_equal, param_lists, seeded
 from oracle import ts_oracle
-from shapes import resnet18_shapes, vit_base_shapes
+from tspipe_amd.shapes import resnet18_shapes, vit_base_shapes
 
 pytestmark = pytest.mark.gpu
 
@@ -290,3 +290,39 @@ def test_ema_and_gather_from_two_threads(device):
         th.join(timeout=100)
     assert not errors, errors
     assert results == {0: (True, True), 1: (True, True)}
+
+
+def test_arena_reuse_waits_for_announced_readers_and_can_be_switched_off(device):
+    from tspipe_amd import ema as ema_mod
+    ema_mod.release_pool()
+    teacher, student = param_lists([(256, 1024), (1024,), (512, 512)], 17)
+    t_dev = [t.to(device) for t in teacher]
+    s_dev = [s.to(device) for s in student]
+    side = torch.cuda.Stream(device)
+    version = ta.momentum_update(0.9, s_dev, t_dev)
+    ptr = version[0].data_ptr()
+    # a reader on another stream, announced to the pool, then the version is dropped without a host sync
+    side.wait_stream(torch.cuda.current_stream(device))
+    with torch.cuda.stream(side):
+        torch.cuda._sleep(2_000_000)
+        copies = [v.clone() for v in version]
+    ema_mod.note_reader(version, side)
+    del version
+    again = ta.momentum_update(0.5, s_dev, t_dev)  # may take the same arena; must not overtake the reader
+    assert again[0].data_ptr() == ptr
+    torch.cuda.synchronize()
+    assert all(bits_equal(c, w) for c, w in zip(copies, ts_oracle.ema_update(0.9, student, teacher)))
+    assert all(bits_equal(a, w) for a, w in zip(again, ts_oracle.ema_update(0.5, student, teacher)))
+    # recycling off: every call returns memory no earlier result used while that result is alive or not
+    ema_mod.set_recycling(False)
+    try:
+        del again, copies
+        a = ta.momentum_update(0.9, s_dev, t_dev)
+        pa = a[0].data_ptr()
+        keep = a  # noqa: F841  (held: torch's allocator cannot hand the block out either)
+        b = ta.momentum_update(0.9, s_dev, t_dev)
+        assert b[0].data_ptr() != pa
+        assert all(bits_equal(x, w) for x, w in zip(b, ts_oracle.ema_update(0.9, student, teacher)))
+    finally:
+        ema_mod.set_recycling(True)
+        ema_mod.release_pool()

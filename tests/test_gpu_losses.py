@@ -115,6 +115,28 @@ def test_kd_identities(device):
     assert l1.item() >= 0
 
 
+@pytest.mark.parametrize("rows,V,dtype", [(6, 100, torch.float32), (4, 1000, torch.float32), (3, 30522, torch.bfloat16),
+                                          (2, 70001, torch.float32)])
+def test_kd_teacher_minus_inf_entries_contribute_nothing(device, rows, V, dtype):
+    # a masked vocabulary: the teacher puts -inf on some entries, the student's are finite.
+    # F.kl_div's xlogy gives those entries a zero term; a plain 0 * (-inf) would be NaN
+    g = seeded(300 + V)
+    s = (torch.randn(rows, V, generator=g) * 3).to(dtype)
+    t = (torch.randn(rows, V, generator=g) * 3).to(dtype)
+    banned = torch.rand(rows, V, generator=g) < 0.3
+    banned[:, 0] = False  # no row is banned entirely
+    t = t.masked_fill(banned, float("-inf"))
+    want, (gw,) = _oracle_grad(lambda a, b: ts_oracle.kd_soft_target(a, b, 2.0), s, others=(t,))
+    assert want == want  # the reference's value is finite
+    sd = s.to(device).requires_grad_()
+    loss = ta.kd_soft_target_loss(sd, t.to(device), 2.0)
+    loss.backward()
+    tol = 2e-5 if dtype == torch.float32 else 1e-3
+    assert rel_err(loss.item(), want) < tol
+    assert torch.isfinite(sd.grad).all()
+    assert max_rel_to_peak(sd.grad, gw) < tol + (0 if dtype == torch.float32 else 2 ** -8)
+
+
 def test_kd_grad_output_scaling_and_no_grad(device):
     g = seeded(8)
     s = (torch.randn(8, 33, generator=g)).to(device)
@@ -464,10 +486,18 @@ def test_distil_loss_fn_clm_and_mse_terms(device, mode):
     peak = gs.abs().max().item()
     # the MSE term is added to a gradient already stored in bf16: two roundings
     assert ((sd.grad.cpu().double() - gs).abs() <= 1e-3 * peak + gs.abs() * 2.0 ** -7).all()
-    with pytest.raises(NotImplementedError):
-        params.alpha_mlm, params.alpha_clm = 1.0, 1.0
-        ta.distil_loss_fn({"logits": sd, "hidden_states": None}, {"logits": t.to(device), "hidden_states": None},
-                          (lm.to(device), att.to(device)), None, params, 0)
+    # both hard-label terms at once, as the reference's loss_fn adds them (distiller.py:742-749)
+    params.alpha_mlm, params.alpha_clm = 0.7, 1.5
+    want, (gs,) = _oracle_grad(
+        lambda a, b: ts_oracle.distil_loss(a, b, None, None, lm, att, 0.5, 0.7, 0.0, 2.0, False, alpha_clm=1.5,
+                                           alpha_mse=a_mse), s, others=(t,))
+    sd = s.to(device).requires_grad_()
+    loss = ta.distil_loss_fn({"logits": sd, "hidden_states": None}, {"logits": t.to(device), "hidden_states": None},
+                             (lm.to(device), att.to(device)), None, params, 0)
+    loss.backward()
+    assert rel_err(loss.item(), want) < 1e-3
+    peak = gs.abs().max().item()
+    assert ((sd.grad.cpu().double() - gs).abs() <= 1e-3 * peak + gs.abs() * 2.0 ** -6).all()
 
 
 @pytest.mark.parametrize("rows,V,dtype", [(256, 100, torch.float32), (33, 5000, torch.float32),

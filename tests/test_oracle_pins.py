@@ -15,7 +15,7 @@ import torch.nn.functional as F
 
 from helpers import seeded
 from oracle import ts_oracle
-from shapes import numel, resnet18_shapes, vit_base_shapes
+from tspipe_amd.shapes import numel, resnet18_shapes, vit_base_shapes
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 

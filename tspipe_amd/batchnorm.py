@@ -84,13 +84,12 @@ class _NormalizeFn(torch.autograd.Function):
         layer = ctx.layer
         ws = layer._workspace(x)
         parity = layer._parity  # shared with the training forward: the calls of a layer alternate
-        layer._parity = 1 - parity
         with torch.cuda.device(x.device):
             status = _lib.lib().ts_bn_backward(x.data_ptr(), dy.data_ptr(), mean.data_ptr(), invstd.data_ptr(),
                                                _ptr(weight), dx.data_ptr(), dgamma.data_ptr(), dbeta.data_ptr(),
                                                ws.data_ptr() + 8 * c, parity, n, c, hw, 1 if ctx.training else 0,
                                                _lib.current_stream_ptr(x.device))
-        _lib.check(status, "ts_bn_backward")
+        layer._after_launch(status, parity, "ts_bn_backward")
         return (dx, dgamma if weight is not None else None, dbeta if ctx.has_bias else None,
                 None, None, None, None, None)
 
@@ -108,13 +107,12 @@ class _TrainForwardFn(torch.autograd.Function):
         invstd = torch.empty(c, dtype=torch.float32, device=x.device)
         ws = layer._workspace(x)
         parity = layer._parity
-        layer._parity = 1 - parity
         with torch.cuda.device(x.device):
             status = _lib.lib().ts_bn_forward_train(
                 x.data_ptr(), y.data_ptr(), _ptr(weight), _ptr(bias), n, c, hw, layer.sum.data_ptr(),
                 layer.sum_squares.data_ptr(), mean.data_ptr(), invstd.data_ptr(), ws.data_ptr() + 8 * c, parity,
                 float(layer.eps), _lib.current_stream_ptr(x.device))
-        _lib.check(status, "ts_bn_forward_train")
+        layer._after_launch(status, parity, "ts_bn_forward_train")
         ctx.save_for_backward(x, weight, mean, invstd)
         ctx.layer = layer
         ctx.training = True
@@ -145,6 +143,7 @@ class DeferredBatchNorm(_BatchNorm):
         # alternate between (``_parity`` says which one the next call reduces into)
         self.register_buffer("_ws", torch.zeros(6 * num_features), persistent=False)
         self._parity = 0
+        self._ws_stream = None  # the stream whose kernels last used the workspace
         self.counter = 0
         self.tracked = 0
         self.chunks = chunks
@@ -154,10 +153,30 @@ class DeferredBatchNorm(_BatchNorm):
             raise ValueError("expected at least 3D input (got %dD input)" % input.dim())
 
     def _workspace(self, x: Tensor) -> Tensor:
-        if self._ws.device != x.device or self._ws.numel() != 6 * self.num_features:
+        """The layer's reduction workspace, on x's device.  Its alternating
+        halves assume that the layer's calls run one after the other on the
+        device, so a call on a stream other than the previous call's first
+        waits for that stream."""
+        if self._ws.device != x.device or self._ws.numel() != 6 * self.num_features or self._ws.dtype != torch.float32:
+            # moved, resized, or cast along with the module (module.half()): start from zeros
             self._ws = torch.zeros(6 * self.num_features, dtype=torch.float32, device=x.device)
             self._parity = 0
+            self._ws_stream = None
+        stream = torch.cuda.current_stream(x.device)
+        if self._ws_stream is not None and self._ws_stream != stream:
+            stream.wait_stream(self._ws_stream)
+        self._ws_stream = stream
         return self._ws
+
+    def _after_launch(self, status: int, parity: int, what: str) -> None:
+        """The half the next call reduces into alternates only once this call
+        is known to have been enqueued.  A refused call may have run part of
+        its launches, so the workspace starts again from zeros."""
+        if status < 0:
+            self._ws = torch.zeros(6 * self.num_features, dtype=torch.float32, device=self._ws.device)
+            self._parity = 0
+            _lib.check(status, what)
+        self._parity = 1 - parity
 
     def _stats(self, x: Tensor, accumulate: bool):
         """One pass over x: micro-batch mean / invstd, optionally ``sum += ...``."""

@@ -12,9 +12,11 @@
 //     uses the fixed reference point x_max = log2(e)/tau instead of a running
 //     maximum: no rescaling of the accumulators, and partial results of
 //     different key ranges just add up;
-//   * the normalisation is applied as fp32 factors after the bf16 contraction
-//     (logit_ij = <q_i,k_j> * rq_i * rk_j / tau), so the raw bf16 inputs feed
-//     the MFMA and no rounded copy of qh / kh is ever made.
+//   * the keys are normalised in fp32 and rounded to bf16 once, by the prep
+//     kernel (the tile images below hold kh); the queries feed the MFMA as
+//     they are (bf16 inputs in place, fp32 / fp16 inputs through a bf16 copy)
+//     and their 1/|q| is applied as an fp32 factor after the contraction
+//     (logit_ij = <q_i, kh_j> * rq_i / tau).
 //
 // Kernels:
 //   prep     per row: rq = 1/max(|q|,eps), rk, the diagonal logit; the keys,

@@ -6,6 +6,7 @@
 #include <torch/csrc/autograd/python_variable.h>
 
 #include <cstdint>
+#include <vector>
 
 namespace {
 
@@ -77,13 +78,25 @@ int64_t data_ptrs(py::list tensors, uintptr_t ptr_out, int64_t capacity) {
 }
 
 // True when every tensor of the list is referenced only by the list itself and
-// by the caller's argument handling (Python refcount == expected).
+// by the caller's argument handling (Python refcount == expected), and no
+// C++ holder keeps its TensorImpl either (a view saved by autograd for a
+// backward pass, a tensor list inside another extension): such a holder
+// changes neither the Python refcount nor the storage's use count.
 bool all_refcounts_equal(py::list tensors, int64_t expected) {
   const int64_t n = py::len(tensors);
-  for (int64_t i = 0; i < n; ++i)
-    if (Py_REFCNT(PyList_GET_ITEM(tensors.ptr(), i)) != expected) return false;
+  for (int64_t i = 0; i < n; ++i) {
+    PyObject* o = PyList_GET_ITEM(tensors.ptr(), i);
+    if (Py_REFCNT(o) != expected) return false;
+    if (!THPVariable_Check(o) || THPVariable_Unpack(o).use_count() != 1) return false;
+  }
   return true;
 }
+
+// Test aid: a C++ owner of a tensor that Python cannot see.  hold() keeps the
+// tensor alive inside this module until drop() is called.
+static std::vector<at::Tensor> g_held;
+void hold(const at::Tensor& t) { g_held.push_back(t); }
+void drop() { g_held.clear(); }
 
 }  // namespace
 
@@ -91,4 +104,6 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("pair_info", &pair_info);
   m.def("data_ptrs", &data_ptrs);
   m.def("all_refcounts_equal", &all_refcounts_equal);
+  m.def("hold", &hold);
+  m.def("drop", &drop);
 }

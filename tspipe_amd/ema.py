@@ -12,6 +12,7 @@ implementations of that plug-in are
 import operator
 import sys
 import threading
+import weakref
 from typing import Iterable, List, Optional, Sequence
 
 import numpy as np
@@ -118,7 +119,7 @@ def _fast_update(m: float, online, target) -> Optional[List[torch.Tensor]]:
     if status != 0:
         return None
     teachers = target if len(target) == n else target[:n]
-    arena = _acquire_arena(teachers, (n, total, shape_hash))
+    arena, views = _acquire_arena(teachers, (n, total, shape_hash))
     if arena.numels.size != n or not np.array_equal(arena.numels, nn[:n]):
         return None  # hash collision between different lists: take the exact path
     device = teachers[0].device
@@ -133,18 +134,18 @@ def _fast_update(m: float, online, target) -> Optional[List[torch.Tensor]]:
         if timed:
             kernel_events.append((start, end))
         table.done()
-    return list(arena.views)
+    return views
 
 
 class _Arena:
     """One flat output allocation and its views, shaped like a parameter list."""
-    __slots__ = ("flat", "views", "ptrs", "numels", "stream")
+    __slots__ = ("flat", "views", "ptrs", "numels", "stream", "readers", "__weakref__")
 
     def __init__(self, teachers: Sequence[torch.Tensor]):
         device = teachers[0].device
         # like a block of torch's caching allocator, the arena belongs to the
         # stream it was made on and is only handed out again on that stream
-        self.stream = torch.cuda.current_stream(device).cuda_stream
+        self.stream = torch.cuda.current_stream(device).cuda_stream if device.type == "cuda" else None
         numels = np.array(list(map(torch.Tensor.numel, teachers)), dtype=np.int64)
         if not (numels & 3).any():
             # every size is a multiple of 4 elements: pieces sit back to back,
@@ -158,17 +159,21 @@ class _Arena:
             self.views = [p[:t.numel()].view(t.shape) for p, t in zip(pieces, teachers)]
         self.ptrs = _ptrs(self.views)
         self.numels = numels
+        self.readers = []  # events of streams that read this version (note_reader)
 
     def is_free(self) -> bool:
         """True when nothing outside this arena can reach its memory: no view
-        object is referenced elsewhere and the storage has no further alias."""
+        object is referenced elsewhere, from Python or from C++ (a tensor saved
+        for a backward pass, a list kept by another extension), and the
+        storage has no further alias."""
         storage = self.flat.untyped_storage()
         if _use_count(storage._cdata) != len(self.views) + 2:  # flat + views + the wrapper just made
             return False
         host = _lib.host_helper()
         if host is not None:
             return host.all_refcounts_equal(self.views, 1)  # only self.views holds them
-        return all(c == 2 for c in map(sys.getrefcount, self.views))
+        return all(c == 2 for c in map(sys.getrefcount, self.views)) and \
+            all(c == 1 for c in map(torch.Tensor._use_count, self.views))
 
 
 # Output arenas whose tensors the caller has dropped are handed out again
@@ -178,6 +183,42 @@ class _Arena:
 _POOL_LIMIT = 6
 _pool = {}
 _pool_lock = threading.Lock()
+_recycle = True
+_by_storage = {}  # data_ptr of an arena's flat allocation -> weak reference to the arena
+
+
+def set_recycling(enabled: bool) -> None:
+    """Switches the reuse of output arenas on (the default) or off.  With it
+    off every call allocates a fresh flat buffer and fresh views, exactly as
+    the reference's ``clone()`` does, at 100+ microseconds of host time per
+    150-tensor list."""
+    global _recycle
+    _recycle = bool(enabled)
+    if not _recycle:
+        release_pool()
+
+
+def note_reader(version: Sequence[torch.Tensor], stream: Optional["torch.cuda.Stream"] = None) -> None:
+    """Tells the pool that ``stream`` (default: the current one) has work
+    enqueued that reads ``version``, a list this module returned.  An event is
+    recorded on that stream, and the arena is only written again after it.
+
+    Needed when a version is read on a stream other than the one that made it
+    and then dropped without a host synchronisation.  The reference's own
+    reader, ``copy_model``, synchronises its copy stream before it returns
+    (tspipe/gpu_task.py:718-724) and needs no note."""
+    if not version:
+        return
+    first = version[0]
+    ref = _by_storage.get(first.untyped_storage().data_ptr())
+    arena = ref() if ref is not None else None
+    if arena is None:
+        return
+    stream = stream if stream is not None else torch.cuda.current_stream(first.device)
+    event = torch.cuda.Event()
+    event.record(stream)
+    with _pool_lock:
+        arena.readers.append(event)
 
 
 def release_pool() -> None:
@@ -186,26 +227,39 @@ def release_pool() -> None:
     cached chunk tables."""
     with _pool_lock:
         _pool.clear()
+        _by_storage.clear()
     _tables.clear_table_cache()
 
 
-def _acquire_arena(teachers: Sequence[torch.Tensor], shapes) -> _Arena:
-    """shapes: anything hashable that identifies the list's shapes (the tuple of
+def _acquire_arena(teachers: Sequence[torch.Tensor], shapes):
+    """Returns (arena, views): an arena nobody else can reach and a fresh list
+    of its view tensors.  The list is made while the pool lock is held, so a
+    second thread asking for the same key sees the arena as taken.
+
+    shapes: anything hashable that identifies the list's shapes (the tuple of
     shapes, or the helper's (count, total, 64-bit shape hash) triple)."""
-    if _use_count is None:
-        return _Arena(teachers)
+    if _use_count is None or not _recycle:
+        arena = _Arena(teachers)
+        return arena, list(arena.views)
     device = teachers[0].device
-    key = (device, torch.cuda.current_stream(device).cuda_stream, shapes)
+    stream = torch.cuda.current_stream(device)
+    key = (device, stream.cuda_stream, shapes)
     with _pool_lock:
         arenas = _pool.setdefault(key, [])
         for arena in arenas:
             if arena.is_free():
-                return arena
+                # streams that were announced as readers of the old contents
+                for event in arena.readers:
+                    stream.wait_event(event)
+                arena.readers = []
+                return arena, list(arena.views)
         arena = _Arena(teachers)
         arenas.append(arena)
+        _by_storage[arena.flat.untyped_storage().data_ptr()] = weakref.ref(arena)
         if len(arenas) > _POOL_LIMIT:
-            arenas.pop(0)  # stays alive for as long as its user holds it
-        return arena
+            old = arenas.pop(0)  # stays alive for as long as its user holds it
+            _by_storage.pop(old.flat.untyped_storage().data_ptr(), None)
+        return arena, list(arena.views)
 
 
 @torch.no_grad()
@@ -222,9 +276,9 @@ def momentum_update(m: float, online_new_param: Iterable[Optional[torch.Tensor]]
     students, teachers, shapes = _prepare(online_new_param, target_param, skip_none)
     if not teachers:
         return []
-    arena = _acquire_arena(teachers, shapes)
+    arena, views = _acquire_arena(teachers, shapes)
     _launch(m, students, teachers, arena.ptrs, arena.numels)
-    return list(arena.views)
+    return views
 
 
 def calculate_target_network_parameters(m, online_new_param, target_param=None):
@@ -263,9 +317,8 @@ def clone_and_update(m: float, online_param: Iterable[torch.Tensor], target_para
     students, teachers, shapes = _prepare(online_param, target_param, skip_none=False)
     if not teachers:
         return [], []
-    ema_arena = _acquire_arena(teachers, shapes)
-    views = list(ema_arena.views)  # held, so the second acquire cannot hand the same arena out
-    clone_arena = _acquire_arena(teachers, shapes)
+    ema_arena, views = _acquire_arena(teachers, shapes)  # views held: the second acquire cannot hand the same arena out
+    clone_arena, clone_views = _acquire_arena(teachers, shapes)
     offset = clone_arena.flat.data_ptr() - ema_arena.flat.data_ptr()
     device = teachers[0].device
     with torch.cuda.device(device):
@@ -279,7 +332,7 @@ def clone_and_update(m: float, online_param: Iterable[torch.Tensor], target_para
         if timed:
             kernel_events.append((start, end))
         table.done()
-    return list(clone_arena.views), views
+    return clone_views, views
 
 
 # ---------------------------------------------------------------------------

@@ -526,34 +526,46 @@ def soft_target_tspipe_loss(model_out: Tensor, ema_model_out: Tensor, label: Ten
     raise AssertionError(f"kd_mode {mode!r}: the reference knows 'st' and 'logits'")
 
 
+def _ce_terms(lm_labels: Tensor, params):
+    """The hard-label terms of DistilBERT's loss as (labels, weight) pairs:
+    masked-LM cross entropy against ``lm_labels`` (distiller.py:742-744) and
+    causal-LM cross entropy, where the logits at position p are scored against
+    the label at p+1 and the last position of a sequence has no target
+    (distiller.py:745-749)."""
+    terms = []
+    alpha_mlm = float(getattr(params, "alpha_mlm", 0.0))
+    alpha_clm = float(getattr(params, "alpha_clm", 0.0))
+    if alpha_mlm > 0.0:
+        terms.append((lm_labels, alpha_mlm))
+    if alpha_clm > 0.0:
+        shifted = torch.full_like(lm_labels, -100)
+        shifted[..., :-1] = lm_labels[..., 1:]
+        terms.append((shifted, alpha_clm))
+    return terms
+
+
 def distil_loss_fn(student_outputs, teacher_outputs, labels, tspipe_args, params, epoch: int) -> Tensor:
     """``TSPipeDistiller.loss_fn`` of benchmarks/distilbert/distiller.py:711-772:
-    ``alpha_ce`` x masked KD, ``alpha_mlm`` x masked-LM cross entropy or
-    ``alpha_clm`` x causal-LM cross entropy (ignore_index -100) -- both in one
-    pass over the logits -- ``alpha_mse`` x squared error of the selected
+    ``alpha_ce`` x masked KD, ``alpha_mlm`` x masked-LM cross entropy and/or
+    ``alpha_clm`` x causal-LM cross entropy (ignore_index -100) -- the first of
+    the two in the same pass over the logits as the KD term, a second one in a
+    pass of its own -- ``alpha_mse`` x squared error of the selected
     logits, and ``alpha_cos`` x cosine embedding loss on the last hidden states.  ``params`` carries
     ``alpha_ce, alpha_mlm, alpha_clm, alpha_mse, alpha_cos, temperature,
     restrict_ce_to_mask`` like the reference's LossComputeParam."""
     s_logits, t_logits = student_outputs["logits"], teacher_outputs["logits"]
     lm_labels, attention_mask = labels
-    alpha_mlm = float(getattr(params, "alpha_mlm", 0.0))
-    alpha_clm = float(getattr(params, "alpha_clm", 0.0))
     alpha_mse = float(getattr(params, "alpha_mse", 0.0))
-    if alpha_mlm > 0.0 and alpha_clm > 0.0:
-        # the reference's own sanity check forbids it (benchmarks/distilbert/train.py:50)
-        raise NotImplementedError("alpha_mlm and alpha_clm are mutually exclusive")
     mask = (lm_labels > -1) if params.restrict_ce_to_mask else attention_mask
-    ce_labels, ce_weight = None, 0.0
-    if alpha_mlm > 0.0:
-        ce_labels, ce_weight = lm_labels, alpha_mlm
-    elif alpha_clm > 0.0:
-        # logits at position p are scored against the label at p+1; the last
-        # position of every sequence has no target (distiller.py:745-749)
-        ce_labels = torch.full_like(lm_labels, -100)
-        ce_labels[..., :-1] = lm_labels[..., 1:]
-        ce_weight = alpha_clm
+    terms = _ce_terms(lm_labels, params)
+    ce_labels, ce_weight = terms[0] if terms else (None, 0.0)
     loss = kd_ce_loss(s_logits, t_logits, ce_labels, params.temperature, kd_weight=params.alpha_ce,
                       ce_weight=ce_weight, row_mask=mask, ignore_index=-100, mse_weight=alpha_mse)
+    for ce_labels, ce_weight in terms[1:]:
+        # both alpha_mlm and alpha_clm set (distiller.py:742-749 adds both terms): the
+        # second cross entropy is a pass of its own over the student logits
+        loss = loss + kd_ce_loss(s_logits, t_logits, ce_labels, params.temperature, kd_weight=0.0,
+                                 ce_weight=ce_weight, row_mask=mask, ignore_index=-100)
     if getattr(params, "alpha_cos", 0.0) > 0.0:
         s_hid = student_outputs["hidden_states"][-1]
         t_hid = teacher_outputs["hidden_states"][-1]
@@ -571,23 +583,17 @@ def distil_loss_fn_pieces(student_pieces, teacher_pieces, labels, tspipe_args, p
     The ``alpha_mse`` term has no piece-wise kernel: use ``distil_loss_fn``."""
     from .batch_ops import Batch, gather
     lm_labels, attention_mask = labels
-    alpha_mlm = float(getattr(params, "alpha_mlm", 0.0))
-    alpha_clm = float(getattr(params, "alpha_clm", 0.0))
     if float(getattr(params, "alpha_mse", 0.0)) > 0.0:
         raise NotImplementedError("alpha_mse needs the gathered logits: call distil_loss_fn")
-    if alpha_mlm > 0.0 and alpha_clm > 0.0:
-        raise NotImplementedError("alpha_mlm and alpha_clm are mutually exclusive")
     mask = (lm_labels > -1) if params.restrict_ce_to_mask else attention_mask
-    ce_labels, ce_weight = None, 0.0
-    if alpha_mlm > 0.0:
-        ce_labels, ce_weight = lm_labels, alpha_mlm
-    elif alpha_clm > 0.0:
-        ce_labels = torch.full_like(lm_labels, -100)
-        ce_labels[..., :-1] = lm_labels[..., 1:]
-        ce_weight = alpha_clm
-    loss = kd_ce_loss_pieces([p["logits"] for p in student_pieces], [p["logits"] for p in teacher_pieces], ce_labels,
-                             params.temperature, kd_weight=params.alpha_ce, ce_weight=ce_weight, row_mask=mask,
-                             ignore_index=-100)
+    terms = _ce_terms(lm_labels, params)
+    ce_labels, ce_weight = terms[0] if terms else (None, 0.0)
+    s_list, t_list = [p["logits"] for p in student_pieces], [p["logits"] for p in teacher_pieces]
+    loss = kd_ce_loss_pieces(s_list, t_list, ce_labels, params.temperature, kd_weight=params.alpha_ce,
+                             ce_weight=ce_weight, row_mask=mask, ignore_index=-100)
+    for ce_labels, ce_weight in terms[1:]:
+        loss = loss + kd_ce_loss_pieces(s_list, t_list, ce_labels, params.temperature, kd_weight=0.0,
+                                        ce_weight=ce_weight, row_mask=mask, ignore_index=-100)
     if getattr(params, "alpha_cos", 0.0) > 0.0:
         s_hid = gather([Batch(p["hidden_states"][-1]) for p in student_pieces])
         t_hid = gather([Batch(p["hidden_states"][-1]) for p in teacher_pieces])

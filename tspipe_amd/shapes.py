@@ -1,4 +1,5 @@
-"""Parameter-shape lists of the two EMA workloads (synthetic, no model code)."""
+"""Parameter-shape lists of the two EMA benchmark workloads (synthetic, no model
+code): what bench.py and the parity tests build their parameter lists from."""
 
 
 def resnet18_shapes():
