@@ -34,12 +34,24 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 TIMED_EVERY = 4  # one EMA launch in four carries kernel timing events
+SETUP_STEPS = 12  # untimed calls before the warm-up steps (resource creation, see run_step_benchmark)
 HBM_PEAK_GBS = 8000.0       # MI355X published HBM3E bandwidth
 MFMA_BF16_PEAK_TFLOPS = 2500.0
-# HBM bytes one ViT-B EMA launch moves, from two rocprofv3 --pmc runs (FETCH_SIZE,
-# WRITE_SIZE) scaled by the same counters on the copy kernel of known size;
-# summary in profiles/hbm_traffic_pmc_all_kernels.md.  Not measured by this script.
-EMA_VITB_TRAFFIC_BYTES = 1035.3e6
+TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "hbm_traffic_pmc_all_kernels.md")
+
+
+def _ema_traffic_bytes():
+    """HBM bytes one ViT-B EMA launch moves, read from the committed rocprofv3
+    --pmc summary (FETCH_SIZE and WRITE_SIZE runs scaled by the same counters
+    on a copy of known size); None when the summary is not in the tree.  The
+    value is a record of those profiler runs, not a product of this run."""
+    try:
+        for line in open(TRAFFIC_SUMMARY):
+            if line.startswith("bench.py roofline.traffic"):
+                return float(line.split("=")[1].split()[0])
+    except OSError:
+        pass
+    return None
 
 
 def _shapes():
@@ -120,24 +132,48 @@ def run_step_benchmark(steps, warmup, dev):
             span[1].record()
         state["loss_enqueued"] = time.perf_counter()
 
-    def run_steps(n, events):
-        failures = []
+    # The two host threads live for the whole benchmark, like TSPipe's worker
+    # threads: what they keep per thread (pinned staging buffers, autograd's
+    # hand-off state) is created once, in the set-up phase.  A phase starts
+    # when main and both workers meet at `gate` and ends at `done`.
+    gate, done = threading.Barrier(3), threading.Barrier(3)
+    phase = {"n": 0, "events": None, "stop": False}
+    failures = []
 
-        def guarded(fn):
-            def body():
-                try:
-                    fn(n, events)
-                except BaseException as exc:  # re-raised on the main thread below
-                    failures.append(exc)
-            return body
-        workers = [threading.Thread(target=guarded(f)) for f in (ema_worker, loss_worker)]
-        for w in workers:
-            w.start()
-        for w in workers:
-            w.join()
+    def worker_loop(fn):
+        while True:
+            gate.wait()
+            if phase["stop"]:
+                return
+            try:
+                fn(phase["n"], phase["events"])
+            except BaseException as exc:  # re-raised on the main thread below
+                failures.append(exc)
+            done.wait()
+
+    workers = [threading.Thread(target=worker_loop, args=(f,), daemon=True) for f in (ema_worker, loss_worker)]
+    for w in workers:
+        w.start()
+
+    def run_steps(n, events):
+        """Runs n steps on the two worker threads; returns the start time and
+        the wall time from the moment both are released to the end of a
+        device-wide synchronize."""
+        phase["n"], phase["events"] = n, events
+        torch.cuda.synchronize()
+        gate.wait()
+        t0 = time.perf_counter()
+        done.wait()
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
         if failures:
             raise failures[0]
+        return t0, elapsed
 
+    # Set-up, not steps: the first calls create the output arenas, the chunk
+    # tables, autograd's device thread and the allocator's blocks on the two
+    # streams.  The W warm-up steps the caller asked for follow.
+    run_steps(SETUP_STEPS, None)
     run_steps(warmup, None)
     torch.cuda.synchronize()
     # Every TIMED_EVERY-th EMA launch of the timed region stamps its own begin
@@ -149,11 +185,12 @@ def run_step_benchmark(steps, warmup, dev):
     events = []
     gc.collect()
     gc.disable()  # as timeit does: no collector pause inside the timed region
-    t0 = time.perf_counter()
-    run_steps(steps, events)
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
+    t0, elapsed = run_steps(steps, events)
     gc.enable()
+    phase["stop"] = True
+    gate.wait()
+    for w in workers:
+        w.join()
     host_ms = {"ema_thread_enqueue_ms_per_step": round((state["ema_enqueued"] - t0) / steps * 1e3, 4),
                "loss_thread_enqueue_ms_per_step": round((state["loss_enqueued"] - t0) / steps * 1e3, 4),
                # first to last command of each stream, by HIP events on that stream
@@ -180,7 +217,10 @@ def run_step_benchmark(steps, warmup, dev):
         "elapsed": elapsed, "n_params": n_params, "loss": float(state["loss"].item()), "host": host_ms,
         "roofline": {"bound": "hbm", "kernel": "ema_multi_kernel", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": EMA_VITB_TRAFFIC_BYTES, "algorithmic_bytes_per_launch": algo_bytes,
+                     "traffic": _ema_traffic_bytes(),
+                     "traffic_source": "profiles/hbm_traffic_pmc_all_kernels.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
+                                       "runs of this script, scaled by a copy of known size); not measured by this run",
+                     "algorithmic_bytes_per_launch": algo_bytes,
                      "avg_kernel_ms": round(avg_ema_ms, 4), "launches_timed": len(ema_ms),
                      "note": "inside the timed region the kernel shares the GPU with the InfoNCE stream; 'alone' is "
                              "the same launch with the other stream idle",
@@ -207,11 +247,31 @@ def _time_stream(fn, iters, warmup=5):
     return a.elapsed_time(b) / iters
 
 
-def run_kernel_table(dev):
+def _cpu_ms(fn, budget_s=1.2, max_iters=20):
+    """Median milliseconds of fn() on the host cores: one untimed call, then
+    calls until the budget is spent (at least one).  Returns (ms, calls)."""
+    t0 = time.perf_counter()
+    fn()
+    first = time.perf_counter() - t0
+    if first > budget_s:
+        return first * 1e3, 1
+    times = []
+    t_end = time.perf_counter() + budget_s
+    while len(times) < max_iters and (not times or time.perf_counter() < t_end):
+        t0 = time.perf_counter()
+        fn()
+        times.append(time.perf_counter() - t0)
+    return statistics.median(times) * 1e3, len(times)
+
+
+def run_kernel_table(dev, with_cpu=True):
     """Stand-alone device timings of each kernel at the other configurations,
-    called through the C ABI with preallocated outputs and workspaces."""
+    called through the C ABI with preallocated outputs and workspaces; beside
+    each, `cpu_ms`: the oracle's eager PyTorch chain for the same operation on
+    the same shape, on the host cores (bounded sample, see _cpu_ms)."""
     import torch
     import tspipe_amd as ta
+    from oracle import ts_oracle
     from tspipe_amd import _lib, _tables
     from tspipe_amd import ema as ema_mod
     numel, r18, vit = _shapes()
@@ -219,6 +279,31 @@ def run_kernel_table(dev):
     out = {}
     g = torch.Generator().manual_seed(0)
     stream = _lib.current_stream_ptr(dev)
+    if with_cpu:
+        cores = os.cpu_count() or 1
+        torch.set_num_threads(min(cores, int(os.environ.get("OMP_NUM_THREADS", cores))))
+
+    def cpu(name, fn):
+        """Adds the host-side timing of the same operation to out[name]."""
+        if not with_cpu:
+            return
+        ms, calls = _cpu_ms(fn)
+        out[name]["cpu_ms"] = round(ms, 3)
+        out[name]["cpu_calls"] = calls
+        out[name]["gpu_over_cpu"] = round(ms / out[name]["ms"], 1)
+
+    def kd_cpu(s, t, T, mask=None):
+        s_c = s.detach().cpu().requires_grad_()
+        t_c = t.detach().cpu()
+        m_c = None if mask is None else mask.cpu()
+
+        def f():
+            s_c.grad = None
+            if m_c is None:
+                ts_oracle.kd_soft_target(s_c, t_c, T).backward()
+            else:
+                ts_oracle.distil_ce(s_c, t_c, m_c, T).backward()
+        return f
 
     def entry(nbytes, ms, note=None, launches=None):
         gbs = nbytes / (ms * 1e-3) / 1e9
@@ -250,7 +335,9 @@ def run_kernel_table(dev):
         nbytes = 12 * sum(numel(s) for s in shapes)
         note = "working set below the 256 MB Infinity Cache: not an HBM figure" if name == "ema_resnet18" else None
         out[name] = entry(nbytes, statistics.median(ms), note, 1)
-        del teacher, student, st
+        t_c, s_c = [t.cpu() for t in teacher], [s_.cpu() for s_ in student]
+        cpu(name, lambda: ts_oracle.ema_update(m, s_c, t_c))
+        del teacher, student, st, t_c, s_c
     ema_mod.release_pool()
 
     # student clone fused into the EMA launch (16 B per parameter: read s, t; write s', t')
@@ -271,7 +358,9 @@ def run_kernel_table(dev):
     ema_mod.kernel_events = None
     out["ema_clone_fused_vit_base"] = entry(16 * sum(numel(s) for s in vit), statistics.median(ms),
                                             "kernel-only events", 1)
-    del teacher, student, keep
+    t_c, s_c = [t.cpu() for t in teacher], [s_.cpu() for s_ in student]
+    cpu("ema_clone_fused_vit_base", lambda: ([p_.detach().clone() for p_ in s_c], ts_oracle.ema_update(0.99, s_c, t_c)))
+    del teacher, student, keep, t_c, s_c
     ema_mod.release_pool()
 
     def kd_call(s, t, mask, T, grad):
@@ -294,6 +383,7 @@ def run_kernel_table(dev):
         f = kd_call(s, t, None, 4.0, torch.empty_like(s))
         out[name] = entry(3 * rows * 100 * 4, _time_stream(f, 50),
                           "latency-bound: 2 launches of a few us each" if rows == 256 else None, 2)
+        cpu(name, kd_cpu(s, t, 4.0))
 
     # an ImageNet-sized class count (not one of the benchmark configurations): rows long enough to stream
     s = (torch.randn(32768, 1000, generator=g) * 3).to(dev)
@@ -301,6 +391,7 @@ def run_kernel_table(dev):
     f = kd_call(s, t, None, 4.0, torch.empty_like(s))
     out["kd_32768x1000_f32"] = entry(3 * 32768 * 1000 * 4, _time_stream(f, 30),
                                      "not one of the benchmark configurations", 2)
+    cpu("kd_32768x1000_f32", kd_cpu(s, t, 4.0))
     del s, t, f
 
     # DistilBERT-shaped masked KD (cfg3) after a gather of 4 micro-batches
@@ -319,6 +410,9 @@ def run_kernel_table(dev):
     ms = _event_ms(_tables.kernel_events)
     _tables.kernel_events = None
     out["gather_4x62.5MB_bf16"] = entry(2 * 250036224, statistics.median(ms), "kernel-only events", 1)
+    pieces_c = [p_.cpu() for p_ in pieces_s]
+    cpu("gather_4x62.5MB_bf16", lambda: ts_oracle.gather(pieces_c))
+    del pieces_c
     t_full = ta.gather([ta.Batch(p) for p in pieces_t])
     row_b = 30522 * 2
     # the same loss straight from the four micro-batch outputs (no gather of s or t)
@@ -343,11 +437,21 @@ def run_kernel_table(dev):
     out["kd_masked_32x128x30522_bf16"] = entry(3 * n_sel * row_b + (4096 - n_sel) * row_b, _time_stream(f, 30),
                                                f"n_sel={n_sel}; bytes = read s,t + write grad for selected rows, "
                                                f"zero-fill of the other rows", 3)
+    if with_cpu:
+        s_c, t_c, m_c = s_full.cpu(), t_full.cpu(), mask.cpu()
+        sp_c, tp_c = list(s_c.chunk(4)), list(t_c.chunk(4))
+        cpu("kd_masked_32x128x30522_bf16", kd_cpu(s_c, t_c, 2.0, m_c))
+
+        def pieces_cpu():  # the reference's order: gather both outputs, then the loss
+            s_all = ts_oracle.gather(sp_c).requires_grad_()
+            ts_oracle.distil_ce(s_all, ts_oracle.gather(tp_c), m_c, 2.0).backward()
+        cpu("kd_masked_4_pieces_8x128x30522_bf16", pieces_cpu)
+        del s_c, t_c, m_c, sp_c, tp_c
     del s_full, t_full, f
 
     # InfoNCE: cfg4 (single pair), the symmetric two-pair call of MoCo-v3's contrastive_loss, and a
     # batch four times as large, where the fixed costs of the three launches weigh less
-    def nce_entry(n, pairs, iters, note=None):
+    def nce_entry(name, n, pairs, iters, note=None):
         mk = lambda: torch.nn.functional.normalize(torch.randn(n, 256, generator=g), dim=1).to(torch.bfloat16).to(dev)
         q1, k1 = mk(), mk()
         q2, k2 = (mk(), mk()) if pairs == 2 else (None, None)
@@ -367,10 +471,19 @@ def run_kernel_table(dev):
              "algorithmic_flop": flops, "kernel_launches": 3}
         if note:
             e["note"] = note
-        return e
-    out["infonce_4096x256_bf16"] = nce_entry(4096, 1, 50)
-    out["infonce_2_pairs_4096x256_bf16"] = nce_entry(4096, 2, 50, "both directions of the symmetric loss in one call")
-    out["infonce_16384x256_bf16"] = nce_entry(16384, 1, 20, "not one of the benchmark configurations: the same kernels at 16x the work")
+        out[name] = e
+        qc = [t.cpu().requires_grad_() for t in ((q1, q2) if pairs == 2 else (q1,))]
+        kc = [t.cpu() for t in ((k1, k2) if pairs == 2 else (k1,))]
+
+        def f_cpu():
+            for t in qc:
+                t.grad = None
+            sum(ts_oracle.infonce(a, b, 0.2) for a, b in zip(qc, kc)).backward()
+        cpu(name, f_cpu)
+    nce_entry("infonce_4096x256_bf16", 4096, 1, 50)
+    nce_entry("infonce_2_pairs_4096x256_bf16", 4096, 2, 50, "both directions of the symmetric loss in one call")
+    nce_entry("infonce_16384x256_bf16", 16384, 1, 20,
+              "not one of the benchmark configurations: the same kernels at 16x the work")
 
     # BYOL loss (latency only)
     loss = torch.empty((), device=dev)
@@ -383,6 +496,14 @@ def run_kernel_table(dev):
                                        wsb.data_ptr(), loss.data_ptr(), g1.data_ptr(), g2.data_ptr(), _lib.TS_F32,
                                        stream), "ts_byol_fwd_bwd")
     out["byol_256x128_f32"] = {"ms": round(_time_stream(f, 50), 4), "note": "latency-bound", "kernel_launches": 2}
+    oc = [t.cpu() for t in o]
+    oc[0].requires_grad_()
+    oc[1].requires_grad_()
+
+    def byol_cpu():
+        oc[0].grad = oc[1].grad = None
+        ts_oracle.byol_contrastive_loss(*oc).backward()
+    cpu("byol_256x128_f32", byol_cpu)
 
     # DeferredBatchNorm (cfg5): statistics only, statistics + normalise, backward
     x = (torch.randn(32, 256, 56, 56, generator=g) * 1.5 + 0.5).to(dev)
@@ -422,6 +543,19 @@ def run_kernel_table(dev):
         par["p"] ^= 1
     out["bn_backward_32x256x56x56_f32"] = entry(x.numel() * 20, _time_stream(bwd, 30),
                                                 "bytes = read x,dy twice + write dx", 2)
+    if with_cpu:
+        x_c, dy_c, gamma_c, beta_c = x.cpu(), dy.cpu(), gamma.cpu(), beta.cpu()
+        ora = ts_oracle.DeferredBNOracle(256, chunks=1 << 30, weight=gamma_c, bias=beta_c)
+        cpu("bn_stats_32x256x56x56_f32", lambda: ora.track(x_c))
+        cpu("bn_stats_normalise_32x256x56x56_f32", lambda: ora.forward(x_c))
+        cpu("bn_forward_train_32x256x56x56_f32", lambda: ora.forward(x_c))
+        xg, wg, bg = x_c.clone().requires_grad_(), gamma_c.clone().requires_grad_(), beta_c.clone().requires_grad_()
+        y_c = torch.nn.functional.batch_norm(xg, None, None, wg, bg, True, 0.0, 1e-5)
+
+        def bn_bwd_cpu():
+            xg.grad = wg.grad = bg.grad = None
+            y_c.backward(dy_c, retain_graph=True)
+        cpu("bn_backward_32x256x56x56_f32", bn_bwd_cpu)
     return out
 
 
@@ -500,7 +634,10 @@ def main():
         "host": res["host"],
     }
     if not args.no_kernels:
-        line["kernels"] = run_kernel_table(dev)
+        line["kernels"] = run_kernel_table(dev, with_cpu=not args.no_cpu)
+        line["kernels_cpu_note"] = ("cpu_ms: the oracle's eager PyTorch chain for the same operation and shape on "
+                                    f"{min(os.cpu_count() or 1, int(os.environ.get('OMP_NUM_THREADS', os.cpu_count() or 1)))} "
+                                    "host threads, median of up to 20 calls within ~1.2 s (a single call when one takes longer)")
     if not args.no_cpu:
         line["cpu_baseline"] = run_cpu_baseline()
     else:

@@ -15,7 +15,7 @@ LIB_PATH = os.path.join(_HERE, "libtspipe_amd.so")
 
 TS_F32, TS_BF16, TS_F16 = 0, 1, 2
 
-_lock = threading.Lock()
+_lock = threading.RLock()  # host_helper() loads lib() while holding it
 _lib = None
 
 # name -> (restype, argtypes); one row per symbol of include/tspipe_amd.h
@@ -114,6 +114,11 @@ def host_helper():
                 spec = importlib.util.spec_from_file_location("_ts_hostlist", HOST_LIB_PATH)
                 mod = importlib.util.module_from_spec(spec)
                 spec.loader.exec_module(mod)
+                if hasattr(mod, "bind_abi"):
+                    handle = lib()
+                    addr = lambda fn: ctypes.cast(fn, c_void_p).value  # noqa: E731
+                    mod.bind_abi(addr(handle.ts_infonce_workspace_bytes), addr(handle.ts_infonce_fwd_bwd),
+                                 addr(handle.ts_scale_rows))
                 _host = mod
             _host_tried = True
     return _host

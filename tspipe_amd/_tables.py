@@ -111,24 +111,24 @@ class CachedTable:
 
 
 _TABLE_CACHE_ENTRIES = 8
+# device index -> OrderedDict(key -> CachedTable); shared by all threads (the
+# key names the stream, so threads on different streams never share an entry)
+_table_caches = {}
+_table_lock = threading.Lock()
 
 
 def _table_cache(device: torch.device) -> "OrderedDict":
-    caches = getattr(_tls, "table_caches", None)
-    if caches is None:
-        caches = _tls.table_caches = {}
     key = device.index if device.index is not None else torch.cuda.current_device()
-    cache = caches.get(key)
+    cache = _table_caches.get(key)
     if cache is None:
-        cache = caches[key] = OrderedDict()
+        cache = _table_caches.setdefault(key, OrderedDict())
     return cache
 
 
 def clear_table_cache() -> None:
-    """Drops the calling thread's cached device tables."""
-    caches = getattr(_tls, "table_caches", None)
-    if caches:
-        caches.clear()
+    """Drops the cached device tables."""
+    with _table_lock:
+        _table_caches.clear()
 
 
 def stage_ema(t_ptrs: np.ndarray, s_ptrs: np.ndarray, o_ptrs: np.ndarray, numels: np.ndarray,
@@ -149,10 +149,11 @@ def stage_ema(t_ptrs: np.ndarray, s_ptrs: np.ndarray, o_ptrs: np.ndarray, numels
     key = b"".join((t_ptrs[:n].tobytes(), s_ptrs[:n].tobytes(), o_ptrs[:n].tobytes(), numels[:n].tobytes(),
                     int(chunk_elems).to_bytes(8, "little"), int(stream_id).to_bytes(8, "little")))
     cache = _table_cache(device)
-    hit = cache.get(key)
-    if hit is not None:
-        cache.move_to_end(key)
-        return hit
+    with _table_lock:
+        hit = cache.get(key)
+        if hit is not None:
+            cache.move_to_end(key)
+            return hit
     args = (t_ptrs.ctypes.data, s_ptrs.ctypes.data, o_ptrs.ctypes.data, numels.ctypes.data, n, chunk_elems)
     ring = _ring(device)
     slot = ring.acquire(0)
@@ -169,9 +170,10 @@ def stage_ema(t_ptrs: np.ndarray, s_ptrs: np.ndarray, o_ptrs: np.ndarray, numels
     # the pinned half of the slot is free again once this copy has run
     StagedTable(slot, count, chunk_elems, device).done()
     entry = CachedTable(dev, count, chunk_elems, key)
-    cache[key] = entry
-    while len(cache) > _TABLE_CACHE_ENTRIES:
-        cache.popitem(last=False)
+    with _table_lock:
+        cache[key] = entry
+        while len(cache) > _TABLE_CACHE_ENTRIES:
+            cache.popitem(last=False)
     return entry
 
 

@@ -92,6 +92,103 @@ bool all_refcounts_equal(py::list tensors, int64_t expected) {
   return true;
 }
 
+// ---------------------------------------------------------------------------
+// InfoNCE as a C++ autograd node.  The arithmetic stays in libtspipe_amd.so:
+// this node only owns the buffers and calls the C ABI through the function
+// addresses the Python side hands over (bind_abi), on the stream the forward
+// was called on.  What it saves over the Python autograd.Function is host
+// time: the backward runs on autograd's device thread without taking the
+// interpreter lock, which is most of what a step of the loss costs the host.
+// ---------------------------------------------------------------------------
+typedef size_t (*nce_ws_fn)(int64_t, int64_t, int);
+typedef int (*nce_fn)(const void*, const void*, const void*, const void*, int64_t, int64_t, float, void*, float*,
+                      void*, void*, int, void*);
+typedef int (*scale_fn)(void*, int64_t, int64_t, int64_t, const float*, int, void*);
+static nce_ws_fn g_nce_ws = nullptr;
+static nce_fn g_nce = nullptr;
+static scale_fn g_scale = nullptr;
+
+void bind_abi(uintptr_t nce_ws, uintptr_t nce, uintptr_t scale) {
+  g_nce_ws = reinterpret_cast<nce_ws_fn>(nce_ws);
+  g_nce = reinterpret_cast<nce_fn>(nce);
+  g_scale = reinterpret_cast<scale_fn>(scale);
+}
+
+inline int dtype_code(at::ScalarType t) {
+  return t == at::kFloat ? 0 : t == at::kBFloat16 ? 1 : t == at::kHalf ? 2 : -1;
+}
+
+struct InfoNCENode : public torch::autograd::Function<InfoNCENode> {
+  static at::Tensor forward(torch::autograd::AutogradContext* ctx, const at::Tensor& q1, const at::Tensor& k1,
+                            const c10::optional<at::Tensor>& q2o, const c10::optional<at::Tensor>& k2o, double tau,
+                            int64_t stream) {
+    const bool two = q2o.has_value();
+    const at::Tensor q2 = two ? *q2o : at::Tensor(), k2 = two ? *k2o : at::Tensor();
+    const int64_t n = q1.size(0), c = q1.size(1);
+    const int code = dtype_code(q1.scalar_type());
+    c10::DeviceGuard guard(q1.device());
+    const auto bytes = (int64_t)g_nce_ws(n, c, two ? 2 : 1);
+    at::Tensor ws = at::empty({bytes}, q1.options().dtype(at::kByte));
+    at::Tensor loss = at::empty({}, q1.options().dtype(at::kFloat));
+    at::Tensor g1, g2;
+    if (q1.requires_grad()) g1 = at::empty_like(q1);
+    if (two && q2.requires_grad()) g2 = at::empty_like(q2);
+    const int rc = g_nce(q1.data_ptr(), k1.data_ptr(), two ? q2.data_ptr() : nullptr, two ? k2.data_ptr() : nullptr, n,
+                         c, (float)tau, ws.data_ptr(), loss.data_ptr<float>(), g1.defined() ? g1.data_ptr() : nullptr,
+                         g2.defined() ? g2.data_ptr() : nullptr, code, reinterpret_cast<void*>(stream));
+    TORCH_CHECK(rc == 0, "ts_infonce_fwd_bwd: status ", rc);
+    ctx->saved_data["g1"] = g1;
+    ctx->saved_data["g2"] = g2;
+    ctx->saved_data["stream"] = stream;
+    ctx->saved_data["done"] = false;
+    return loss;
+  }
+
+  static torch::autograd::variable_list backward(torch::autograd::AutogradContext* ctx,
+                                                 torch::autograd::variable_list grad_out) {
+    TORCH_CHECK(!ctx->saved_data["done"].toBool(),
+                "the fused loss keeps one gradient buffer: backward can run once per forward");
+    ctx->saved_data["done"] = true;
+    // the context lets go of the buffers, so that autograd can adopt them as .grad instead of copying
+    at::Tensor g1 = ctx->saved_data["g1"].toTensor(), g2 = ctx->saved_data["g2"].toTensor();
+    ctx->saved_data["g1"] = at::Tensor();
+    ctx->saved_data["g2"] = at::Tensor();
+    void* stream = reinterpret_cast<void*>(ctx->saved_data["stream"].toInt());
+    at::Tensor go = grad_out[0];
+    if (go.scalar_type() != at::kFloat) go = go.to(at::kFloat);
+    for (at::Tensor* g : {&g1, &g2}) {
+      if (!g->defined()) continue;
+      // grad *= grad_output on the device; the kernel returns at once when it is 1
+      const int rc = g_scale(g->data_ptr(), g->size(0), g->size(1), g->size(1), go.data_ptr<float>(),
+                             dtype_code(g->scalar_type()), stream);
+      TORCH_CHECK(rc == 0, "ts_scale_rows: status ", rc);
+    }
+    return {g1, at::Tensor(), g2, at::Tensor(), at::Tensor(), at::Tensor()};
+  }
+};
+
+// Returns None when the call is not of the plain kind (then the Python
+// autograd.Function takes it and raises the proper errors): 2-D dense device
+// tensors of one shape and dtype, 64 / 128 / 256 features.
+py::object infonce(const at::Tensor& q1, const at::Tensor& k1, const c10::optional<at::Tensor>& q2,
+                   const c10::optional<at::Tensor>& k2, double tau, int64_t stream) {
+  if (!g_nce || !g_nce_ws || !g_scale) return py::none();
+  const bool two = q2.has_value();
+  if (two != k2.has_value()) return py::none();
+  const at::Tensor* all[4] = {&q1, &k1, two ? &*q2 : nullptr, two ? &*k2 : nullptr};
+  for (const at::Tensor* t : all) {
+    if (!t) continue;
+    if (!t->is_cuda() || t->dim() != 2 || !t->is_contiguous() || t->sizes() != q1.sizes() ||
+        t->scalar_type() != q1.scalar_type() || t->device() != q1.device())
+      return py::none();
+  }
+  const int64_t c = q1.size(1);
+  if ((c != 64 && c != 128 && c != 256) || dtype_code(q1.scalar_type()) < 0 || !(tau >= 0.03)) return py::none();
+  if (k1.requires_grad() || (two && k2->requires_grad())) return py::none();
+  at::Tensor loss = InfoNCENode::apply(q1, k1, q2, k2, tau, stream);
+  return py::cast(loss);
+}
+
 // Test aid: a C++ owner of a tensor that Python cannot see.  hold() keeps the
 // tensor alive inside this module until drop() is called.
 static std::vector<at::Tensor> g_held;
@@ -104,6 +201,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("pair_info", &pair_info);
   m.def("data_ptrs", &data_ptrs);
   m.def("all_refcounts_equal", &all_refcounts_equal);
+  m.def("bind_abi", &bind_abi);
+  m.def("infonce", &infonce);
   m.def("hold", &hold);
   m.def("drop", &drop);
 }

@@ -223,8 +223,7 @@ def note_reader(version: Sequence[torch.Tensor], stream: Optional["torch.cuda.St
 
 def release_pool() -> None:
     """Drops every cached output arena (memory returns to torch's allocator
-    once the caller's own references are gone) and the calling thread's
-    cached chunk tables."""
+    once the caller's own references are gone) and the cached chunk tables."""
     with _pool_lock:
         _pool.clear()
         _by_storage.clear()

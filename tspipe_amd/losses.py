@@ -482,16 +482,28 @@ class _InfoNCEFn(torch.autograd.Function):
         return out1, None, out2, None, None
 
 
+def _infonce(q1: Tensor, k1: Tensor, q2: Optional[Tensor], k2: Optional[Tensor], tau: float) -> Tensor:
+    """The plain case (dense 2-D device tensors, 64 / 128 / 256 features) goes
+    to the C++ autograd node of the host helper, whose backward needs no
+    interpreter lock; everything else, and every error, to the Python one."""
+    host = _lib.host_helper()
+    if host is not None and type(q1) is Tensor and q1.is_cuda and hasattr(host, "infonce"):
+        out = host.infonce(q1, k1, q2, k2, tau, torch.cuda.current_stream(q1.device).cuda_stream)
+        if out is not None:
+            return out
+    return _InfoNCEFn.apply(q1, k1, q2, k2, tau)
+
+
 def infonce_loss(q: Tensor, k: Tensor, tau: float) -> Tensor:
     """One direction of MoCo-v3's loss: ``CE(q^ k^T / tau, arange(N)) * 2 tau``
     (benchmarks/moco-v3/main.py:149-160)."""
-    return _InfoNCEFn.apply(q, k, None, None, float(tau))
+    return _infonce(q, k, None, None, float(tau))
 
 
 def moco_contrastive_loss_pair(online_view_1: Tensor, online_view_2: Tensor, target_view_1: Tensor,
                                target_view_2: Tensor, tau: float) -> Tensor:
     """``loss(o1, t2) + loss(o2, t1)`` in one launch (benchmarks/moco-v3/main.py:162)."""
-    return _InfoNCEFn.apply(online_view_1, target_view_2, online_view_2, target_view_1, float(tau))
+    return _infonce(online_view_1, target_view_2, online_view_2, target_view_1, float(tau))
 
 
 # ---------------------------------------------------------------------------
