@@ -238,6 +238,20 @@ int ts_byol_fwd_bwd(const void* x1, const void* y1, const void* x2, const void* 
                     int64_t c, float* workspace, float* loss_out, void* gx1, void* gx2,
                     int dtype, ts_stream_t stream);
 
+/* The same loss on projections that were never concatenated: x, y and gx of
+ * each pair come as up to 8 row blocks (the micro-batch outputs that
+ * tspipe/gpu_task.py:188-191 concatenates with torch.cat before calling
+ * loss_fn); the gradient goes straight into one buffer per piece.  Host arrays
+ * of n_pieces device pointers, piece p being a contiguous [piece_rows[p], c]
+ * matrix; the second pair's arrays may be NULL; the gx arrays may be NULL (or
+ * hold NULLs) for loss only.  workspace: 2 * (sum of piece_rows) floats.
+ * More than 8 pieces: TS_ERR_RANGE. */
+int ts_byol_pieces_fwd_bwd(const void* const* x1_pieces, const void* const* y1_pieces,
+                           void* const* gx1_pieces, const void* const* x2_pieces,
+                           const void* const* y2_pieces, void* const* gx2_pieces,
+                           const int64_t* piece_rows, int n_pieces, int64_t c, float* workspace,
+                           float* loss_out, int dtype, ts_stream_t stream);
+
 /* Squared error between student and teacher logits, forward and backward:
  *   Logits.forward (benchmarks/soft_target/kd_losses/logits.py:17-20), F.mse_loss
  *     with its mean over all elements: per_element = 1, row_mask = NULL;
@@ -292,6 +306,22 @@ size_t ts_infonce_workspace_bytes(int64_t n, int64_t c, int n_pairs);
 int ts_infonce_fwd_bwd(const void* q1, const void* k1, const void* q2, const void* k2, int64_t n,
                        int64_t c, float tau, void* workspace, float* loss_out, void* dq1,
                        void* dq2, int dtype, ts_stream_t stream);
+
+/* The same loss on embeddings that were never concatenated: q, k and dq of
+ * each pair come as up to 8 row blocks (the micro-batch outputs that
+ * tspipe/gpu_task.py:170-171,188-191 concatenates with torch.cat before calling
+ * loss_fn; the gradient goes straight into one buffer per piece).
+ *   q1_pieces, k1_pieces, dq1_pieces (and the second pair's, or NULLs): host
+ *     arrays of n_pieces device pointers, piece p being a contiguous
+ *     [piece_rows[p], c] matrix, 16-byte aligned; the dq arrays may be NULL
+ *     (or hold NULLs) for loss only.  Both pairs share piece_rows.
+ * workspace: ts_infonce_workspace_bytes(sum of piece_rows, c, n_pairs).
+ * More than 8 pieces: TS_ERR_RANGE. */
+int ts_infonce_pieces_fwd_bwd(const void* const* q1_pieces, const void* const* k1_pieces,
+                              void* const* dq1_pieces, const void* const* q2_pieces,
+                              const void* const* k2_pieces, void* const* dq2_pieces,
+                              const int64_t* piece_rows, int n_pieces, int64_t c, float tau,
+                              void* workspace, float* loss_out, int dtype, ts_stream_t stream);
 
 /* ------------------------------------------------------------------------ */
 /* DeferredBatchNorm (tspipe/batchnorm.py).                           */

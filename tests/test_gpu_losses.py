@@ -656,3 +656,85 @@ def test_kd_masked_cfg3_full_size_properties(device):
     got = s.grad.reshape(-1, 30522)[rows.to(device)].cpu().double()
     peak = ss.grad.abs().max().item()
     assert ((got - ss.grad).abs() <= 1e-3 * peak + ss.grad.abs() * 2.0 ** -8).all()
+
+
+@pytest.mark.parametrize("dtype,tau,noise,tol", [
+    # (k = q + noise: the teacher nearly agrees with the student, the regime of a trained model)
+    (torch.bfloat16, 0.2, 0.01, 6e-3), (torch.bfloat16, 0.2, 1.0, 4e-3),
+    (torch.float32, 0.2, 0.01, 4e-3), (torch.float32, 0.2, 1.0, 1e-3),
+    (torch.bfloat16, 0.07, 0.1, 1.5e-2), (torch.float32, 0.07, 0.1, 1.5e-2)])
+def test_infonce_nearly_aligned_pairs(device, dtype, tau, noise, tol):
+    # With k_i close to q_i the gradient is what is left after two cancellations: the positive key
+    # against its own soft-max weight, and the component along q that the normalisation projects out.
+    # The kernel keeps the positive key in fp32 and takes the projection from the gradient itself, so
+    # the error stays a few bf16 roundings (2^-9) of the NEGATIVE keys' weighted sum.  Bounds measured
+    # on MI355X (error over the gradient's peak): 2.3e-3 .. 3.9e-3 at tau = 0.2, 1.1e-2 at tau = 0.07,
+    # where the peak itself is 1e-7; the previous formulation (positive key rounded with the others,
+    # projection from separately accumulated sums) gave 2.7e-2 and 1.8e+2 there.
+    n, c = 512, 256
+    g = seeded(77)
+    q = torch.nn.functional.normalize(torch.randn(n, c, generator=g), dim=1)
+    k = torch.nn.functional.normalize(q + noise * torch.randn(n, c, generator=g) / 16, dim=1)
+    q, k = q.to(dtype), k.to(dtype)
+    want, (gw,) = _oracle_grad(lambda a, b: ts_oracle.infonce(a, b, tau), q, others=(k,))
+    qd = q.to(device).requires_grad_()
+    loss = ta.infonce_loss(qd, k.to(device), tau)
+    loss.backward()
+    assert abs(loss.item() - want) < 1e-3 * abs(want) + 1e-6
+    assert max_rel_to_peak(qd.grad, gw) < tol
+
+
+@pytest.mark.parametrize("dtype,c,rows", [(torch.bfloat16, 256, [96, 32, 100, 28]), (torch.float32, 128, [40, 40, 17]),
+                                         (torch.bfloat16, 64, [64])])
+def test_moco_loss_on_pieces_equals_the_gathered_loss(device, dtype, c, rows):
+    from argparse import Namespace
+    n = sum(rows)
+    g = seeded(500 + c)
+    full = [torch.randn(n, c, generator=g).to(dtype) for _ in range(4)]  # o1, o2, t1, t2
+    extra = Namespace(moco_t=0.2)
+    # the oracle on the concatenated tensors
+    want, grads = _oracle_grad(lambda a, b, t1, t2: ts_oracle.moco_contrastive_loss(a, b, t1, t2, 0.2),
+                               full[0], full[1], others=(full[2], full[3]))
+    # the gathered kernel
+    o1, o2 = full[0].to(device).requires_grad_(), full[1].to(device).requires_grad_()
+    whole = ta.moco_contrastive_loss(o1, o2, full[2].to(device), full[3].to(device), None, extra)
+    whole.backward()
+    # the same from the pieces, never concatenated
+    split = lambda t: [p.contiguous().to(device) for p in t.split(rows)]  # noqa: E731
+    p1, p2 = [p.requires_grad_() for p in split(full[0])], [p.requires_grad_() for p in split(full[1])]
+    loss = ta.moco_contrastive_loss_pieces(p1, p2, split(full[2]), split(full[3]), None, extra)
+    loss.backward()
+    assert torch.equal(loss, whole)
+    assert torch.equal(torch.cat([p.grad for p in p1]), o1.grad)
+    assert torch.equal(torch.cat([p.grad for p in p2]), o2.grad)
+    tol = 1e-3 if dtype == torch.bfloat16 else 2e-3  # fp32 inputs meet the bf16 contraction: the bf16 tolerance
+    assert rel_err(loss.item(), want) < tol
+    for got, ref in ((o1.grad, grads[0]), (o2.grad, grads[1])):
+        peak = ref.abs().max().item()
+        assert ((got.cpu().double() - ref).abs() <= tol * peak + ref.abs() * (2.0 ** -8 if dtype == torch.bfloat16 else 0)).all()
+
+
+def test_byol_loss_on_pieces_equals_the_gathered_loss(device):
+    rows = [100, 28, 64, 64]
+    n, c = sum(rows), 128
+    g = seeded(611)
+    full = [torch.randn(n, c, generator=g) for _ in range(4)]  # o1, o2, t1, t2
+    want, grads = _oracle_grad(ts_oracle.byol_contrastive_loss, full[0], full[1], others=(full[2], full[3]))
+    o1, o2 = full[0].to(device).requires_grad_(), full[1].to(device).requires_grad_()
+    whole = ta.byol_contrastive_loss(o1, o2, full[2].to(device), full[3].to(device))
+    whole.backward()
+    split = lambda t: [p.contiguous().to(device) for p in t.split(rows)]  # noqa: E731
+    p1, p2 = [p.requires_grad_() for p in split(full[0])], [p.requires_grad_() for p in split(full[1])]
+    loss = ta.byol_contrastive_loss_pieces(p1, p2, split(full[2]), split(full[3]))
+    loss.backward()
+    assert torch.equal(loss, whole)
+    assert torch.equal(torch.cat([p.grad for p in p1]), o1.grad)
+    assert torch.equal(torch.cat([p.grad for p in p2]), o2.grad)
+    assert rel_err(loss.item(), want) < 1e-5
+    assert max_rel_to_peak(o1.grad, grads[0]) < 1e-5 and max_rel_to_peak(o2.grad, grads[1]) < 1e-5
+    # argument errors: piece counts must agree, at most 8 pieces
+    with pytest.raises(ValueError):
+        ta.byol_contrastive_loss_pieces(p1, p2[:2], split(full[2]), split(full[3]))
+    nine = [torch.randn(4, c, generator=g).to(device) for _ in range(9)]
+    with pytest.raises(Exception):
+        ta.byol_contrastive_loss_pieces(nine, nine, nine, nine)

@@ -13,50 +13,62 @@
 //     maximum: no rescaling of the accumulators, and partial results of
 //     different key ranges just add up;
 //   * the keys are normalised in fp32 and rounded to bf16 once, by the prep
-//     kernel (the tile images below hold kh); the queries feed the MFMA as
-//     they are (bf16 inputs in place, fp32 / fp16 inputs through a bf16 copy)
-//     and their 1/|q| is applied as an fp32 factor after the contraction
-//     (logit_ij = <q_i, kh_j> * rq_i / tau).
+//     kernel; the queries feed the MFMA as they are (bf16 inputs in place,
+//     fp32 / fp16 inputs through a bf16 copy) and their 1/|q| is applied as an
+//     fp32 factor after the contraction (logit_ij = <q_i, kh_j> * rq_i / tau).
 //
 // Kernels:
-//   prep     per row: rq = 1/max(|q|,eps), rk, the diagonal logit; the keys,
-//            normalised and rounded to bf16, are written as "tile images":
-//            for every 32 keys the exact bytes, in the exact order, that the
-//            main kernel's MFMA operand reads want to find in LDS (below).
-//            fp32 and fp16 queries are also rounded to a bf16 copy here.
-//   main     grid (q tile of 128 rows, key split); 4 wavefronts, each owning
-//            32 q rows; per 32-key tile: S^T = Kh Q^T (MFMA 32x32x16),
-//            P = 2^(S*scale - x_max), l += P, O^T += Kh^T P (MFMA).  Tile
-//            images go from global memory straight into LDS (no registers),
-//            three tiles ahead.  Writes per-split partial l and O^T in
-//            register-native order.
-//   combine  per 32-row q tile: adds the splits and forms dq; its first
+//   prep     per row: rq = 1/max(|q|,eps), rk, and the normalised key row
+//            rounded to bf16 (row-major, zero rows up to a multiple of 64).
+//   main     grid (q tile of 64 rows, key split); 4 wavefronts = 2 pairs, a
+//            pair owning 32 q rows.  Keys come in stages of 64 (two tiles of
+//            32), global memory -> LDS without passing through registers,
+//            double-buffered.  Per stage, wavefront a of a pair computes
+//            S^T = Kh Q^T (MFMA 32x32x16) for tile a over all features,
+//            P = 2^(S*scale - x_max) rounded to bf16, hands P to its partner
+//            through LDS, and accumulates O^T += Kh^T P for ITS HALF of the
+//            features over both tiles.  So a wavefront keeps 64 accumulator
+//            registers for O and 64 for its Q fragments, fits in 256
+//            registers, and two workgroups share a CU: one's soft-max runs
+//            under the other's MFMAs.  Kh^T operands are read from the same
+//            row-major LDS tile as the Kh operands, with the transposing LDS
+//            read of gfx950 (ds_read_b64_tr_b16).
+//   combine  per 32 q rows: adds the key splits, forms dq; its first
 //            workgroup adds up the loss from the split row sums.
 //
-// Tile image (C features, KK = C/16, FB = C/32; 1 KB fragments, lane L =
-// 32h + col reads bytes 16L..16L+15 of a fragment as one MFMA A operand):
-//   fragment kk < KK        : Kh[key = col][16kk + 8h .. +7]       (first product)
-//   fragment KK + tt*FB + fb: Kh[16tt + 8gg + 4h + j][32fb + col],  (second product)
-//                             gg = 0,1, j = 0..3 -> element 4gg + j
-// so every operand read is a linear, conflict-free 1 KB of LDS.
+// Accuracy: the row sum l is taken over the bf16-rounded P that the second
+// product uses, so O / l is an exact convex combination of the rounded keys,
+// and the positive key's own term is taken out of O again (by the main kernel,
+// which knows P_ii as it rounded it) and replaced by the fp32 kh_i.  The
+// projection <qh, dqh> is formed from dqh itself.  The gradient then carries
+// the bf16 rounding of the NEGATIVE keys only, weighted by their
+// probabilities, also when P_ii -> 1.
+//
+// LDS tile: 64 key rows of C bf16, the 16-byte chunks of a row XOR-swizzled
+// with a function of the row index chosen so that both operand reads are
+// free of bank conflicts (nce_swz).
 //
 // MFMA 32x32x16 operand layout used throughout (lane l, half h = l/32):
 //   A: row l%32, contraction slots 8h..8h+7;  B: column l%32, same slots;
 //   D[i]: row (i%4) + 4h + 8(i/4), column l%32.
+#include <type_traits>
+
 #include "common.h"
 
 namespace ts {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
 
 constexpr float kNceLog2e = 1.4426950408889634f;
 constexpr float kNceLn2 = 0.6931471805599453f;
 constexpr float kNormEps = 1e-12f;  // F.normalize's eps
-constexpr int kQTile = 128;         // q rows per workgroup (32 per wavefront)
-constexpr int kKTile = 32;          // keys per inner iteration
+constexpr int kQTile = 64;          // q rows per workgroup (32 per wavefront pair)
+constexpr int kStageKeys = 64;      // keys per LDS stage (two tiles of 32)
 constexpr int kNceBlock = 256;
+constexpr int kNceMaxPieces = 8;
 
 // defined in losses.hip
 int launch_sum_scale(const float* v, int64_t n, float scale, float denom, float* out, hipStream_t stream);
@@ -69,37 +81,82 @@ struct NceLayout {
   int64_t npad;
   int splits;
   size_t head_bytes;
-  size_t off_rq, off_rk, off_diag, off_lpart, off_apart, off_kimg, off_qb, off_opart, pair_bytes;
+  size_t off_rq, off_rk, off_pdiag, off_lpart, off_khat, off_qb, off_opart, pair_bytes;
 };
 
 // One (q, k) pair's pointers; the kernels pick theirs by blockIdx.z, so the two
-// pairs of the symmetric loss share every launch.
+// pairs of the symmetric loss share every launch.  q, k and dq may come as up
+// to kNceMaxPieces row blocks (micro-batch outputs that were never
+// concatenated): piece i holds rows row0[i] .. row0[i+1]-1.  n_pieces == 0
+// means the single matrices q / k / dq.
 struct NcePair {
   const void* q;
   const void* k;
   void* dq;
-  const uint16_t* qsrc;  // bf16 queries the MFMA reads: q itself or the rounded copy
-  float *rq, *rk, *diag, *lpart, *apart, *opart;
-  uint8_t* kimg;
-  uint16_t* qb;
+  float *rq, *rk, *pdiag, *lpart, *opart;
+  uint16_t* khat;  // normalised keys, bf16, [npad][C]
+  uint16_t* qb;    // bf16 copy of the queries for fp32 / fp16 inputs, else null
+  int n_pieces;
+  int64_t row0[kNceMaxPieces];
+  const void* qp[kNceMaxPieces];
+  const void* kp[kNceMaxPieces];
+  void* dqp[kNceMaxPieces];
 };
 struct NceArgs {
   NcePair p[2];
 };
 
+struct NceRow {
+  const void* q;
+  const void* k;
+  void* dq;
+};
+
+// Pointers to one batch row of q, k and dq (T: the storage type).
+template <typename T>
+__device__ __forceinline__ NceRow nce_row(const NcePair& pr, int64_t row, int C) {
+  NceRow r;
+  if (pr.n_pieces == 0) {
+    r.q = (const T*)pr.q + row * C;
+    r.k = (const T*)pr.k + row * C;
+    r.dq = pr.dq ? (T*)pr.dq + row * C : nullptr;
+    return r;
+  }
+  const void* qb = pr.qp[0];
+  const void* kb = pr.kp[0];
+  void* db = pr.dqp[0];
+  int64_t r0 = 0;
+#pragma unroll
+  for (int i = 1; i < kNceMaxPieces; ++i) {
+    const bool ge = i < pr.n_pieces && row >= pr.row0[i];
+    qb = ge ? pr.qp[i] : qb;
+    kb = ge ? pr.kp[i] : kb;
+    db = ge ? pr.dqp[i] : db;
+    r0 = ge ? pr.row0[i] : r0;
+  }
+  const int64_t local = row - r0;
+  r.q = (const T*)qb + local * C;
+  r.k = (const T*)kb + local * C;
+  r.dq = db ? (T*)db + local * C : nullptr;
+  return r;
+}
+
 inline size_t nce_align(size_t x) { return (x + 255) & ~(size_t)255; }
 
+// Key splits: enough workgroups for two per CU (a workgroup is 4 wavefronts
+// of at most 256 registers and 72 KB of LDS, so two share a CU and overlap
+// each other's matrix and vector phases).
 inline int nce_splits(int64_t npad, int n_pairs) {
   const int64_t qtiles = npad / kQTile * n_pairs;
-  const int64_t ktiles = npad / kKTile;
-  int64_t s = (256 + qtiles - 1) / qtiles;  // one workgroup per CU: the kernel's registers allow no more
+  const int64_t stages = npad / kStageKeys;
+  int64_t s = (512 + qtiles - 1) / qtiles;
   if (s > 16) s = 16;
-  if (s > ktiles) s = ktiles;
+  if (s > stages) s = stages;
   if (s < 1) s = 1;
   return (int)s;
 }
 
-inline NceLayout nce_layout(int64_t n, int64_t c, int n_pairs, bool fp32_in) {
+inline NceLayout nce_layout(int64_t n, int64_t c, int n_pairs) {
   NceLayout L;
   L.npad = nce_round_up(n > 0 ? n : 1, kQTile);
   L.splits = nce_splits(L.npad, n_pairs);
@@ -107,71 +164,50 @@ inline NceLayout nce_layout(int64_t n, int64_t c, int n_pairs, bool fp32_in) {
   size_t o = 0;
   L.off_rq = o;       o += nce_align(L.npad * 4);
   L.off_rk = o;       o += nce_align(L.npad * 4);
-  L.off_diag = o;     o += nce_align(L.npad * 4);
+  L.off_pdiag = o;    o += nce_align(L.npad * 8);
   L.off_lpart = o;    o += nce_align((size_t)L.splits * L.npad * 4);
-  L.off_apart = o;    o += nce_align((size_t)L.splits * L.npad * 4);
-  L.off_kimg = o;     o += nce_align((size_t)L.npad * c * 4);  // npad/32 tile images of 128 c bytes
-  L.off_qb = o;       o += fp32_in ? nce_align((size_t)L.npad * c * 2) : 0;
+  L.off_khat = o;     o += nce_align((size_t)L.npad * c * 2);
+  L.off_qb = o;       o += nce_align((size_t)L.npad * c * 2);  // used for fp32 / fp16 inputs only
   L.off_opart = o;    o += nce_align((size_t)L.splits * L.npad * c * 4);
   L.pair_bytes = o;
   return L;
 }
 
 // ---------------------------------------------------------------------------
-// prep: 16-byte row loads, a group of C/VEC lanes per row; one workgroup per
-// 32 rows, whose normalised keys pass through LDS to come out as a tile image
+// prep: 16-byte row loads, a group of C/VEC lanes per row
 // ---------------------------------------------------------------------------
-template <int C>
-struct NceTile {
-  static constexpr int KK = C / 16;             // contraction steps of S^T = fragments of the first product
-  static constexpr int FB = C / 32;             // feature blocks of O^T
-  static constexpr int FRAGS = KK + 2 * FB;     // 1 KB fragments per image
-  static constexpr int BYTES = FRAGS * 1024;    // 32 KB at C = 256
-};
-
 template <typename T, int C>
 struct NcePrep {
   static constexpr int VEC = 16 / sizeof(T);  // elements per 16-byte load
   static constexpr int LPR = C / VEC;         // lanes per row (8 .. 64)
   static constexpr int RPP = kWave / LPR;     // rows per wavefront pass
-  static constexpr int ROWS = kKTile;         // rows per workgroup: one key tile
-  static constexpr int LD = C + 8;            // bf16 per LDS row (16-byte aligned rows)
+  static constexpr int ROWS = (4 * RPP > 16) ? 4 * RPP : 16;  // rows per workgroup (divides 64)
+  static constexpr int NP = ROWS / (4 * RPP);                 // passes
 };
 
 template <typename T, int C>
-__global__ __launch_bounds__(kNceBlock) void nce_prep_kernel(NceArgs args, int64_t n, int64_t npad, float scale2) {
+__global__ __launch_bounds__(kNceBlock) void nce_prep_kernel(NceArgs args, int64_t n, int64_t npad) {
   const NcePair& pr = args.p[blockIdx.z];
-  const T* __restrict__ q = (const T*)pr.q;
-  const T* __restrict__ k = (const T*)pr.k;
-  float* __restrict__ rq = pr.rq;
-  float* __restrict__ rk = pr.rk;
-  float* __restrict__ diag = pr.diag;
-  uint8_t* __restrict__ kimg = pr.kimg;
-  uint16_t* __restrict__ qb = pr.qb;
   using P = NcePrep<T, C>;
-  using TI = NceTile<C>;
-  __shared__ __attribute__((aligned(16))) uint16_t tile[P::ROWS * P::LD];
   const int lane = threadIdx.x % kWave, w = threadIdx.x / kWave;
   const int sub = lane / P::LPR, li = lane % P::LPR;  // row within the pass, lane within the row
   const int64_t row0 = (int64_t)blockIdx.x * P::ROWS;
 
   // the loads of all of this wavefront's rows go out before any is used
-  constexpr int NP = P::ROWS / (4 * P::RPP);  // passes (rows per lane group)
-  static_assert(NP >= 1 && NP * 4 * P::RPP == P::ROWS, "rows divide evenly among the wavefronts");
-  u32x4 rawq[NP], rawk[NP];
+  u32x4 rawq[P::NP], rawk[P::NP];
 #pragma unroll
-  for (int pass = 0; pass < NP; ++pass) {
-    const int64_t row = row0 + w * P::RPP + sub + pass * 4 * P::RPP;
+  for (int pass = 0; pass < P::NP; ++pass) {
+    const int64_t row = row0 + (pass * 4 + w) * P::RPP + sub;
     rawq[pass] = rawk[pass] = u32x4{0u, 0u, 0u, 0u};  // zero rows beyond n (0.0 in every dtype)
     if (row < n) {
-      rawq[pass] = *reinterpret_cast<const u32x4*>(q + row * C + li * P::VEC);
-      rawk[pass] = *reinterpret_cast<const u32x4*>(k + row * C + li * P::VEC);
+      const NceRow rp = nce_row<T>(pr, row, C);
+      rawq[pass] = *reinterpret_cast<const u32x4*>((const T*)rp.q + li * P::VEC);
+      rawk[pass] = *reinterpret_cast<const u32x4*>((const T*)rp.k + li * P::VEC);
     }
   }
 #pragma unroll
-  for (int pass = 0; pass < NP; ++pass) {
-    const int r = w * P::RPP + sub + pass * 4 * P::RPP;
-    const int64_t row = row0 + r;
+  for (int pass = 0; pass < P::NP; ++pass) {
+    const int64_t row = row0 + (pass * 4 + w) * P::RPP + sub;
     const bool live = row < n;
     float qv[P::VEC], kv[P::VEC];
     {
@@ -197,44 +233,19 @@ __global__ __launch_bounds__(kNceBlock) void nce_prep_kernel(NceArgs args, int64
     }
     const float a = live ? 1.f / fmaxf(sqrtf(sqq), kNormEps) : 0.f;
     const float b = live ? 1.f / fmaxf(sqrtf(skk), kNormEps) : 0.f;
-    // the diagonal logit uses the values the MFMA will see: q rounded to
-    // bf16, k normalised and then rounded
-    float sqk = 0.f;
-    uint16_t qbits[P::VEC];
+    uint16_t kbits[P::VEC], qbits[P::VEC];
 #pragma unroll
     for (int e = 0; e < P::VEC; ++e) {
+      kbits[e] = f32_to_bf16_bits(kv[e] * b);
       qbits[e] = f32_to_bf16_bits(qv[e]);
-      const uint16_t kbits = f32_to_bf16_bits(kv[e] * b);
-      tile[r * P::LD + li * P::VEC + e] = kbits;
-      sqk += bf16_bits_to_f32(qbits[e]) * bf16_bits_to_f32(kbits);
     }
-    if (qb) {
-#pragma unroll
-      for (int e = 0; e < P::VEC; ++e) qb[row * C + li * P::VEC + e] = qbits[e];
-    }
-#pragma unroll
-    for (int off = P::LPR / 2; off > 0; off >>= 1) sqk += __shfl_xor(sqk, off, kWave);
+    // VEC bf16 values: 16 bytes for the 2-byte input types, 8 for fp32
+    __builtin_memcpy(pr.khat + row * C + li * P::VEC, kbits, sizeof(kbits));
+    if (pr.qb) __builtin_memcpy(pr.qb + row * C + li * P::VEC, qbits, sizeof(qbits));
     if (li == 0) {
-      rq[row] = a;
-      rk[row] = b;
-      diag[row] = sqk * a * scale2;
+      pr.rq[row] = a;
+      pr.rk[row] = b;
     }
-  }
-  __syncthreads();
-  // the tile image, 16 bytes per store, consecutive threads -> consecutive chunks
-  uint8_t* img = kimg + (int64_t)blockIdx.x * TI::BYTES;
-  for (int id = threadIdx.x; id < TI::FRAGS * kWave; id += kNceBlock) {
-    const int fr = id / kWave, L = id % kWave;
-    const int col = L % 32, h = L / 32;
-    u16x8 v;
-    if (fr < TI::KK) {
-      v = *reinterpret_cast<const u16x8*>(&tile[col * P::LD + fr * 16 + h * 8]);
-    } else {
-      const int tt = (fr - TI::KK) / TI::FB, fb = (fr - TI::KK) % TI::FB;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) v[e] = tile[(16 * tt + 8 * (e / 4) + 4 * h + (e % 4)) * P::LD + fb * 32 + col];
-    }
-    *reinterpret_cast<u16x8*>(img + (int64_t)id * 16) = v;
   }
 }
 
@@ -243,289 +254,376 @@ __global__ __launch_bounds__(kNceBlock) void nce_prep_kernel(NceArgs args, int64
 // ---------------------------------------------------------------------------
 typedef __attribute__((address_space(3))) void nce_lds_void;
 typedef __attribute__((address_space(1))) const void nce_glb_void;
-constexpr int kNceBufs = 4;  // tile images in LDS: two in use (tiles t, t+1), two on their way
+typedef __attribute__((address_space(3))) s16x4 nce_lds_s16x4;
 
-template <int C>
-__global__ __launch_bounds__(kNceBlock) void nce_main_kernel(NceArgs args, int64_t n, int64_t npad, int splits,
-                                                             float scale2 /* log2(e)/tau */, int qtile_major) {
+// XOR swizzle of the 16-byte chunk index of a row of the LDS tile.  Rows that
+// differ in their low two bits get swizzles that differ in bits 2-3 and vice
+// versa, which spreads over the banks both the 16 rows a quarter-wavefront
+// reads at one chunk (first product) and the 4 rows x 4 chunks a
+// quarter-wavefront reads in a transposing load (second product).
+template <int CPR>
+__device__ __forceinline__ int nce_swz(int row) {
+  const int r = row & 15;
+  return (((r & 3) << 2) | (r >> 2)) & (CPR - 1);
+}
+
+// HP: the partial O^T goes out as bf16 (inputs and gradient are 2-byte types
+// anyway) instead of fp32, which halves the traffic between this kernel and
+// the combine.
+template <int C, bool HP>
+__global__ __launch_bounds__(kNceBlock, 2) void nce_main_kernel(NceArgs args, int64_t n, int64_t npad, int splits,
+                                                                float scale2 /* log2(e)/tau */, int qtile_major) {
   const NcePair& pr = args.p[blockIdx.z];
-  const uint16_t* __restrict__ qg = pr.qsrc;
-  const uint8_t* __restrict__ kimg = pr.kimg;
-  const float* __restrict__ rq = pr.rq;
-  float* __restrict__ lpart = pr.lpart;
-  float* __restrict__ apart = pr.apart;
-  float* __restrict__ opart = pr.opart;
-  using TI = NceTile<C>;
-  constexpr int KK = TI::KK, FB = TI::FB;
-  __shared__ __attribute__((aligned(16))) uint8_t sm[kNceBufs][TI::BYTES];
+  constexpr int KK = C / 16;          // contraction steps of S^T
+  constexpr int FBH = C / 64;         // 32-feature blocks of O^T per wavefront (half of the features)
+  constexpr int CPR = C / 8;          // 16-byte chunks per key row
+  constexpr int ROWB = C * 2;         // bytes per key row
+  constexpr int STAGE = kStageKeys * ROWB;
+  constexpr int NU = STAGE / (4 * 1024);  // 1 KB fetches per wavefront and stage
+  constexpr int KL = KK < 8 ? KK : 8;     // first-product chunk addresses kept in registers
+  // two separate arrays, so that the compiler can tell that a fetch into one
+  // does not touch what is being read from the other (it would otherwise wait
+  // for every outstanding fetch in front of every LDS read)
+  __shared__ __attribute__((aligned(1024))) uint8_t sm0[STAGE];
+  __shared__ __attribute__((aligned(1024))) uint8_t sm1[STAGE];
+  __shared__ __attribute__((aligned(1024))) uint8_t xch[2][2][2][1024];  // [pair][tile][step][lane * 16]
   const int tid = threadIdx.x, lane = tid % kWave, w = tid / kWave;
   const int col = lane % 32, h = lane / 32;
-  // Workgroup ids are dealt round-robin to the 8 XCDs.  While all key images
-  // fit an XCD's L2 (4 MB at N = 4096), the q tile is the fastest index: the
-  // key splits of a q tile run on one XCD, which streams every image through
-  // its L2 (measured 5 % faster there).  For more keys the split is the
-  // fastest index, so that an XCD keeps seeing the same share of the images.
+  const int p = w >> 1, a = w & 1;
+  // Workgroup ids are dealt round-robin to the 8 XCDs.  While all keys fit an
+  // XCD's L2, the q tile is the fastest index: the key splits of a q tile run
+  // on one XCD.  For more keys the split is the fastest index, so that an XCD
+  // keeps seeing the same share of the keys.
   const int split = qtile_major ? blockIdx.y : blockIdx.x;
   const int64_t qtile = qtile_major ? blockIdx.x : blockIdx.y;
-  const int64_t qrow = qtile * kQTile + w * 32 + col;  // the q row this lane is a column of
+  const int64_t qrow = qtile * kQTile + p * 32 + col;  // the q row this lane is a column of
 
-  const int64_t ktiles = npad / kKTile;
-  const int64_t t0 = ktiles * split / splits, t1 = ktiles * (split + 1) / splits;
+  const int64_t stages = npad / kStageKeys;
+  const int64_t s0 = stages * split / splits, s1 = stages * (split + 1) / splits;
 
-  // Global -> LDS without passing through registers: every wavefront moves a
-  // quarter of the image, 1 KB (16 bytes per lane) per instruction, and the
-  // hardware writes lane L's bytes at (LDS base) + 16 L, which is exactly
-  // the image's own order.  Completion is the issuing wavefront's vector
-  // memory counter; the barrier after it makes all four quarters visible.
-  constexpr int FPW = TI::FRAGS / 4;  // fragments per wavefront
-  auto fetch_tile = [&](int64_t t, int buf) {
-    const uint8_t* src = kimg + t * TI::BYTES + (w * FPW) * 1024 + lane * 16;
+  // Global -> LDS without passing through registers: lane L's 16 bytes land
+  // at (LDS base) + 16 L, so the swizzle is applied on the global side: the
+  // lane that fills slot (row, c') loads chunk c' ^ swz(row) of that row.
+  uint32_t goff[NU];
 #pragma unroll
-    for (int u = 0; u < FPW; ++u)
-      __builtin_amdgcn_global_load_lds((nce_glb_void*)(src + u * 1024),
-                                       (nce_lds_void*)(&sm[buf][(w * FPW + u) * 1024]), 16, 0, 0);
+  for (int u = 0; u < NU; ++u) {
+    const int slot = (w * NU + u) * kWave + lane;
+    const int row = slot / CPR, cs = slot % CPR;
+    goff[u] = (uint32_t)(row * ROWB + ((cs ^ nce_swz<CPR>(row)) << 4));
+  }
+  const uint8_t* __restrict__ khat = reinterpret_cast<const uint8_t*>(pr.khat);
+  // one 1 KB piece of a stage (piece u of this wavefront's NU)
+  auto fetch_piece = [&](int64_t st, int buf, int u) {
+    const uint8_t* src = khat + st * STAGE;
+    uint8_t* dst = (buf ? sm1 : sm0) + (w * NU + u) * 1024;
+    __builtin_amdgcn_global_load_lds((nce_glb_void*)(src + goff[u]), (nce_lds_void*)dst, 16, 0, 0);
   };
-  auto wait_fetches_and_sync = [&]() {
-    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wavefront's fetches have landed
-    __syncthreads();
+  auto fetch_stage = [&](int64_t st, int buf) {
+#pragma unroll
+    for (int u = 0; u < NU; ++u) fetch_piece(st, buf, u);
   };
-
-  if (t0 < t1) fetch_tile(t0, 0);
-  if (t0 + 1 < t1) fetch_tile(t0 + 1, 1);
-  if (t0 + 2 < t1) fetch_tile(t0 + 2, 2);
+  if (s0 < s1) fetch_stage(s0, 0);
 
   // Q fragments: B operand of S^T, resident for the whole kernel.
+  const uint16_t* qg;
+  if (pr.qb) {
+    qg = pr.qb + qrow * C;
+  } else {
+    qg = (const uint16_t*)nce_row<bf16_t>(pr, qrow < n ? qrow : 0, C).q;
+  }
   bf16x8 qf[KK];
 #pragma unroll
   for (int kk = 0; kk < KK; ++kk) {
     u32x4 raw = {0u, 0u, 0u, 0u};
-    if (qrow < n) raw = *reinterpret_cast<const u32x4*>(qg + qrow * C + kk * 16 + h * 8);
+    if (qrow < n) raw = *reinterpret_cast<const u32x4*>(qg + kk * 16 + h * 8);
     __builtin_memcpy(&qf[kk], &raw, 16);
   }
-  const float rq_i = (qrow < n) ? rq[qrow] : 0.f;
+  const float rq_i = (qrow < n) ? pr.rq[qrow] : 0.f;
   const float sc_i = rq_i * scale2;
 
-  f32x16 oacc[FB];
+  // LDS byte offsets of this lane's operand reads within a stage (the parts
+  // that depend on a compile-time index only through an addition are left to
+  // the instruction's immediate offset).
+  // first product, A operand: key row 32a + col, chunk 2kk + h
+  uint32_t ak[KL];
+  {
+    const int row = 32 * a + col;
+    const int sw = nce_swz<CPR>(row);
 #pragma unroll
-  for (int fb = 0; fb < FB; ++fb)
+    for (int kl = 0; kl < KL; ++kl) ak[kl] = (uint32_t)(row * ROWB + (((2 * kl + h) ^ sw) << 4));
+  }
+  // second product, A operand through the transposing read: within a group of
+  // 16 lanes, lane s supplies the address of 4 features of one key row and
+  // receives one feature of 4 key rows.  Group g = lane / 16 covers features
+  // 16 (g % 2) .. +15 of a 32-feature block and the key slots of half g / 2.
+  uint32_t at[FBH][2];
+  {
+    const int g = lane >> 4, s = lane & 15;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) oacc[fb][i] = 0.f;
-  float lsum = 0.f;  // sum_j P_ij
-  float asum = 0.f;  // sum_j P_ij (x_ij - x_max), x: logit in the log2 domain; x_max * l is added at the end
-  // tiles from this one on contain padded keys (never reached when n is a multiple of the tile)
-  const int64_t t_pad = n / kKTile;
-
-  // The loop is software-pipelined so that the matrix pipe and the vector
-  // ALU work at the same time: tile t+1's first product is issued before
-  // tile t's soft-max, whose exponentials then run while those MFMAs execute.
-  // Operand fragments are read from LDS a phase ahead of their MFMAs for the
-  // same reason: tile t's K^T fragments while tile t+1's first product runs,
-  // tile t+2's K fragments while tile t's second product runs.
-  bf16x8 ka[KK];
-  auto read_ka = [&](int buf) {
+    for (int r = 0; r < 2; ++r) {
+      const int row = 8 * r + 4 * (g >> 1) + (s >> 2);
+      const int sw = nce_swz<CPR>(row);
 #pragma unroll
-    for (int kk = 0; kk < KK; ++kk) {
-      const u32x4 raw = *reinterpret_cast<const u32x4*>(&sm[buf][kk * 1024 + lane * 16]);
-      __builtin_memcpy(&ka[kk], &raw, 16);
+      for (int fbl = 0; fbl < FBH; ++fbl) {
+        const int chunk = 4 * (a * FBH + fbl) + 2 * (g & 1) + ((s & 3) >> 1);
+        at[fbl][r] = (uint32_t)(row * ROWB + ((chunk ^ sw) << 4) + 8 * (s & 1));
+      }
     }
-  };
-  // S^T[key][q] = sum_f Kh[key][f] Q[q][f], as two independent accumulation
-  // chains: a dependent MFMA waits for its predecessor's result.
-  struct SAcc {
-    f32x16 a, b;
-  };
-  auto first_product = [&](SAcc& s) {
-#pragma unroll
-    for (int i = 0; i < 16; ++i) s.a[i] = s.b[i] = 0.f;
-#pragma unroll
-    for (int kk = 0; kk < KK; kk += 2) {
-      s.a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[kk], qf[kk], s.a, 0, 0, 0);
-      s.b = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[kk + 1], qf[kk + 1], s.b, 0, 0, 0);
-    }
-  };
-
-  int cur = 0;  // buffer of tile t
-  auto next_buf = [](int b) { return b == kNceBufs - 1 ? 0 : b + 1; };
-
-  // One tile; sa holds S^T of tile t on entry, sb receives tile t+1's.
-  auto step = [&](int64_t t, const SAcc& sa, SAcc& sb) {
-    const int b1 = next_buf(cur), b2 = next_buf(b1), b3 = next_buf(b2);
-    // After this barrier tile t+2 is complete in LDS (its fetches were issued
-    // a whole tile ago) and every wavefront has finished reading tile t-1,
-    // whose buffer the fetch below overwrites.
-    wait_fetches_and_sync();
-
-    // no branch (one would split the scheduling regions below): near the end
-    // the fetch repeats the last tile into a buffer nobody reads any more
-    fetch_tile(t + 3 < ktiles ? t + 3 : ktiles - 1, b3);
-    __builtin_amdgcn_sched_barrier(0);
-
-    // Phase 1: tile t+1's first product; in its shadow tile t's soft-max and
-    // the reads of tile t's K^T fragments, which take over the registers of
-    // the K fragments as the MFMAs release them.
-    first_product(sb);  // stale operands after the last tile: result unused
-    bf16x8 ta[2 * FB];
-#pragma unroll
-    for (int x = 0; x < 2 * FB; ++x) {
-      const u32x4 raw = *reinterpret_cast<const u32x4*>(&sm[cur][(KK + x) * 1024 + lane * 16]);
-      __builtin_memcpy(&ta[x], &raw, 16);
-    }
-    // P = 2^(S * rq_i * log2e/tau - x_max); keys this lane holds:
-    // key(i) = (i%4) + 4h + 8(i/4).  With u = x - x_max the kernel sums
-    // l = sum P and a' = sum P u; sum P x follows as a' + x_max l at the end.
-    float pv[16], uv[16];
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      uv[i] = fmaf(sa.a[i] + sa.b[i], sc_i, -scale2);
-      pv[i] = fast_exp2(uv[i]);
-    }
-    bf16x8 pb[2];
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      lsum += pv[i];
-      asum = fmaf(pv[i], uv[i], asum);
-      pb[i / 8][i % 8] = (__bf16)pv[i];
-    }
-    // An MFMA occupies the matrix pipe for tens of cycles, but the wavefront
-    // issues in order: only instructions placed between two MFMAs run in
-    // their shadow.  Ask the scheduler for that interleaving.
-#pragma unroll
-    for (int kk = 0; kk < KK; ++kk) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                    // one MFMA
-      __builtin_amdgcn_sched_group_barrier(0x100, (2 * FB + KK - 1) / KK, 0);  // LDS reads
-      __builtin_amdgcn_sched_group_barrier(0x002, (112 + KK - 1) / KK, 0);  // its share of the soft-max
-    }
-    __builtin_amdgcn_sched_barrier(0);
-
-    // Phase 2: O^T[f][q] += sum_key Kh^T[f][key] * P[key][q]; contraction slot
-    // 8h + 4gg + j of step tt is key 16tt + 8gg + 4h + j on both operands.
-    // In its shadow the reads of tile t+2's K fragments (stale bytes near the
-    // end, never used), into the registers the K^T fragments release.
-#pragma unroll
-    for (int tt = 0; tt < 2; ++tt)
-#pragma unroll
-      for (int fb = 0; fb < FB; ++fb)
-        oacc[fb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ta[tt * FB + fb], pb[tt], oacc[fb], 0, 0, 0);
-    read_ka(b2);
-#pragma unroll
-    for (int x = 0; x < 2 * FB; ++x) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, (KK + 2 * FB - 1) / (2 * FB), 0);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    cur = b1;
-  };
-
-  // prologue: S^T of the first tile, K fragments of the second
-  SAcc sx, sy;
-  wait_fetches_and_sync();
-  read_ka(0);
-  first_product(sx);
-  __builtin_amdgcn_sched_barrier(0);
-  read_ka(1);
-  __builtin_amdgcn_sched_barrier(0);
-
-  // two tiles per trip, so that the S^T registers alternate without copies
-  for (int64_t t = t0; t < t1; t += 2) {
-    step(t, sx, sy);
-    if (t + 1 < t1) step(t + 1, sy, sx);
   }
 
-  // The last trips fetched tiles nobody reads; they must have landed before
+  f32x16 oacc[FBH];
+#pragma unroll
+  for (int fb = 0; fb < FBH; ++fb)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) oacc[fb][i] = 0.f;
+  float lsum = 0.f;                      // sum_j of the bf16-rounded P_ij over this wavefront's tiles
+  float pd_exact = 0.f, pd_round = 0.f;  // P_ii before and after the rounding (set by the lane that meets it)
+  const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
+  // the lane of column col that holds key `col` of a diagonal tile: D register i*, half h*
+  const int hstar = (col >> 2) & 1, istar = (col & 3) + 4 * (col >> 3);
+
+  // Operand fragments are read from LDS four MFMAs ahead of their use, into a
+  // ring of four registers sets; the order below is pinned with scheduling
+  // barriers, because left to itself the compiler reads every fragment right
+  // in front of its MFMA and the LDS latency is paid sixteen times per phase.
+  constexpr int RING = 4;
+  constexpr int NSTEP = 4 * FBH;  // MFMAs of the second product per stage
+  auto one_stage = [&](int64_t st, auto buf_tag) {
+    constexpr int BUF = decltype(buf_tag)::value;
+    const uint8_t* stage = BUF ? sm1 : sm0;
+    auto read_k = [&](int kk) {
+      const u32x4 raw = *reinterpret_cast<const u32x4*>(stage + ak[kk % KL] + (kk / KL) * (KL * 32));
+      bf16x8 v;
+      __builtin_memcpy(&v, &raw, 16);
+      return v;
+    };
+    // step s of the second product: key step T = s / FBH (16 keys), feature block s % FBH
+    auto read_t = [&](int step) {
+      const int T = step / FBH, fbl = step % FBH;
+      const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((nce_lds_s16x4*)(stage + at[fbl][0] + T * 16 * ROWB));
+      const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((nce_lds_s16x4*)(stage + at[fbl][1] + T * 16 * ROWB));
+      bf16x8 v;
+      __builtin_memcpy(&v, &lo, 8);
+      __builtin_memcpy(reinterpret_cast<char*>(&v) + 8, &hi, 8);
+      return v;
+    };
+    // After this barrier stage st is complete in LDS (its fetches were issued
+    // a whole stage ago) and every wavefront has finished reading stage st-1,
+    // whose buffer the fetches below overwrite, and the exchanged P of st-1.
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wavefront's fetches have landed
+    __syncthreads();
+    // near the end the fetch repeats the last stage into the idle buffer (no branch)
+    const int64_t st_next = st + 1 < s1 ? st + 1 : s1 - 1;
+
+    // S^T[key][q] = sum_f Kh[key][f] Q[q][f] for tile a of the stage; the
+    // next stage's fetches are issued between the MFMAs
+    f32x16 sacc;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) sacc[i] = 0.f;
+    bf16x8 kr[RING];
+#pragma unroll
+    for (int i = 0; i < RING; ++i) kr[i] = read_k(i);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kr[kk % RING], qf[kk], sacc, 0, 0, 0);
+      if (kk + RING < KK) kr[kk % RING] = read_k(kk + RING);
+      if (kk < NU) fetch_piece(st_next, BUF ^ 1, kk);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // P = 2^(S * rq_i * log2e/tau - x_max), rounded to bf16; keys this lane
+    // holds: key(i) = (i%4) + 4h + 8(i/4).  The row sum is taken over the
+    // rounded values (v_dot2 of the packed pairs with ones).
+    // The soft-max is the part of a stage in which this wavefront has no MFMA
+    // to issue; with issue priority it gets through while the other
+    // workgroup's wavefront on this SIMD keeps the matrix pipe busy.
+    __builtin_amdgcn_s_setprio(2);
+    float pv[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) pv[i] = fast_exp2(fmaf(sacc[i], sc_i, -scale2));
+    bf16x8 pb[2];
+#pragma unroll
+    for (int i = 0; i < 16; i += 2) {
+      const bf16x2 pk = {(__bf16)pv[i], (__bf16)pv[i + 1]};
+      lsum = __builtin_amdgcn_fdot2_f32_bf16(pk, ones, lsum, false);
+      pb[i / 8][i % 8] = pk[0];
+      pb[i / 8][i % 8 + 1] = pk[1];
+    }
+    if (st == qtile && a == p) {  // the tile that holds this pair's own keys (uniform per wavefront)
+      float pe = pv[0];
+#pragma unroll
+      for (int i = 1; i < 16; ++i) pe = (i == istar) ? pv[i] : pe;
+      if (h == hstar) {
+        pd_exact = pe;
+        pd_round = (float)(__bf16)pe;
+      }
+    }
+    // hand this tile's P to the partner (and to the second product below)
+#pragma unroll
+    for (int t2 = 0; t2 < 2; ++t2) {
+      u32x4 raw;
+      __builtin_memcpy(&raw, &pb[t2], 16);
+      *reinterpret_cast<u32x4*>(&xch[p][a][t2][lane * 16]) = raw;
+    }
+    // the first Kh^T fragments do not depend on the exchange: on their way during the barrier
+    bf16x8 tr[RING];
+#pragma unroll
+    for (int i = 0; i < RING; ++i) tr[i] = read_t(i);
+    __builtin_amdgcn_s_setprio(0);
+    // barrier without waiting for the global -> LDS fetches of the next stage
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the P written above is in LDS
+    __builtin_amdgcn_s_barrier();
+    // O^T[f][q] += sum_key Kh^T[f][key] P[key][q] over both tiles, for this
+    // wavefront's half of the features; contraction slot 8h + 4r + j of step
+    // T is key 16T + 8r + 4h + j on both operands.
+    bf16x8 pbT[4];
+#pragma unroll
+    for (int T = 0; T < 4; ++T) {
+      const u32x4 praw = *reinterpret_cast<const u32x4*>(&xch[p][T >> 1][T & 1][lane * 16]);
+      __builtin_memcpy(&pbT[T], &praw, 16);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int step = 0; step < NSTEP; ++step) {
+      oacc[step % FBH] =
+          __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr[step % RING], pbT[step / FBH], oacc[step % FBH], 0, 0, 0);
+      if (step + RING < NSTEP) tr[step % RING] = read_t(step + RING);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+  // two stages per trip, so that the buffer index is a compile-time constant
+  for (int64_t st = s0; st < s1; st += 2) {
+    one_stage(st, std::integral_constant<int, 0>{});
+    if (st + 1 < s1) one_stage(st + 1, std::integral_constant<int, 1>{});
+  }
+
+  // The last trip fetched a stage nobody reads; it must have landed before
   // this workgroup's LDS can be handed to another one.
   __builtin_amdgcn_s_waitcnt(0x0f70);
 
-  // Padded keys (image rows of zeros) took part in the row sums with the same
-  // term for every row, 2^(0 - x_max); take this lane's share of them out.
+  // Padded keys (zero rows of Kh) took part in the row sums with the same
+  // term for every row, the rounded 2^(0 - x_max); take this lane's share out.
   {
     int cnt = 0;
-    for (int64_t t = (t0 > t_pad ? t0 : t_pad); t < t1; ++t)
+    const int64_t st_pad = n / kStageKeys;
+    for (int64_t st = (s0 > st_pad ? s0 : st_pad); st < s1; ++st)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) cnt += (t * kKTile + 4 * h + 8 * (i / 4) + (i % 4) >= n) ? 1 : 0;
-    const float u0 = fmaf(0.f, sc_i, -scale2);
-    const float c0 = (float)cnt * fast_exp2(u0);
-    lsum -= c0;
-    asum = fmaf(-c0, u0, asum);
+      for (int i = 0; i < 16; ++i) cnt += (st * kStageKeys + 32 * a + 4 * h + 8 * (i / 4) + (i % 4) >= n) ? 1 : 0;
+    const float c0 = (float)(__bf16)fast_exp2(fmaf(0.f, sc_i, -scale2));
+    lsum -= (float)cnt * c0;
   }
 
-  // partial results in register-native order
-  const float ltot = lsum + __shfl_xor(lsum, 32, kWave);
-  // sum_j P_ij x_ij = <qh_i, sum_j P_ij kh_j> * log2e/tau
-  const float atot = asum + __shfl_xor(asum, 32, kWave) + scale2 * ltot;
-  if (h == 0) {
-    lpart[(int64_t)split * npad + qtile * kQTile + w * 32 + col] = ltot;
-    apart[(int64_t)split * npad + qtile * kQTile + w * 32 + col] = atot;
+  // row sums: the two halves of a lane pair, then the two wavefronts of the pair (through LDS);
+  // the same exchange hands P~_ii to every lane of the q row's column
+  const bool has_diag = qtile >= s0 && qtile < s1;  // this split met the pair's own keys (uniform)
+  float ltot = lsum + __shfl_xor(lsum, 32, kWave);
+  __syncthreads();  // everybody is done with xch
+  float* lx = reinterpret_cast<float*>(&xch[0][0][0][0]);
+  if (a == 1 && h == 0) lx[p * 32 + col] = ltot;
+  if (has_diag && a == p && h == hstar) lx[64 + p * 32 + col] = pd_round;
+  __syncthreads();
+  if (a == 0 && h == 0) {
+    ltot += lx[p * 32 + col];
+    pr.lpart[(int64_t)split * npad + qrow] = ltot;
   }
-  const int64_t tile32 = qtile * (kQTile / 32) + w;
-  // [split][q tile of 32][fb][i/4][lane][i%4]: 16 bytes per lane and store
-  f32x4* op = reinterpret_cast<f32x4*>(opart + (((int64_t)split * (npad / 32) + tile32) * FB) * 16 * kWave);
-#pragma unroll
-  for (int fb = 0; fb < FB; ++fb)
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const f32x4 v = {oacc[fb][4 * g], oacc[fb][4 * g + 1], oacc[fb][4 * g + 2], oacc[fb][4 * g + 3]};
-      op[(fb * 4 + g) * kWave + lane] = v;
+  if (has_diag) {
+    if (a == p && h == hstar) {
+      const f32x2 v = {pd_exact, pd_round};
+      *reinterpret_cast<f32x2*>(pr.pdiag + 2 * qrow) = v;
     }
+    // The positive key's own term P~_ii kh~_i leaves the sum here, where it is
+    // known to the last bit; the combine puts (1 - P~_ii / l~) kh_i in fp32 in
+    // its place.  What is stored is the negatives' sum, which may be rounded.
+    const float prr = lx[64 + p * 32 + col];
+    const uint16_t* krow = pr.khat + qrow * C + a * (C / 2) + 4 * h;
+#pragma unroll
+    for (int fb = 0; fb < FBH; ++fb)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        uint16_t kb4[4];
+        __builtin_memcpy(kb4, krow + 32 * fb + 8 * g, 8);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) oacc[fb][4 * g + j] = fmaf(-prr, bf16_bits_to_f32(kb4[j]), oacc[fb][4 * g + j]);
+      }
+  }
+  // partial O^T in register-native order, [split][tile of 32 q rows][feature half a][fb] and then
+  //   fp32: [i/4][lane][i%4]      (16 bytes per lane and store)
+  //   bf16: [i/8][lane][i%8]      (16 bytes per lane and store)
+  const int64_t tile32 = qtile * (kQTile / 32) + p;
+  const int64_t blk = (((int64_t)split * (npad / 32) + tile32) * 2 + a) * FBH;  // 32-feature blocks in front
+  if (HP) {
+    u32x4* op = reinterpret_cast<u32x4*>(reinterpret_cast<uint16_t*>(pr.opart) + blk * 16 * kWave);
+#pragma unroll
+    for (int fb = 0; fb < FBH; ++fb)
+#pragma unroll
+      for (int g2 = 0; g2 < 2; ++g2) {
+        bf16x8 v;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = (__bf16)oacc[fb][8 * g2 + e];
+        u32x4 raw;
+        __builtin_memcpy(&raw, &v, 16);
+        op[(fb * 2 + g2) * kWave + lane] = raw;
+      }
+  } else {
+    f32x4* op = reinterpret_cast<f32x4*>(pr.opart + blk * 16 * kWave);
+#pragma unroll
+    for (int fb = 0; fb < FBH; ++fb)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const f32x4 v = {oacc[fb][4 * g], oacc[fb][4 * g + 1], oacc[fb][4 * g + 2], oacc[fb][4 * g + 3]};
+        op[(fb * 4 + g) * kWave + lane] = v;
+      }
+  }
 }
 
 // ---------------------------------------------------------------------------
-// combine: one wavefront per (32 q rows, 32-feature block); purely
-// element-wise, because <qh_i, dqh_i> follows from the row sums:
-//   <qh_i, sum_j P_ij kh_j> = (tau/log2e) A_i / l_i,  <qh_i, kh_i> = (tau/log2e) diag_i
+// combine: one workgroup per 32 q rows, two wavefronts per 32-feature block.
+// Lane (col = row, h) of wavefront (fb, g2) holds features
+// 32 fb + 8 g + 4 h + j for g = 2 g2, 2 g2 + 1 and j = 0..3, the order the
+// partial O^T was stored in.  With O'_i the negatives' sum (the main kernel
+// took the positive key's term out):
+//   dqh_i = (2/N) [ O'_i / l~_i  -  (1 - P~_ii / l~_i) kh_i ]
+// (~: rounded to bf16 as the MFMA saw it; kh_i: fp32), then the projection
+// with <qh_i, dqh_i>, summed over the row through LDS.
 // ---------------------------------------------------------------------------
 // The scalar loss, by one workgroup straight from the split row sums:
-//   loss = loss_scale / n * sum over pairs and rows of ln2 (x_max + log2 l_i - diag_i).
+//   loss = loss_scale / n * sum over pairs and rows of ln( l_i / P_ii ),
+//   l_i = (l~_i - P~_ii) + P_ii  (the positive term unrounded).
 // Re-deriving l_i here instead of reading the other workgroups' results keeps
 // the reduction inside this launch; the order of every addition is fixed.
+// Four rows per thread and trip, all loads of a trip issued before the first use.
+template <int NT>
 __device__ __forceinline__ void nce_loss_block(const NceArgs& args, int pairs, int64_t n, int64_t npad, int splits,
-                                               float scale2, float loss_scale, float* __restrict__ loss_out) {
-  __shared__ float red[kNceBlock / kWave];
+                                               float loss_scale, float* __restrict__ loss_out) {
+  __shared__ float red[NT / kWave];
   const int tid = threadIdx.x;
-  constexpr int U = 4;   // row quads per thread and trip
-  constexpr int SC = 4;  // splits per batch of loads
-  const int64_t quads = npad / 4;
+  constexpr int SC = 8;  // splits per batch of loads
   float acc = 0.f;
   for (int p = 0; p < pairs; ++p) {
     const float* __restrict__ lpart = args.p[p].lpart;
-    const float* __restrict__ diag = args.p[p].diag;
-    for (int64_t q0 = tid; q0 < quads; q0 += (int64_t)U * kNceBlock) {
-      // Loads of a batch are all issued before the first is used; a quad or a
-      // split beyond the end re-reads a valid address and is added as zero, so
-      // no branch separates the loads.
-      int64_t quad[U];
-      float keep_q[U];
-      f32x4 l[U], d[U];
-#pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const int64_t want = q0 + (int64_t)u * kNceBlock;
-        keep_q[u] = want < quads ? 1.f : 0.f;
-        quad[u] = want < quads ? want : q0;
-        l[u] = f32x4{0.f, 0.f, 0.f, 0.f};
-        d[u] = *reinterpret_cast<const f32x4*>(diag + 4 * quad[u]);
-      }
+    const float* __restrict__ pdiag = args.p[p].pdiag;
+    for (int64_t quad = tid; quad < npad / 4; quad += NT) {
+      const f32x4 d0 = *reinterpret_cast<const f32x4*>(pdiag + 8 * quad);      // rows 4q, 4q+1: exact, rounded
+      const f32x4 d1 = *reinterpret_cast<const f32x4*>(pdiag + 8 * quad + 4);  // rows 4q+2, 4q+3
+      f32x4 l = {0.f, 0.f, 0.f, 0.f};
       for (int s0 = 0; s0 < splits; s0 += SC) {
-        f32x4 v[SC][U];
-        float keep_s[SC];
+        f32x4 v[SC];
+        float keep[SC];
 #pragma unroll
         for (int c = 0; c < SC; ++c) {
-          keep_s[c] = s0 + c < splits ? 1.f : 0.f;
+          keep[c] = s0 + c < splits ? 1.f : 0.f;
           const int sp = s0 + c < splits ? s0 + c : s0;
-#pragma unroll
-          for (int u = 0; u < U; ++u) v[c][u] = *reinterpret_cast<const f32x4*>(lpart + (int64_t)sp * npad + 4 * quad[u]);
+          v[c] = *reinterpret_cast<const f32x4*>(lpart + (int64_t)sp * npad + 4 * quad);
         }
 #pragma unroll
-        for (int c = 0; c < SC; ++c)
-#pragma unroll
-          for (int u = 0; u < U; ++u) l[u] += v[c][u] * keep_s[c];
+        for (int c = 0; c < SC; ++c) l += v[c] * keep[c];
       }
+      const float pe[4] = {d0[0], d0[2], d1[0], d1[2]}, pr[4] = {d0[1], d0[3], d1[1], d1[3]};
 #pragma unroll
-      for (int u = 0; u < U; ++u) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const bool live = keep_q[u] != 0.f && 4 * quad[u] + j < n;
-          const float term = kNceLn2 * (scale2 + log2f(l[u][j]) - d[u][j]);
-          acc += live ? term : 0.f;
-        }
+      for (int j = 0; j < 4; ++j) {
+        const float t = kNceLn2 * (log2f((l[j] - pr[j]) + pe[j]) - log2f(pe[j]));
+        acc += (4 * quad + j < n) ? t : 0.f;
       }
     }
   }
@@ -535,123 +633,110 @@ __device__ __forceinline__ void nce_loss_block(const NceArgs& args, int pairs, i
   if (tid == 0) {
     float total = 0.f;
 #pragma unroll
-    for (int w = 0; w < kNceBlock / kWave; ++w) total += red[w];
+    for (int w = 0; w < NT / kWave; ++w) total += red[w];
     *loss_out = total * loss_scale / (float)n;
   }
 }
 
-template <typename T, int C>
-__global__ __launch_bounds__(kNceBlock) void nce_combine_kernel(NceArgs args, int64_t n, int64_t npad, int splits,
-                                                                float scale2, float loss_scale,
-                                                                float* __restrict__ loss_out) {
-  // workgroup 0 of the first pair computes the loss; the (q tile, feature block) items start at workgroup 1
+template <typename T, int C, bool HP>
+__global__ __launch_bounds__(4 * C) void nce_combine_kernel(NceArgs args, int64_t n, int64_t npad, int splits,
+                                                            float loss_scale, float* __restrict__ loss_out) {
+  constexpr int NW = C / 16;  // wavefronts: two per 32-feature block
+  constexpr int FBH = C / 64;
+  // workgroup 0 of the first pair computes the loss; the 32-row tiles start at workgroup 1
   if (blockIdx.x == 0) {
-    if (blockIdx.z == 0) nce_loss_block(args, (int)gridDim.z, n, npad, splits, scale2, loss_scale, loss_out);
+    if (blockIdx.z == 0) nce_loss_block<4 * C>(args, (int)gridDim.z, n, npad, splits, loss_scale, loss_out);
     return;
   }
   const NcePair& pr = args.p[blockIdx.z];
-  const T* __restrict__ q = (const T*)pr.q;
-  const T* __restrict__ k = (const T*)pr.k;
-  const float* __restrict__ rq = pr.rq;
-  const float* __restrict__ rk = pr.rk;
-  const float* __restrict__ diag = pr.diag;
-  const float* __restrict__ lpart = pr.lpart;
-  const float* __restrict__ apart = pr.apart;
-  const float* __restrict__ opart = pr.opart;
-  T* __restrict__ dq = (T*)pr.dq;
-  constexpr int FB = C / 32;
-  const int lane = threadIdx.x % kWave, w = threadIdx.x / kWave;
+  __shared__ float dots[NW][32];
+  const int lane = threadIdx.x % kWave, wv = threadIdx.x / kWave;
+  const int fb = wv >> 1, g2 = wv & 1;
   const int col = lane % 32, h = lane / 32;
-  const int64_t item = (int64_t)(blockIdx.x - 1) * (kNceBlock / kWave) + w;
-  const int64_t tile32 = item / FB;
-  const int fb = (int)(item % FB);
-  if (tile32 >= npad / 32) return;
+  const int64_t tile32 = (int64_t)blockIdx.x - 1;
   const int64_t row = tile32 * 32 + col;
   const bool live = row < n;
+  const int a = fb / FBH, fbl = fb % FBH;
 
-  // The kernel is bound by memory latency, not by arithmetic: every load whose
-  // address is known up front is issued before the first use of any of them
-  // (the row sums, the k and q values of this lane, the first four splits of
-  // the partial O^T).
+  // Bound by memory latency, not arithmetic: every load is issued before the
+  // first use of any of them (up to 8 splits; more come in further rounds).
   const int64_t qk_row = live ? row : 0;  // padded rows read row 0 and discard it
-  T kv[4][4], qv[4][4];
-  if (dq) {
+  const NceRow rp = nce_row<T>(pr, qk_row, C);
+  T kv[2][4], qv[2][4];
 #pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const int f0 = 32 * fb + 8 * g + 4 * h;  // this lane holds features f0 .. f0+3 of its row
-      __builtin_memcpy(kv[g], k + qk_row * C + f0, sizeof(kv[g]));
-      __builtin_memcpy(qv[g], q + qk_row * C + f0, sizeof(qv[g]));
-    }
+  for (int gg = 0; gg < 2; ++gg) {
+    const int f0 = 32 * fb + 8 * (2 * g2 + gg) + 4 * h;  // this lane holds features f0 .. f0+3 of its row
+    __builtin_memcpy(kv[gg], (const T*)rp.k + f0, sizeof(kv[gg]));
+    __builtin_memcpy(qv[gg], (const T*)rp.q + f0, sizeof(qv[gg]));
   }
-  const float d = diag[row];
-  const float rq_i = rq[row], rk_i = rk[row];
-  float l = 0.f, A = 0.f;
-  {
-    int s = 0;
-    for (; s + 4 <= splits; s += 4) {
-      float lv[4], av[4];
+  const f32x2 pd = *reinterpret_cast<const f32x2*>(pr.pdiag + 2 * row);
+  const float rq_i = pr.rq[row], rk_i = pr.rk[row];
+  float o[8];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        lv[u] = lpart[(int64_t)(s + u) * npad + row];
-        av[u] = apart[(int64_t)(s + u) * npad + row];
+  for (int i = 0; i < 8; ++i) o[i] = 0.f;
+  float l = 0.f;
+  const int64_t blk = (tile32 * 2 + a) * FBH + fbl;                // 32-feature blocks in front, within a split
+  const int64_t split_blocks = (npad / 32) * 2 * FBH;              // 32-feature blocks per split
+  constexpr int SC = 8;
+  for (int s0 = 0; s0 < splits; s0 += SC) {
+    float lv[SC];
+    f32x4 vf[SC][2];
+    u32x4 vh[SC];
+#pragma unroll
+    for (int u = 0; u < SC; ++u) {
+      const int sp = s0 + u < splits ? s0 + u : s0;  // a split beyond the end re-reads a valid one and is dropped
+      lv[u] = pr.lpart[(int64_t)sp * npad + row];
+      const int64_t b = (int64_t)sp * split_blocks + blk;
+      if (HP) {
+        vh[u] = reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(pr.opart) + b * 16 * kWave)[g2 * kWave + lane];
+      } else {
+        const f32x4* src = reinterpret_cast<const f32x4*>(pr.opart + b * 16 * kWave);
+        vf[u][0] = src[(2 * g2) * kWave + lane];
+        vf[u][1] = src[(2 * g2 + 1) * kWave + lane];
       }
+    }
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        l += lv[u];
-        A += av[u];
+    for (int u = 0; u < SC; ++u) {
+      if (s0 + u >= splits) continue;
+      l += lv[u];
+      if (HP) {
+        uint16_t hb[8];
+        __builtin_memcpy(hb, &vh[u], 16);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[e] += bf16_bits_to_f32(hb[e]);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[e] += vf[u][e / 4][e % 4];
       }
     }
-    for (; s < splits; ++s) {
-      l += lpart[(int64_t)s * npad + row];
-      A += apart[(int64_t)s * npad + row];
-    }
   }
-  if (!dq) return;
-
-  float o[16];
-#pragma unroll
-  for (int i = 0; i < 16; ++i) o[i] = 0.f;
-  const int64_t split_stride = (npad / 32) * FB * 16 * kWave;  // floats
-  const f32x4* op0 = reinterpret_cast<const f32x4*>(opart + (tile32 * FB + fb) * 16 * kWave) + lane;
-  int s0 = 0;
-  for (; s0 + 4 <= splits; s0 += 4) {
-    f32x4 v[4][4];
-#pragma unroll
-    for (int u = 0; u < 4; ++u)
-#pragma unroll
-      for (int g = 0; g < 4; ++g)
-        v[u][g] = reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(op0) + (s0 + u) * split_stride)[g * kWave];
-#pragma unroll
-    for (int u = 0; u < 4; ++u)
-#pragma unroll
-      for (int g = 0; g < 4; ++g)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) o[4 * g + j] += v[u][g][j];
-  }
-  for (; s0 < splits; ++s0) {
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const f32x4 v = reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(op0) + s0 * split_stride)[g * kWave];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) o[4 * g + j] += v[j];
-    }
-  }
-  if (!live) return;
   const float inv_l = 1.f / l;
   const float gn = 2.f / (float)n;
-  // below eps the norm is the constant eps and normalize() is linear: no projection
-  const bool clamped = rq_i >= 1.f / kNormEps;
-  const float dot = clamped ? 0.f : gn * (A * inv_l - d) / scale2;
+  const float w_neg = (l - pd[1]) * inv_l;  // 1 - P~_ii / l~
+  float dqh[8], qh[8];
+  float dot = 0.f;
 #pragma unroll
-  for (int g = 0; g < 4; ++g) {
-    const int f0 = 32 * fb + 8 * g + 4 * h;
+  for (int e = 0; e < 8; ++e) {
+    dqh[e] = gn * (o[e] * inv_l - w_neg * (to_f32(kv[e / 4][e % 4]) * rk_i));
+    qh[e] = to_f32(qv[e / 4][e % 4]) * rq_i;
+    dot = fmaf(qh[e], dqh[e], dot);
+  }
+  dot += __shfl_xor(dot, 32, kWave);
+  if (h == 0) dots[wv][col] = dot;
+  __syncthreads();
+  if (!live || !rp.dq) return;
+  float total = 0.f;
+#pragma unroll
+  for (int x = 0; x < NW; ++x) total += dots[x][col];
+  // below eps the norm is the constant eps and normalize() is linear: no projection
+  if (rq_i >= 1.f / kNormEps) total = 0.f;
+#pragma unroll
+  for (int gg = 0; gg < 2; ++gg) {
+    const int f0 = 32 * fb + 8 * (2 * g2 + gg) + 4 * h;
     T out[4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const float dqh = gn * (o[4 * g + j] * inv_l - to_f32(kv[g][j]) * rk_i);
-      out[j] = from_f32<T>((dqh - to_f32(qv[g][j]) * rq_i * dot) * rq_i);
-    }
-    __builtin_memcpy(dq + row * C + f0, out, sizeof(out));
+    for (int j = 0; j < 4; ++j) out[j] = from_f32<T>((dqh[4 * gg + j] - qh[4 * gg + j] * total) * rq_i);
+    __builtin_memcpy((T*)rp.dq + f0, out, sizeof(out));
   }
 }
 
@@ -660,21 +745,23 @@ int nce_run(const NceArgs& args, int pairs, int64_t n, float tau, const NceLayou
             hipStream_t stream) {
   const float scale2 = kNceLog2e / tau;
   const unsigned z = (unsigned)pairs;
-  hipLaunchKernelGGL((nce_prep_kernel<T, C>), dim3((unsigned)(L.npad / kKTile), 1, z), dim3(kNceBlock), 0, stream, args,
-                     n, L.npad, scale2);
+  using P = NcePrep<T, C>;
+  hipLaunchKernelGGL((nce_prep_kernel<T, C>), dim3((unsigned)(L.npad / P::ROWS), 1, z), dim3(kNceBlock), 0, stream, args,
+                     n, L.npad);
   int rc = check_launch();
   if (rc) return rc;
   // see the kernel for the choice of the fastest grid index
-  const bool qtile_major = (size_t)L.npad * C * 4 <= ((size_t)4 << 20);
+  const bool qtile_major = (size_t)L.npad * C * 2 <= ((size_t)4 << 20);
   const dim3 main_grid = qtile_major ? dim3((unsigned)(L.npad / kQTile), (unsigned)L.splits, z)
                                      : dim3((unsigned)L.splits, (unsigned)(L.npad / kQTile), z);
-  hipLaunchKernelGGL((nce_main_kernel<C>), main_grid, dim3(kNceBlock), 0, stream, args, n, L.npad, L.splits, scale2,
+  // fp32 inputs keep fp32 partial sums; the 2-byte types, whose gradient is rounded to 2^-9 anyway, bf16 ones
+  constexpr bool HP = sizeof(T) == 2;
+  hipLaunchKernelGGL((nce_main_kernel<C, HP>), main_grid, dim3(kNceBlock), 0, stream, args, n, L.npad, L.splits, scale2,
                      qtile_major ? 1 : 0);
   rc = check_launch();
   if (rc) return rc;
-  const int64_t items = L.npad / 32 * (C / 32);  // a multiple of 4: npad is a multiple of 128
-  hipLaunchKernelGGL((nce_combine_kernel<T, C>), dim3((unsigned)(items / 4 + 1), 1, z), dim3(kNceBlock), 0, stream,
-                     args, n, L.npad, L.splits, scale2, 2.f * tau, loss_out);
+  hipLaunchKernelGGL((nce_combine_kernel<T, C, HP>), dim3((unsigned)(L.npad / 32 + 1), 1, z), dim3(4 * C), 0, stream,
+                     args, n, L.npad, L.splits, 2.f * tau, loss_out);
   return check_launch();
 }
 
@@ -689,14 +776,49 @@ int nce_dispatch_c(const NceArgs& args, int pairs, int64_t n, int64_t c, float t
   }
 }
 
+// Fills the per-pair workspace pointers and launches.
+int nce_launch(NceArgs& args, int pairs, int64_t n, int64_t c, float tau, void* workspace, float* loss_out,
+               int dtype, hipStream_t st) {
+  const NceLayout L = nce_layout(n, c, pairs);
+  char* ws = (char*)workspace;
+  for (int p = 0; p < 2; ++p) {
+    const int src = p < pairs ? p : 0;  // an unused second slot mirrors the first
+    if (p >= pairs) args.p[p] = args.p[0];
+    char* wsp = ws + L.head_bytes + (size_t)src * L.pair_bytes;
+    NcePair& P = args.p[p];
+    P.rq = (float*)(wsp + L.off_rq);
+    P.rk = (float*)(wsp + L.off_rk);
+    P.pdiag = (float*)(wsp + L.off_pdiag);
+    P.lpart = (float*)(wsp + L.off_lpart);
+    P.opart = (float*)(wsp + L.off_opart);
+    P.khat = (uint16_t*)(wsp + L.off_khat);
+    // fp32 and fp16 queries are rounded to a bf16 copy for the MFMA; bf16 ones are read in place
+    P.qb = dtype != TS_BF16 ? (uint16_t*)(wsp + L.off_qb) : nullptr;
+  }
+  // loss = 2 tau / n * sum over all pairs' rows, written by the combine launch
+  if (dtype == TS_F32) return nce_dispatch_c<float>(args, pairs, n, c, tau, L, loss_out, st);
+  if (dtype == TS_F16) return nce_dispatch_c<f16_t>(args, pairs, n, c, tau, L, loss_out, st);
+  return nce_dispatch_c<bf16_t>(args, pairs, n, c, tau, L, loss_out, st);
+}
+
+inline void nce_clear_pieces(NcePair& P) {
+  P.q = P.k = nullptr;
+  P.dq = nullptr;
+  P.n_pieces = 0;
+  for (int i = 0; i < kNceMaxPieces; ++i) {
+    P.row0[i] = 0;
+    P.qp[i] = P.kp[i] = nullptr;
+    P.dqp[i] = nullptr;
+  }
+}
+
 }  // namespace ts
 
 extern "C" {
 
 size_t ts_infonce_workspace_bytes(int64_t n, int64_t c, int n_pairs) {
   if (n < 0 || c <= 0 || n_pairs < 1 || n_pairs > 2) return 0;
-  // sized for fp32 inputs (the larger layout) so one query serves both dtypes
-  const ts::NceLayout L = ts::nce_layout(n, c, n_pairs, true);
+  const ts::NceLayout L = ts::nce_layout(n, c, n_pairs);
   return L.head_bytes + L.pair_bytes * (size_t)n_pairs;
 }
 
@@ -720,31 +842,56 @@ int ts_infonce_fwd_bwd(const void* q1, const void* k1, const void* q2, const voi
     // cross entropy over zero rows: mean of nothing = NaN, as torch gives
     return ts::launch_sum_scale((const float*)workspace, 0, 1.f, 0.f, loss_out, st);
   }
-  const ts::NceLayout L = ts::nce_layout(n, c, pairs, true);
-  char* ws = (char*)workspace;
   ts::NceArgs args;
   for (int p = 0; p < 2; ++p) {
-    const int src = p < pairs ? p : 0;  // an unused second slot mirrors the first
-    char* wsp = ws + L.head_bytes + (size_t)src * L.pair_bytes;
-    ts::NcePair& P = args.p[p];
-    P.q = src ? q2 : q1;
-    P.k = src ? k2 : k1;
-    P.dq = src ? dq2 : dq1;
-    P.rq = (float*)(wsp + L.off_rq);
-    P.rk = (float*)(wsp + L.off_rk);
-    P.diag = (float*)(wsp + L.off_diag);
-    P.lpart = (float*)(wsp + L.off_lpart);
-    P.apart = (float*)(wsp + L.off_apart);
-    P.opart = (float*)(wsp + L.off_opart);
-    P.kimg = (uint8_t*)(wsp + L.off_kimg);
-    // fp32 and fp16 queries are rounded to a bf16 copy for the MFMA; bf16 ones are read in place
-    P.qb = dtype != TS_BF16 ? (uint16_t*)(wsp + L.off_qb) : nullptr;
-    P.qsrc = dtype != TS_BF16 ? P.qb : (const uint16_t*)P.q;
+    ts::nce_clear_pieces(args.p[p]);
+    const int src = p < pairs ? p : 0;
+    args.p[p].q = src ? q2 : q1;
+    args.p[p].k = src ? k2 : k1;
+    args.p[p].dq = src ? dq2 : dq1;
   }
-  // loss = 2 tau / n * sum over all pairs' rows, written by the combine launch
-  if (dtype == TS_F32) return ts::nce_dispatch_c<float>(args, pairs, n, c, tau, L, loss_out, st);
-  if (dtype == TS_F16) return ts::nce_dispatch_c<ts::f16_t>(args, pairs, n, c, tau, L, loss_out, st);
-  return ts::nce_dispatch_c<ts::bf16_t>(args, pairs, n, c, tau, L, loss_out, st);
+  return ts::nce_launch(args, pairs, n, c, tau, workspace, loss_out, dtype, st);
+}
+
+int ts_infonce_pieces_fwd_bwd(const void* const* q1_pieces, const void* const* k1_pieces, void* const* dq1_pieces,
+                              const void* const* q2_pieces, const void* const* k2_pieces, void* const* dq2_pieces,
+                              const int64_t* piece_rows, int n_pieces, int64_t c, float tau, void* workspace,
+                              float* loss_out, int dtype, ts_stream_t stream) {
+  if (!q1_pieces || !k1_pieces || !piece_rows || !workspace || !loss_out) return TS_ERR_ARG;
+  if ((q2_pieces == nullptr) != (k2_pieces == nullptr)) return TS_ERR_ARG;
+  if (n_pieces < 1 || n_pieces > ts::kNceMaxPieces) return TS_ERR_RANGE;
+  if (!(tau > 0.f)) return TS_ERR_ARG;
+  if (c != 64 && c != 128 && c != 256) return TS_ERR_ARG;
+  if (dtype != TS_F32 && dtype != TS_BF16 && dtype != TS_F16) return TS_ERR_ARG;
+  if (tau < 0.03f) return TS_ERR_RANGE;
+  if ((uintptr_t)workspace & 255u) return TS_ERR_ALIGN;
+  const int pairs = q2_pieces ? 2 : 1;
+  ts::NceArgs args;
+  int64_t n = 0;
+  for (int p = 0; p < 2; ++p) {
+    ts::NcePair& P = args.p[p];
+    ts::nce_clear_pieces(P);
+    if (p >= pairs) continue;
+    const void* const* qs = p ? q2_pieces : q1_pieces;
+    const void* const* ks = p ? k2_pieces : k1_pieces;
+    void* const* ds = p ? dq2_pieces : dq1_pieces;
+    const bool want = ds && ds[0];
+    int64_t rows = 0;
+    for (int i = 0; i < n_pieces; ++i) {
+      if (piece_rows[i] <= 0 || !qs[i] || !ks[i]) return TS_ERR_ARG;
+      if (want != (ds && ds[i] != nullptr)) return TS_ERR_ARG;
+      if (((uintptr_t)qs[i] | (uintptr_t)ks[i] | (uintptr_t)(want ? ds[i] : nullptr)) & 15u) return TS_ERR_ALIGN;
+      P.row0[i] = rows;
+      P.qp[i] = qs[i];
+      P.kp[i] = ks[i];
+      P.dqp[i] = want ? ds[i] : nullptr;
+      rows += piece_rows[i];
+    }
+    P.n_pieces = n_pieces;
+    n = rows;
+  }
+  if (n > (1 << 24)) return TS_ERR_RANGE;
+  return ts::nce_launch(args, pairs, n, c, tau, workspace, loss_out, dtype, (hipStream_t)stream);
 }
 
 }  // extern "C"

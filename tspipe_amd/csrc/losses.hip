@@ -36,23 +36,45 @@ __global__ __launch_bounds__(256) void scale_rows_kernel(T* __restrict__ grad, i
 }
 
 // ---- BYOL ---------------------------------------------------------------
+// The operands of both (x, y) pairs as up to kByolMaxPieces row blocks each
+// (micro-batch outputs that were never concatenated): piece i holds rows
+// row0[i] .. row0[i+1]-1.  A single matrix is one piece.
+constexpr int kByolMaxPieces = 8;
+struct ByolArgs {
+  int n_pieces;
+  int64_t row0[kByolMaxPieces];
+  const void* x[2][kByolMaxPieces];
+  const void* y[2][kByolMaxPieces];
+  void* g[2][kByolMaxPieces];  // per pair: all null or all set
+};
+
 // One wavefront per (pair, row).  x^ = x / max(|x|, eps) as F.normalize does.
 template <typename T>
-__global__ __launch_bounds__(256) void byol_rows_kernel(const T* __restrict__ x1, const T* __restrict__ y1,
-                                                        const T* __restrict__ x2, const T* __restrict__ y2,
-                                                        int64_t n, int64_t c, float* __restrict__ row_loss,
-                                                        T* __restrict__ gx1, T* __restrict__ gx2) {
+__global__ __launch_bounds__(256) void byol_rows_kernel(const ByolArgs args, int pairs, int64_t n, int64_t c,
+                                                        float* __restrict__ row_loss) {
   constexpr float kEps = 1e-12f;
   const int lane = threadIdx.x % kWave;
   const int64_t vrow = (int64_t)blockIdx.x * (256 / kWave) + threadIdx.x / kWave;
-  const int64_t total = x2 ? 2 * n : n;
+  const int64_t total = pairs * n;
   if (vrow >= total) return;
-  const bool second = vrow >= n;
+  const int second = vrow >= n ? 1 : 0;
   const int64_t row = second ? vrow - n : vrow;
-  const T* x = (second ? x2 : x1) + row * c;
-  const T* y = (second ? y2 : y1) + row * c;
-  T* gx = second ? gx2 : gx1;
-  if (gx) gx += row * c;
+  // the piece is found with a chain of selects (uniform per wavefront)
+  const void* xb = args.x[second][0];
+  const void* yb = args.y[second][0];
+  void* gb = args.g[second][0];
+  int64_t r0 = 0;
+#pragma unroll
+  for (int i = 1; i < kByolMaxPieces; ++i) {
+    const bool ge = i < args.n_pieces && row >= args.row0[i];
+    xb = ge ? args.x[second][i] : xb;
+    yb = ge ? args.y[second][i] : yb;
+    gb = ge ? args.g[second][i] : gb;
+    r0 = ge ? args.row0[i] : r0;
+  }
+  const T* x = (const T*)xb + (row - r0) * c;
+  const T* y = (const T*)yb + (row - r0) * c;
+  T* gx = gb ? (T*)gb + (row - r0) * c : nullptr;
 
   float sxx = 0.f, syy = 0.f, sxy = 0.f;
   for (int64_t i = lane; i < c; i += kWave) {
@@ -246,18 +268,25 @@ int launch_cosine(const void* x, const void* y, const uint8_t* mask, int64_t n, 
 }
 
 template <typename T>
-int launch_byol(const void* x1, const void* y1, const void* x2, const void* y2, int64_t n, int64_t c,
-                float* ws, float* loss_out, void* gx1, void* gx2, hipStream_t stream) {
-  const int64_t total = x2 ? 2 * n : n;
+int launch_byol(const ByolArgs& args, int pairs, int64_t n, int64_t c, float* ws, float* loss_out,
+                hipStream_t stream) {
+  const int64_t total = pairs * n;
   const int64_t blocks = (total + 3) / 4;
-  hipLaunchKernelGGL((byol_rows_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, stream,
-                     (const T*)x1, (const T*)y1, (const T*)x2, (const T*)y2, n, c, ws, (T*)gx1,
-                     (T*)gx2);
+  hipLaunchKernelGGL((byol_rows_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, stream, args, pairs, n, c, ws);
   int rc = check_launch();
   if (rc) return rc;
   hipLaunchKernelGGL(sum_scale_kernel, dim3(1), dim3(1024), 0, stream, ws, total, 1.0f,
                      (const int*)nullptr, (float)n, loss_out);
   return check_launch();
+}
+
+int byol_dispatch(const ByolArgs& args, int pairs, int64_t n, int64_t c, float* ws, float* loss_out, int dtype,
+                  hipStream_t st) {
+  switch (dtype) {
+    case TS_F32: return launch_byol<float>(args, pairs, n, c, ws, loss_out, st);
+    case TS_BF16: return launch_byol<bf16_t>(args, pairs, n, c, ws, loss_out, st);
+    default: return launch_byol<f16_t>(args, pairs, n, c, ws, loss_out, st);
+  }
 }
 
 inline size_t dtype_size(int dtype) { return dtype == TS_F32 ? 4 : 2; }
@@ -380,14 +409,49 @@ int ts_byol_fwd_bwd(const void* x1, const void* y1, const void* x2, const void* 
                        (int64_t)0, 1.0f, (const int*)nullptr, 0.f, loss_out);
     return ts::check_launch();
   }
-  switch (dtype) {
-    case TS_F32:
-      return ts::launch_byol<float>(x1, y1, x2, y2, n, c, workspace, loss_out, gx1, gx2, st);
-    case TS_BF16:
-      return ts::launch_byol<ts::bf16_t>(x1, y1, x2, y2, n, c, workspace, loss_out, gx1, gx2, st);
-    default:
-      return ts::launch_byol<ts::f16_t>(x1, y1, x2, y2, n, c, workspace, loss_out, gx1, gx2, st);
+  ts::ByolArgs args = {};
+  args.n_pieces = 1;
+  args.x[0][0] = x1;
+  args.y[0][0] = y1;
+  args.g[0][0] = gx1;
+  args.x[1][0] = x2;
+  args.y[1][0] = y2;
+  args.g[1][0] = gx2;
+  return ts::byol_dispatch(args, x2 ? 2 : 1, n, c, workspace, loss_out, dtype, st);
+}
+
+int ts_byol_pieces_fwd_bwd(const void* const* x1_pieces, const void* const* y1_pieces, void* const* gx1_pieces,
+                           const void* const* x2_pieces, const void* const* y2_pieces, void* const* gx2_pieces,
+                           const int64_t* piece_rows, int n_pieces, int64_t c, float* workspace, float* loss_out,
+                           int dtype, ts_stream_t stream) {
+  if (!x1_pieces || !y1_pieces || !piece_rows || !workspace || !loss_out) return TS_ERR_ARG;
+  if ((x2_pieces == nullptr) != (y2_pieces == nullptr)) return TS_ERR_ARG;
+  if (n_pieces < 1 || n_pieces > ts::kByolMaxPieces) return TS_ERR_RANGE;
+  if (c <= 0) return TS_ERR_ARG;
+  if (dtype != TS_F32 && dtype != TS_BF16 && dtype != TS_F16) return TS_ERR_ARG;
+  const int pairs = x2_pieces ? 2 : 1;
+  ts::ByolArgs args = {};
+  args.n_pieces = n_pieces;
+  int64_t n = 0;
+  for (int p = 0; p < pairs; ++p) {
+    const void* const* xs = p ? x2_pieces : x1_pieces;
+    const void* const* ys = p ? y2_pieces : y1_pieces;
+    void* const* gs = p ? gx2_pieces : gx1_pieces;
+    const bool want = gs && gs[0];
+    int64_t rows = 0;
+    for (int i = 0; i < n_pieces; ++i) {
+      if (piece_rows[i] <= 0 || !xs[i] || !ys[i]) return TS_ERR_ARG;
+      if (want != (gs && gs[i] != nullptr)) return TS_ERR_ARG;
+      args.row0[i] = rows;
+      args.x[p][i] = xs[i];
+      args.y[p][i] = ys[i];
+      args.g[p][i] = want ? gs[i] : nullptr;
+      rows += piece_rows[i];
+    }
+    n = rows;
   }
+  if (n > (1 << 28)) return TS_ERR_RANGE;
+  return ts::byol_dispatch(args, pairs, n, c, workspace, loss_out, dtype, (hipStream_t)stream);
 }
 
 }  // extern "C"

@@ -507,6 +507,101 @@ def moco_contrastive_loss_pair(online_view_1: Tensor, online_view_2: Tensor, tar
 
 
 # ---------------------------------------------------------------------------
+# The self-supervised losses on micro-batch outputs that were never gathered
+# ---------------------------------------------------------------------------
+
+class _PairPiecesFn(torch.autograd.Function):
+    """InfoNCE or BYOL loss over two (student, teacher) pairs whose operands
+    come as lists of micro-batch pieces (split along dim 0): the kernels read
+    every piece where it lies and write one gradient buffer per student piece,
+    so neither ``torch.cat`` of tspipe/gpu_task.py:188-191 is needed."""
+
+    @staticmethod
+    def forward(ctx, kind: str, n: int, tau: float, *pieces: Tensor):
+        import ctypes
+        o1, t2, o2, t1 = (pieces[i * n:(i + 1) * n] for i in range(4))  # pairs (o1, t2) and (o2, t1)
+        _require_cuda(*pieces)
+        first = o1[0]
+        c, dtype, dev = int(first.shape[1]), first.dtype, first.device
+        rows = []
+        for group in zip(o1, t2, o2, t1):
+            if any(t.dim() != 2 or t.shape != group[0].shape or t.dtype != dtype for t in group) or \
+                    int(group[0].shape[1]) != c:
+                raise ValueError("the pieces of all four operands must agree in shape and dtype, piece by piece")
+            rows.append(int(group[0].shape[0]))
+        total = sum(rows)
+        dense = [[t.detach() if t.is_contiguous() else t.detach().contiguous() for t in grp] for grp in (o1, t2, o2, t1)]
+        need1 = [ctx.needs_input_grad[3 + i] for i in range(n)]
+        need2 = [ctx.needs_input_grad[3 + 2 * n + i] for i in range(n)]
+        g1 = [torch.empty_like(t) for t in dense[0]] if any(need1) else None
+        g2 = [torch.empty_like(t) for t in dense[2]] if any(need2) else None
+        lib = _lib.lib()
+        code = _lib.dtype_code(dtype)
+        loss = torch.empty((), dtype=torch.float32, device=dev)
+        ptrs = lambda ts: None if ts is None else (ctypes.c_void_p * n)(*[t.data_ptr() for t in ts])  # noqa: E731
+        rows_arr = (ctypes.c_int64 * n)(*rows)
+        with torch.cuda.device(dev):
+            stream = _lib.current_stream_ptr(dev)
+            if kind == "infonce":
+                if c not in (64, 128, 256):
+                    raise ValueError(f"InfoNCE on pieces takes 64, 128 or 256 features, got {c} (gather and pad instead)")
+                if not tau >= 0.03:
+                    raise ValueError(f"InfoNCE kernels need a temperature of at least 0.03, got {tau}")
+                ws = torch.empty(lib.ts_infonce_workspace_bytes(total, c, 2), dtype=torch.uint8, device=dev)
+                status = lib.ts_infonce_pieces_fwd_bwd(ptrs(dense[0]), ptrs(dense[1]), ptrs(g1), ptrs(dense[2]),
+                                                       ptrs(dense[3]), ptrs(g2), rows_arr, n, c, tau, ws.data_ptr(),
+                                                       loss.data_ptr(), code, stream)
+                _lib.check(status, "ts_infonce_pieces_fwd_bwd")
+            else:
+                ws = torch.empty(2 * max(total, 1), dtype=torch.float32, device=dev)
+                status = lib.ts_byol_pieces_fwd_bwd(ptrs(dense[0]), ptrs(dense[1]), ptrs(g1), ptrs(dense[2]),
+                                                    ptrs(dense[3]), ptrs(g2), rows_arr, n, c, ws.data_ptr(),
+                                                    loss.data_ptr(), code, stream)
+                _lib.check(status, "ts_byol_pieces_fwd_bwd")
+        ctx.g1, ctx.g2, ctx.need1, ctx.need2, ctx.n = g1, g2, need1, need2, n
+        ctx.dims = [(r, c) for r in rows]
+        ctx.backward_done = False
+        return loss
+
+    @staticmethod
+    def backward(ctx, grad_output: Tensor):
+        _once(ctx)
+        n = ctx.n
+        g1, g2 = ctx.g1, ctx.g2
+        ctx.g1 = ctx.g2 = None
+        out1 = [None] * n if g1 is None else [
+            _scale_saved_grad(g, grad_output, *d) if need else None for g, need, d in zip(g1, ctx.need1, ctx.dims)]
+        out2 = [None] * n if g2 is None else [
+            _scale_saved_grad(g, grad_output, *d) if need else None for g, need, d in zip(g2, ctx.need2, ctx.dims)]
+        return (None, None, None) + tuple(out1) + (None,) * n + tuple(out2) + (None,) * n
+
+
+def _pair_pieces(kind: str, o1, o2, t1, t2, tau: float) -> Tensor:
+    o1, o2, t1, t2 = list(o1), list(o2), list(t1), list(t2)
+    n = len(o1)
+    if n == 0 or any(len(x) != n for x in (o2, t1, t2)):
+        raise ValueError("need the same number of pieces, at least one, for all four operands")
+    return _PairPiecesFn.apply(kind, n, float(tau), *o1, *t2, *o2, *t1)
+
+
+def moco_contrastive_loss_pieces(online_view_1, online_view_2, target_view_1, target_view_2, args,
+                                 extra_args) -> Tensor:
+    """``moco_contrastive_loss`` for a pipeline that hands over the lists of
+    micro-batch outputs instead of gathering them first (the ``torch.cat`` at
+    tspipe/gpu_task.py:188-191): each argument is a list of ``[rows_i, C]``
+    pieces, the same split for all four.  Same value as the loss on the
+    concatenated tensors; the gradient arrives per student piece."""
+    return _pair_pieces("infonce", online_view_1, online_view_2, target_view_1, target_view_2,
+                        float(extra_args.moco_t))
+
+
+def byol_contrastive_loss_pieces(online_view_1, online_view_2, target_view_1, target_view_2,
+                                 args: Namespace = None, extra_args: Namespace = None) -> Tensor:
+    """``byol_contrastive_loss`` on lists of micro-batch pieces, as above."""
+    return _pair_pieces("byol", online_view_1, online_view_2, target_view_1, target_view_2, 0.0)
+
+
+# ---------------------------------------------------------------------------
 # loss_fn plug-ins with the reference's signatures
 # ---------------------------------------------------------------------------
 
