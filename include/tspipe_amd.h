@@ -336,7 +336,9 @@ int ts_infonce_pieces_fwd_bwd(const void* const* q1_pieces, const void* const* k
  *     unless those are NULL;
  *   - turned into ub_mean = S/cnt and ub_invstd = 1/sqrt(max(Q/cnt - mean^2,0)
  *     + eps), cnt = N*HW, unless those are NULL.
- * ws: 2*C floats that are ZERO on entry; the call leaves them zero again. */
+ * One launch: the last workgroup of a channel to finish does the channel's
+ * bookkeeping.  ws: 3*C floats that are ZERO on entry (two sums and a ticket
+ * counter per channel); the call leaves them zero again. */
 int ts_bn_stats(const float* x, int64_t N, int64_t C, int64_t HW, float* ws, float* sum,
                 float* sum_squares, float* ub_mean, float* ub_invstd, float eps,
                 ts_stream_t stream);

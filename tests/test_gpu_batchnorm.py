@@ -23,8 +23,8 @@ def _check_workspace(bn):
     # one the NEXT call will reduce into is zero
     c = bn.num_features
     ws = bn._ws.cpu()
-    assert (ws[:2 * c] == 0).all()
-    nxt = 2 * c + bn._parity * 2 * c
+    assert (ws[:3 * c] == 0).all()
+    nxt = 3 * c + bn._parity * 2 * c
     assert (ws[nxt:nxt + 2 * c] == 0).all()
 
 def _rel(a, b):
@@ -220,7 +220,7 @@ def test_fused_training_forward_equals_the_two_calls(device):
     g = seeded(77)
     z = lambda n: torch.zeros(n, device=device)  # noqa: E731
     gamma, beta = torch.rand(C, generator=g).to(device) + 0.5, torch.randn(C, generator=g).to(device)
-    ws2, ws4 = z(2 * C), z(4 * C)
+    ws2, ws4 = z(3 * C), z(4 * C)
     sum_a, sq_a, sum_b, sq_b = z(C), z(C), z(C), z(C)
     for call in range(5):
         x = (torch.randn(N, C, H, W, generator=g) * 1.5 + 0.5).to(device)
@@ -278,3 +278,30 @@ def test_a_refused_call_leaves_the_next_forward_correct(device, monkeypatch):
     want = F.batch_norm(xs[0].double(), None, None, bn.weight.detach().cpu().double(), bn.bias.detach().cpu().double(),
                         True, 0.0, 1e-5)
     assert (y.cpu().double() - want).abs().max() < 2e-5
+
+
+def test_stand_alone_statistics_pass_is_one_launch_that_cleans_up(device):
+    # ts_bn_stats with several workgroups per channel: the last one to finish does the channel's
+    # bookkeeping and leaves the 3C-float workspace (sums and ticket counters) zero again
+    from tspipe_amd import _lib
+    lib = _lib.lib()
+    st = torch.cuda.current_stream(device).cuda_stream
+    N, C, H, W = 16, 24, 56, 56
+    g = seeded(91)
+    z = lambda n: torch.zeros(n, device=device)  # noqa: E731
+    ws, acc_s, acc_q, mean, inv = z(3 * C), z(C), z(C), z(C), z(C)
+    tot_s, tot_q = torch.zeros(C, dtype=torch.float64), torch.zeros(C, dtype=torch.float64)
+    for call in range(3):
+        x = torch.randn(N, C, H, W, generator=g) * 1.5 + 0.5
+        xd = x.to(device)
+        _lib.check(lib.ts_bn_stats(xd.data_ptr(), N, C, H * W, ws.data_ptr(), acc_s.data_ptr(), acc_q.data_ptr(),
+                                   mean.data_ptr(), inv.data_ptr(), 1e-5, st), "ts_bn_stats")
+        torch.cuda.synchronize()
+        assert (ws == 0).all()
+        x64 = x.double()
+        tot_s += x64.sum(dim=(0, 2, 3))
+        tot_q += (x64 ** 2).sum(dim=(0, 2, 3))
+        m64 = x64.mean(dim=(0, 2, 3))
+        v64 = x64.var(dim=(0, 2, 3), unbiased=False)
+        assert _rel(acc_s, tot_s) < 1e-6 and _rel(acc_q, tot_q) < 1e-6
+        assert _rel(mean, m64) < 1e-5 and _rel(inv, 1.0 / torch.sqrt(v64 + 1e-5)) < 1e-6

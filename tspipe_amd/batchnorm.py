@@ -87,7 +87,7 @@ class _NormalizeFn(torch.autograd.Function):
         with torch.cuda.device(x.device):
             status = _lib.lib().ts_bn_backward(x.data_ptr(), dy.data_ptr(), mean.data_ptr(), invstd.data_ptr(),
                                                _ptr(weight), dx.data_ptr(), dgamma.data_ptr(), dbeta.data_ptr(),
-                                               ws.data_ptr() + 8 * c, parity, n, c, hw, 1 if ctx.training else 0,
+                                               ws.data_ptr() + 12 * c, parity, n, c, hw, 1 if ctx.training else 0,
                                                _lib.current_stream_ptr(x.device))
         layer._after_launch(status, parity, "ts_bn_backward")
         return (dx, dgamma if weight is not None else None, dbeta if ctx.has_bias else None,
@@ -110,7 +110,7 @@ class _TrainForwardFn(torch.autograd.Function):
         with torch.cuda.device(x.device):
             status = _lib.lib().ts_bn_forward_train(
                 x.data_ptr(), y.data_ptr(), _ptr(weight), _ptr(bias), n, c, hw, layer.sum.data_ptr(),
-                layer.sum_squares.data_ptr(), mean.data_ptr(), invstd.data_ptr(), ws.data_ptr() + 8 * c, parity,
+                layer.sum_squares.data_ptr(), mean.data_ptr(), invstd.data_ptr(), ws.data_ptr() + 12 * c, parity,
                 float(layer.eps), _lib.current_stream_ptr(x.device))
         layer._after_launch(status, parity, "ts_bn_forward_train")
         ctx.save_for_backward(x, weight, mean, invstd)
@@ -137,11 +137,12 @@ class DeferredBatchNorm(_BatchNorm):
         super().__init__(num_features, eps, momentum, affine, track_running_stats=True)
         self.register_buffer("sum", torch.zeros_like(self.running_mean))
         self.register_buffer("sum_squares", torch.zeros_like(self.running_var))
-        # reduction workspace of the kernels, not part of the state dict: 2C
-        # floats that are zero between calls (stand-alone statistics) and two
-        # halves of 2C floats that the training forward and the backward
-        # alternate between (``_parity`` says which one the next call reduces into)
-        self.register_buffer("_ws", torch.zeros(6 * num_features), persistent=False)
+        # reduction workspace of the kernels, not part of the state dict: 3C
+        # floats that are zero between calls (stand-alone statistics: two sums
+        # and a ticket counter per channel) and two halves of 2C floats that
+        # the training forward and the backward alternate between
+        # (``_parity`` says which one the next call reduces into)
+        self.register_buffer("_ws", torch.zeros(7 * num_features), persistent=False)
         self._parity = 0
         self._ws_stream = None  # the stream whose kernels last used the workspace
         self.counter = 0
@@ -157,9 +158,9 @@ class DeferredBatchNorm(_BatchNorm):
         halves assume that the layer's calls run one after the other on the
         device, so a call on a stream other than the previous call's first
         waits for that stream."""
-        if self._ws.device != x.device or self._ws.numel() != 6 * self.num_features or self._ws.dtype != torch.float32:
+        if self._ws.device != x.device or self._ws.numel() != 7 * self.num_features or self._ws.dtype != torch.float32:
             # moved, resized, or cast along with the module (module.half()): start from zeros
-            self._ws = torch.zeros(6 * self.num_features, dtype=torch.float32, device=x.device)
+            self._ws = torch.zeros(7 * self.num_features, dtype=torch.float32, device=x.device)
             self._parity = 0
             self._ws_stream = None
         stream = torch.cuda.current_stream(x.device)
@@ -173,7 +174,7 @@ class DeferredBatchNorm(_BatchNorm):
         is known to have been enqueued.  A refused call may have run part of
         its launches, so the workspace starts again from zeros."""
         if status < 0:
-            self._ws = torch.zeros(6 * self.num_features, dtype=torch.float32, device=self._ws.device)
+            self._ws = torch.zeros(7 * self.num_features, dtype=torch.float32, device=self._ws.device)
             self._parity = 0
             _lib.check(status, what)
         self._parity = 1 - parity

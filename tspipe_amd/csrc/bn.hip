@@ -6,9 +6,10 @@
 // vectors over runs of HW floats.  gridDim = (slabs, C).
 //
 // Reductions are two-level: registers -> LDS tree inside the workgroup, then
-// one hardware fp32 atomic add per workgroup and quantity into a 2*C float
-// workspace.  The workspace is zero between calls: the small per-channel
-// kernel that consumes it also clears it.
+// one hardware fp32 atomic add per workgroup and quantity into a small float
+// workspace.  The workspace is zero between calls: whoever consumes it (the
+// last workgroup of a channel in the stand-alone statistics pass, the
+// normalising kernel in the fused passes) also clears it.
 //
 // Sums are taken about a per-channel shift k_c = x[0, c, 0] (the channel's
 // first value): S' = sum(x - k), Q' = sum((x - k)^2).  The variance
@@ -41,7 +42,7 @@ __device__ __forceinline__ PlaneSplit split_plane(const float* p, int64_t HW) {
 // Planes are taken two at a time so that the loads of both are in flight
 // before either is consumed (a plane of a small feature map is only a few
 // vectors per thread).
-template <bool TWO, typename F>
+template <bool TWO, int BLOCK = 256, typename F>
 __device__ __forceinline__ void slab_reduce(const float* __restrict__ x, const float* __restrict__ y,
                                             int64_t n0, int64_t n1, int64_t C, int64_t c, int64_t HW,
                                             float& a, float& b, F f) {
@@ -71,7 +72,7 @@ __device__ __forceinline__ void slab_reduce(const float* __restrict__ x, const f
         if (it < HW) f(px[p][it], TWO ? py[p][it] : 0.f, a, b);
       }
     }
-    for (int64_t base = 0; base < maxvec; base += kBnBlock * kBnUnroll) {
+    for (int64_t base = 0; base < maxvec; base += BLOCK * kBnUnroll) {
       f32x4 vx[PL][kBnUnroll], vy[PL][kBnUnroll];
 #pragma unroll
       for (int p = 0; p < PL; ++p) {
@@ -79,7 +80,7 @@ __device__ __forceinline__ void slab_reduce(const float* __restrict__ x, const f
         const f32x4* py4 = reinterpret_cast<const f32x4*>(py[p] + sp[p].head);
 #pragma unroll
         for (int u = 0; u < kBnUnroll; ++u) {
-          const int64_t i = base + u * kBnBlock + tid;
+          const int64_t i = base + u * BLOCK + tid;
           if (live[p] && i < sp[p].nvec) {
             vx[p][u] = px4[i];
             if (TWO) {
@@ -97,7 +98,7 @@ __device__ __forceinline__ void slab_reduce(const float* __restrict__ x, const f
       for (int p = 0; p < PL; ++p) {
 #pragma unroll
         for (int u = 0; u < kBnUnroll; ++u) {
-          const int64_t i = base + u * kBnBlock + tid;
+          const int64_t i = base + u * BLOCK + tid;
           if (live[p] && i < sp[p].nvec) {
             f(vx[p][u].x, TWO ? vy[p][u].x : 0.f, a, b);
             f(vx[p][u].y, TWO ? vy[p][u].y : 0.f, a, b);
@@ -110,9 +111,23 @@ __device__ __forceinline__ void slab_reduce(const float* __restrict__ x, const f
   }
 }
 
+// Statistics of one micro-batch in ONE launch: every workgroup adds its slab's
+// sums into the workspace with returning atomics, then takes a ticket from the
+// channel's counter; the workgroup that draws the last ticket knows that all
+// other additions have been performed (each was complete before its ticket
+// was drawn), collects the totals with atomic exchanges -- which also leave
+// the workspace zero for the next call -- and does the channel's bookkeeping.
+// Atomics act at the device's point of coherence, so no cache has to be
+// flushed or invalidated for this hand-off.
+//   ws: [0, C) sum(x - k), [C, 2C) sum((x - k)^2), [2C, 3C) tickets (as uint32)
+// FINAL = false is the first launch of the fused passes: sums only, the
+// launch that follows consumes them.
+template <bool FINAL>
 __global__ __launch_bounds__(kBnBlock) void bn_stats_kernel(const float* __restrict__ x, int64_t N,
-                                                            int64_t C, int64_t HW, int64_t slab,
-                                                            float* __restrict__ ws) {
+                                                            int64_t C, int64_t HW, int64_t slab, float cnt,
+                                                            float* __restrict__ ws, float* sum,
+                                                            float* sum_squares, float* ub_mean,
+                                                            float* ub_invstd, float eps) {
   __shared__ float lds[kBnBlock / kWave];
   const int64_t c = blockIdx.y;
   const int64_t n0 = (int64_t)blockIdx.x * slab;
@@ -126,29 +141,30 @@ __global__ __launch_bounds__(kBnBlock) void bn_stats_kernel(const float* __restr
   });
   S = block_sum<kBnBlock / kWave>(S, lds);
   Q = block_sum<kBnBlock / kWave>(Q, lds);
-  if (threadIdx.x == 0) {
-    unsafeAtomicAdd(ws + c, S);
-    unsafeAtomicAdd(ws + C + c, Q);
+  if (!FINAL) {
+    if (threadIdx.x == 0) {
+      unsafeAtomicAdd(ws + c, S);
+      unsafeAtomicAdd(ws + C + c, Q);
+    }
+    return;
   }
-}
-
-// One thread per channel: consumes and clears the workspace.
-__global__ __launch_bounds__(256) void bn_stats_finalize_kernel(const float* __restrict__ x, int64_t C,
-                                                                int64_t HW, float cnt,
-                                                                float* __restrict__ ws, float* sum,
-                                                                float* sum_squares, float* ub_mean,
-                                                                float* ub_invstd, float eps) {
-  const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (c >= C) return;
-  const float S = ws[c], Q = ws[C + c];
-  ws[c] = 0.f;
-  ws[C + c] = 0.f;
-  const float k = x[c * HW];
-  if (sum) sum[c] += S + cnt * k;
-  if (sum_squares) sum_squares[c] += Q + 2.f * k * S + cnt * k * k;
-  const float dm = S / cnt;  // mean - k
-  if (ub_mean) ub_mean[c] = k + dm;
-  if (ub_invstd) ub_invstd[c] = 1.f / sqrtf(fmaxf(Q / cnt - dm * dm, 0.f) + eps);
+  if (threadIdx.x == 0) {
+    unsigned* tickets = reinterpret_cast<unsigned*>(ws + 2 * C);
+    // the returned values are waited for: the additions are done before the ticket is drawn
+    const float r0 = atomicAdd(ws + c, S);
+    const float r1 = atomicAdd(ws + C + c, Q);
+    asm volatile("" ::"v"(r0), "v"(r1) : "memory");
+    const unsigned ticket = atomicAdd(tickets + c, 1u);
+    if (ticket == gridDim.x - 1) {
+      const float St = atomicExch(ws + c, 0.f), Qt = atomicExch(ws + C + c, 0.f);
+      atomicExch(tickets + c, 0u);
+      if (sum) sum[c] += St + cnt * k;
+      if (sum_squares) sum_squares[c] += Qt + 2.f * k * St + cnt * k * k;
+      const float dm = St / cnt;  // mean - k
+      if (ub_mean) ub_mean[c] = k + dm;
+      if (ub_invstd) ub_invstd[c] = 1.f / sqrtf(fmaxf(Qt / cnt - dm * dm, 0.f) + eps);
+    }
+  }
 }
 
 // The reference's rounding order, one fp32 operation at a time:
@@ -248,7 +264,7 @@ __global__ __launch_bounds__(kBnBlock) void bn_apply_kernel(const float* __restr
 // Training forward, second launch: normalises with the micro-batch statistics
 // that bn_stats_kernel left in `ws_in` (every workgroup derives mean and
 // 1/std of its channel from the two sums itself), and the first workgroup of
-// each channel does what bn_stats_finalize_kernel does -- running sums,
+// each channel does the channel's bookkeeping -- running sums,
 // saved statistics -- except that it clears the OTHER workspace half: this
 // one is still being read by the channel's other workgroups, the other one
 // was consumed by the previous call.
@@ -381,8 +397,11 @@ __global__ __launch_bounds__(kBnBlock) void bn_bwd_dx_kernel(const float* __rest
 
 // Samples per workgroup: about 8K elements each, so small feature maps do
 // not degenerate into one workgroup per few hundred bytes.
-inline int64_t bn_slab(int64_t N, int64_t HW) {
-  int64_t s = (8192 + HW - 1) / HW;
+// Samples per workgroup: about `target` elements.  The fused passes use 8192;
+// the stand-alone statistics pass, whose workgroups end with a few dependent
+// atomics, is a little faster with twice that (fewer, longer workgroups).
+inline int64_t bn_slab(int64_t N, int64_t HW, int64_t target = 8192) {
+  int64_t s = (target + HW - 1) / HW;
   s += s & 1;  // planes are consumed in pairs
   if (s < 1) s = 1;
   if (s > N) s = N;
@@ -408,15 +427,12 @@ int ts_bn_stats(const float* x, int64_t N, int64_t C, int64_t HW, float* ws, flo
   int rc = ts::bn_check_dims(N, C, HW);
   if (rc) return rc;
   if ((uintptr_t)x & 3u) return TS_ERR_ALIGN;
-  const int64_t slab = ts::bn_slab(N, HW);
-  dim3 grid((unsigned)((N + slab - 1) / slab), (unsigned)C);
   hipStream_t st = (hipStream_t)stream;
-  hipLaunchKernelGGL(ts::bn_stats_kernel, grid, dim3(ts::kBnBlock), 0, st, x, N, C, HW, slab, ws);
-  rc = ts::check_launch();
-  if (rc) return rc;
-  hipLaunchKernelGGL(ts::bn_stats_finalize_kernel, dim3((unsigned)((C + 255) / 256)), dim3(256), 0, st,
-                     x, C, HW, (float)((double)N * (double)HW), ws, sum, sum_squares, ub_mean, ub_invstd,
-                     eps);
+  const float cnt = (float)((double)N * (double)HW);
+  const int64_t slab = ts::bn_slab(N, HW, 16384);
+  dim3 grid((unsigned)((N + slab - 1) / slab), (unsigned)C);
+  hipLaunchKernelGGL(ts::bn_stats_kernel<true>, grid, dim3(ts::kBnBlock), 0, st, x, N, C, HW, slab,
+                     (float)((double)N * (double)HW), ws, sum, sum_squares, ub_mean, ub_invstd, eps);
   return ts::check_launch();
 }
 
@@ -467,7 +483,8 @@ int ts_bn_forward_train(const float* x, float* y, const float* gamma, const floa
   hipStream_t st = (hipStream_t)stream;
   float* ws_now = ws + (int64_t)parity * 2 * C;
   float* ws_other = ws + (int64_t)(1 - parity) * 2 * C;
-  hipLaunchKernelGGL(ts::bn_stats_kernel, grid, dim3(ts::kBnBlock), 0, st, x, N, C, HW, slab, ws_now);
+  hipLaunchKernelGGL(ts::bn_stats_kernel<false>, grid, dim3(ts::kBnBlock), 0, st, x, N, C, HW, slab, 0.f, ws_now,
+                     (float*)nullptr, (float*)nullptr, (float*)nullptr, (float*)nullptr, 0.f);
   rc = ts::check_launch();
   if (rc) return rc;
   hipLaunchKernelGGL(ts::bn_apply_train_kernel, grid, dim3(ts::kBnBlock), 0, st, x, y, gamma, beta, N, C, HW, slab,

@@ -434,10 +434,6 @@ __global__ __launch_bounds__(kNceBlock, 2) void nce_main_kernel(NceArgs args, in
     // P = 2^(S * rq_i * log2e/tau - x_max), rounded to bf16; keys this lane
     // holds: key(i) = (i%4) + 4h + 8(i/4).  The row sum is taken over the
     // rounded values (v_dot2 of the packed pairs with ones).
-    // The soft-max is the part of a stage in which this wavefront has no MFMA
-    // to issue; with issue priority it gets through while the other
-    // workgroup's wavefront on this SIMD keeps the matrix pipe busy.
-    __builtin_amdgcn_s_setprio(2);
     float pv[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) pv[i] = fast_exp2(fmaf(sacc[i], sc_i, -scale2));
@@ -469,7 +465,6 @@ __global__ __launch_bounds__(kNceBlock, 2) void nce_main_kernel(NceArgs args, in
     bf16x8 tr[RING];
 #pragma unroll
     for (int i = 0; i < RING; ++i) tr[i] = read_t(i);
-    __builtin_amdgcn_s_setprio(0);
     // barrier without waiting for the global -> LDS fetches of the next stage
     __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the P written above is in LDS
     __builtin_amdgcn_s_barrier();
