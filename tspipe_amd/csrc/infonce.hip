@@ -19,20 +19,22 @@
 //
 // Kernels:
 //   prep     per row: rq = 1/max(|q|,eps), rk, and the normalised key row
-//            rounded to bf16 (row-major, zero rows up to a multiple of 64).
-//   main     grid (q tile of 64 rows, key split); 4 wavefronts = 2 pairs, a
-//            pair owning 32 q rows.  Keys come in stages of 64 (two tiles of
-//            32), global memory -> LDS without passing through registers,
-//            double-buffered.  Per stage, wavefront a of a pair computes
-//            S^T = Kh Q^T (MFMA 32x32x16) for tile a over all features,
-//            P = 2^(S*scale - x_max) rounded to bf16, hands P to its partner
-//            through LDS, and accumulates O^T += Kh^T P for ITS HALF of the
-//            features over both tiles.  So a wavefront keeps 64 accumulator
-//            registers for O and 64 for its Q fragments, fits in 256
-//            registers, and two workgroups share a CU: one's soft-max runs
-//            under the other's MFMAs.  Kh^T operands are read from the same
-//            row-major LDS tile as the Kh operands, with the transposing LDS
-//            read of gfx950 (ds_read_b64_tr_b16).
+//            rounded to bf16 (row-major, zero rows up to a multiple of 128).
+//   main     grid (q tile of 128 rows, key split); 8 wavefronts = 4 pairs, a
+//            pair owning 32 q rows, two wavefronts on every SIMD.  Keys come
+//            in stages of 64 (two tiles of 32), global memory -> LDS without
+//            passing through registers, three buffers.  Per stage, wavefront
+//            a of a pair computes S^T = Kh Q^T (MFMA 32x32x16) for tile a over
+//            all features, P = 2^(S*scale - x_max) rounded to bf16, hands P to
+//            its partner through LDS, and accumulates O^T += Kh^T P for ITS
+//            HALF of the features over both tiles.  So a wavefront keeps 64
+//            accumulator registers for O and 64 for its Q fragments and fits
+//            in 256 registers.  The loop is software-pipelined with one
+//            barrier per stage: the second product runs a stage behind the
+//            first, and the exponentials of stage st are issued between the
+//            MFMAs of the second product of stage st-1.  Kh^T operands are
+//            read from the same row-major LDS tile as the Kh operands, with
+//            the transposing LDS read of gfx950 (ds_read_b64_tr_b16).
 //   combine  per 32 q rows: adds the key splits, forms dq; its first
 //            workgroup adds up the loss from the split row sums.
 //
@@ -65,9 +67,10 @@ typedef short s16x4 __attribute__((ext_vector_type(4)));
 constexpr float kNceLog2e = 1.4426950408889634f;
 constexpr float kNceLn2 = 0.6931471805599453f;
 constexpr float kNormEps = 1e-12f;  // F.normalize's eps
-constexpr int kQTile = 64;          // q rows per workgroup (32 per wavefront pair)
+constexpr int kQTile = 128;         // q rows per workgroup of the main kernel (32 per wavefront pair)
 constexpr int kStageKeys = 64;      // keys per LDS stage (two tiles of 32)
-constexpr int kNceBlock = 256;
+constexpr int kNceBlock = 256;      // prep kernel
+constexpr int kNceMainBlock = 512;  // main kernel: 8 wavefronts, two per SIMD
 constexpr int kNceMaxPieces = 8;
 
 // defined in losses.hip
@@ -143,13 +146,13 @@ __device__ __forceinline__ NceRow nce_row(const NcePair& pr, int64_t row, int C)
 
 inline size_t nce_align(size_t x) { return (x + 255) & ~(size_t)255; }
 
-// Key splits: enough workgroups for two per CU (a workgroup is 4 wavefronts
-// of at most 256 registers and 72 KB of LDS, so two share a CU and overlap
-// each other's matrix and vector phases).
+// Key splits: enough workgroups for one per CU (a workgroup is 4 wavefronts,
+// one per SIMD, each with its own software pipeline; its three stage buffers
+// take most of a CU's LDS).
 inline int nce_splits(int64_t npad, int n_pairs) {
   const int64_t qtiles = npad / kQTile * n_pairs;
   const int64_t stages = npad / kStageKeys;
-  int64_t s = (512 + qtiles - 1) / qtiles;
+  int64_t s = (256 + qtiles - 1) / qtiles;
   if (s > 16) s = 16;
   if (s > stages) s = stages;
   if (s < 1) s = 1;
@@ -271,23 +274,26 @@ __device__ __forceinline__ int nce_swz(int row) {
 // anyway) instead of fp32, which halves the traffic between this kernel and
 // the combine.
 template <int C, bool HP>
-__global__ __launch_bounds__(kNceBlock, 2) void nce_main_kernel(NceArgs args, int64_t n, int64_t npad, int splits,
-                                                                float scale2 /* log2(e)/tau */, int qtile_major) {
+__global__ __launch_bounds__(kNceMainBlock) void nce_main_kernel(NceArgs args, int64_t n, int64_t npad, int splits,
+                                                                 float scale2 /* log2(e)/tau */, int qtile_major) {
   const NcePair& pr = args.p[blockIdx.z];
   constexpr int KK = C / 16;          // contraction steps of S^T
   constexpr int FBH = C / 64;         // 32-feature blocks of O^T per wavefront (half of the features)
   constexpr int CPR = C / 8;          // 16-byte chunks per key row
   constexpr int ROWB = C * 2;         // bytes per key row
   constexpr int STAGE = kStageKeys * ROWB;
-  constexpr int NU = STAGE / (4 * 1024);  // 1 KB fetches per wavefront and stage
-  constexpr int KL = KK < 8 ? KK : 8;     // first-product chunk addresses kept in registers
-  // two separate arrays, so that the compiler can tell that a fetch into one
-  // does not touch what is being read from the other (it would otherwise wait
-  // for every outstanding fetch in front of every LDS read)
-  __shared__ __attribute__((aligned(1024))) uint8_t sm0[STAGE];
-  __shared__ __attribute__((aligned(1024))) uint8_t sm1[STAGE];
-  __shared__ __attribute__((aligned(1024))) uint8_t xch[2][2][2][1024];  // [pair][tile][step][lane * 16]
-  const int tid = threadIdx.x, lane = tid % kWave, w = tid / kWave;
+  constexpr int NW = kNceMainBlock / kWave;
+  constexpr int NU = STAGE / (NW * 1024);  // 1 KB fetches per wavefront and stage
+  constexpr int KL = KK < 8 ? KK : 8;      // first-product chunk addresses kept in registers
+  // Three stage buffers, stage st in buffer (st - s0) % 3: the one of the
+  // first product, the one of the second product (a stage behind) and the one
+  // being fetched.
+  __shared__ __attribute__((aligned(1024))) uint8_t sm[3 * STAGE];
+  // exchanged P, double-buffered by stage parity: [parity][pair][tile][step][lane * 16]
+  __shared__ __attribute__((aligned(1024))) uint8_t xch[2][NW / 2][2][2][1024];
+  constexpr int XPAR = (NW / 2) * 4096;  // bytes per parity
+  const int tid = threadIdx.x, lane = tid % kWave;
+  const int w = __builtin_amdgcn_readfirstlane(tid / kWave);
   const int col = lane % 32, h = lane / 32;
   const int p = w >> 1, a = w & 1;
   // Workgroup ids are dealt round-robin to the 8 XCDs.  While all keys fit an
@@ -298,8 +304,8 @@ __global__ __launch_bounds__(kNceBlock, 2) void nce_main_kernel(NceArgs args, in
   const int64_t qtile = qtile_major ? blockIdx.x : blockIdx.y;
   const int64_t qrow = qtile * kQTile + p * 32 + col;  // the q row this lane is a column of
 
-  const int64_t stages = npad / kStageKeys;
-  const int64_t s0 = stages * split / splits, s1 = stages * (split + 1) / splits;
+  const int stages = (int)(npad / kStageKeys);
+  const int s0 = (int)((int64_t)stages * split / splits), s1 = (int)((int64_t)stages * (split + 1) / splits);
 
   // Global -> LDS without passing through registers: lane L's 16 bytes land
   // at (LDS base) + 16 L, so the swizzle is applied on the global side: the
@@ -311,18 +317,27 @@ __global__ __launch_bounds__(kNceBlock, 2) void nce_main_kernel(NceArgs args, in
     const int row = slot / CPR, cs = slot % CPR;
     goff[u] = (uint32_t)(row * ROWB + ((cs ^ nce_swz<CPR>(row)) << 4));
   }
-  const uint8_t* __restrict__ khat = reinterpret_cast<const uint8_t*>(pr.khat);
-  // one 1 KB piece of a stage (piece u of this wavefront's NU)
-  auto fetch_piece = [&](int64_t st, int buf, int u) {
-    const uint8_t* src = khat + st * STAGE;
-    uint8_t* dst = (buf ? sm1 : sm0) + (w * NU + u) * 1024;
-    __builtin_amdgcn_global_load_lds((nce_glb_void*)(src + goff[u]), (nce_lds_void*)dst, 16, 0, 0);
+  // one 1 KB piece of a stage (piece u of this wavefront's NU) into the buffer at byte offset `base`
+  auto fetch_piece = [&](int st, int base, int u) {
+    // Issued as assembly on purpose.  The compiler books an LDS-DMA load on
+    // both memory counters and, while one is in flight, turns every wait for an
+    // LDS read into a wait for ALL of them, which would undo the read-ahead of
+    // the operand rings below.  Completion of these fetches is awaited
+    // explicitly (vmcnt(0) in front of the stage barrier).  M0 carries the LDS
+    // destination; nothing else in this kernel uses it.
+#if defined(__HIP_DEVICE_COMPILE__)
+    const uint8_t* src = reinterpret_cast<const uint8_t*>(pr.khat) + (int64_t)st * STAGE + goff[u];
+    const uint32_t lds = (uint32_t)(uintptr_t)(nce_lds_void*)sm + (uint32_t)(base + (w * NU + u) * 1024);
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                 :
+                 : "v"(src), "s"(__builtin_amdgcn_readfirstlane(lds))
+                 : "memory");
+#endif
   };
-  auto fetch_stage = [&](int64_t st, int buf) {
+  if (s0 < s1) {
 #pragma unroll
-    for (int u = 0; u < NU; ++u) fetch_piece(st, buf, u);
-  };
-  if (s0 < s1) fetch_stage(s0, 0);
+    for (int u = 0; u < NU; ++u) fetch_piece(s0, 0, u);
+  }
 
   // Q fragments: B operand of S^T, resident for the whole kernel.
   const uint16_t* qg;
@@ -343,7 +358,7 @@ __global__ __launch_bounds__(kNceBlock, 2) void nce_main_kernel(NceArgs args, in
 
   // LDS byte offsets of this lane's operand reads within a stage (the parts
   // that depend on a compile-time index only through an addition are left to
-  // the instruction's immediate offset).
+  // the instruction's immediate offset; the buffer's base is added per stage).
   // first product, A operand: key row 32a + col, chunk 2kk + h
   uint32_t ak[KL];
   {
@@ -381,42 +396,88 @@ __global__ __launch_bounds__(kNceBlock, 2) void nce_main_kernel(NceArgs args, in
   const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
   // the lane of column col that holds key `col` of a diagonal tile: D register i*, half h*
   const int hstar = (col >> 2) & 1, istar = (col & 3) + 4 * (col >> 3);
+  // the pair's own keys are tile p of the q tile's four: stage 2 qtile + p/2, its tile p%2
+  const int diag_stage = (int)(2 * qtile) + (p >> 1);
+  const bool diag_wave = a == (p & 1);
 
+  // Software pipeline, one barrier per stage.  In stage st a wavefront issues
+  //   16 MFMAs of S^T(st)                     (+ the fetches of stage st+1),
+  //   16 MFMAs of O^T += Kh^T(st-1) P(st-1)   with the soft-max of S^T(st)
+  //                                           between them on the vector unit,
+  // then writes P(st) for its partner and meets the others at the barrier.  A
+  // SIMD holds two wavefronts of the workgroup, so the vector work of one runs
+  // under the MFMAs of the other.
+  //
   // Operand fragments are read from LDS four MFMAs ahead of their use, into a
-  // ring of four registers sets; the order below is pinned with scheduling
-  // barriers, because left to itself the compiler reads every fragment right
-  // in front of its MFMA and the LDS latency is paid sixteen times per phase.
+  // ring of four registers sets; the order is pinned with scheduling barriers,
+  // because left to itself the compiler reads every fragment right in front of
+  // its MFMA and the LDS latency is paid sixteen times per phase.
   constexpr int RING = 4;
-  constexpr int NSTEP = 4 * FBH;  // MFMAs of the second product per stage
-  auto one_stage = [&](int64_t st, auto buf_tag) {
-    constexpr int BUF = decltype(buf_tag)::value;
-    const uint8_t* stage = BUF ? sm1 : sm0;
-    auto read_k = [&](int kk) {
-      const u32x4 raw = *reinterpret_cast<const u32x4*>(stage + ak[kk % KL] + (kk / KL) * (KL * 32));
-      bf16x8 v;
-      __builtin_memcpy(&v, &raw, 16);
-      return v;
-    };
-    // step s of the second product: key step T = s / FBH (16 keys), feature block s % FBH
+  constexpr int NSTEP = 4 * FBH;      // MFMAs of the second product per stage (== KK)
+  constexpr int EPS = 16 / NSTEP;     // soft-max elements handled between two of them
+  static_assert(NSTEP == KK && EPS >= 1, "feature width");
+  const uint32_t xlane = (uint32_t)(p * 4096 + lane * 16);
+  uint8_t* const xch0 = &xch[0][0][0][0][0];
+  // O^T[f][q] += sum_key Kh^T[f][key] P[key][q] over both tiles of the stage in
+  // the buffer at `base`, for this wavefront's half of the features;
+  // contraction slot 8h + 4r + j of step T is key 16T + 8r + 4h + j on both
+  // operands.  `between(step)` runs after the MFMA of each step.
+  auto second_product = [&](int base, int parity, auto&& between) {
+    uint32_t atc[FBH][2];
+#pragma unroll
+    for (int fbl = 0; fbl < FBH; ++fbl) {
+      atc[fbl][0] = at[fbl][0] + (uint32_t)base;
+      atc[fbl][1] = at[fbl][1] + (uint32_t)base;
+    }
     auto read_t = [&](int step) {
+      // step s: key step T = s / FBH (16 keys), feature block s % FBH
       const int T = step / FBH, fbl = step % FBH;
-      const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((nce_lds_s16x4*)(stage + at[fbl][0] + T * 16 * ROWB));
-      const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((nce_lds_s16x4*)(stage + at[fbl][1] + T * 16 * ROWB));
+      const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((nce_lds_s16x4*)(sm + atc[fbl][0] + T * 16 * ROWB));
+      const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((nce_lds_s16x4*)(sm + atc[fbl][1] + T * 16 * ROWB));
       bf16x8 v;
       __builtin_memcpy(&v, &lo, 8);
       __builtin_memcpy(reinterpret_cast<char*>(&v) + 8, &hi, 8);
       return v;
     };
-    // After this barrier stage st is complete in LDS (its fetches were issued
-    // a whole stage ago) and every wavefront has finished reading stage st-1,
-    // whose buffer the fetches below overwrite, and the exchanged P of st-1.
-    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wavefront's fetches have landed
-    __syncthreads();
+    bf16x8 pbT[4];
+#pragma unroll
+    for (int T = 0; T < 4; ++T) {
+      const u32x4 praw = *reinterpret_cast<const u32x4*>(xch0 + parity * XPAR + xlane + T * 1024);
+      __builtin_memcpy(&pbT[T], &praw, 16);
+    }
+    bf16x8 tr[RING];
+#pragma unroll
+    for (int i = 0; i < RING; ++i) tr[i] = read_t(i);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int step = 0; step < NSTEP; ++step) {
+      oacc[step % FBH] =
+          __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr[step % RING], pbT[step / FBH], oacc[step % FBH], 0, 0, 0);
+      if (step + RING < NSTEP) tr[step % RING] = read_t(step + RING);
+      between(step);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+  // cur / prev / nxt: byte offsets of the buffers of stages st, st-1, st+1
+  auto one_stage = [&](int st, int cur, int prev, int nxt, auto first_tag) {
+    constexpr bool FIRST = decltype(first_tag)::value;
+    uint32_t akc[KL];
+#pragma unroll
+    for (int kl = 0; kl < KL; ++kl) akc[kl] = ak[kl] + (uint32_t)cur;
+    auto read_k = [&](int kk) {
+      const u32x4 raw = *reinterpret_cast<const u32x4*>(sm + akc[kk % KL] + (kk / KL) * (KL * 32));
+      bf16x8 v;
+      __builtin_memcpy(&v, &raw, 16);
+      return v;
+    };
     // near the end the fetch repeats the last stage into the idle buffer (no branch)
-    const int64_t st_next = st + 1 < s1 ? st + 1 : s1 - 1;
+    const int st_next = st + 1 < s1 ? st + 1 : s1 - 1;
 
     // S^T[key][q] = sum_f Kh[key][f] Q[q][f] for tile a of the stage; the
-    // next stage's fetches are issued between the MFMAs
+    // next stage's fetches are issued between the MFMAs, into the buffer that
+    // held stage st-2 (every wavefront finished with it before the barrier
+    // that ended stage st-1)
     f32x16 sacc;
 #pragma unroll
     for (int i = 0; i < 16; ++i) sacc[i] = 0.f;
@@ -428,109 +489,103 @@ __global__ __launch_bounds__(kNceBlock, 2) void nce_main_kernel(NceArgs args, in
     for (int kk = 0; kk < KK; ++kk) {
       sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kr[kk % RING], qf[kk], sacc, 0, 0, 0);
       if (kk + RING < KK) kr[kk % RING] = read_k(kk + RING);
-      if (kk < NU) fetch_piece(st_next, BUF ^ 1, kk);
+      if (kk < NU) fetch_piece(st_next, nxt, kk);
       __builtin_amdgcn_sched_barrier(0);
     }
     // P = 2^(S * rq_i * log2e/tau - x_max), rounded to bf16; keys this lane
     // holds: key(i) = (i%4) + 4h + 8(i/4).  The row sum is taken over the
     // rounded values (v_dot2 of the packed pairs with ones).
     float pv[16];
-#pragma unroll
-    for (int i = 0; i < 16; ++i) pv[i] = fast_exp2(fmaf(sacc[i], sc_i, -scale2));
+    float pe = 0.f;
     bf16x8 pb[2];
+    auto softmax_slice = [&](int step) {
 #pragma unroll
-    for (int i = 0; i < 16; i += 2) {
-      const bf16x2 pk = {(__bf16)pv[i], (__bf16)pv[i + 1]};
-      lsum = __builtin_amdgcn_fdot2_f32_bf16(pk, ones, lsum, false);
-      pb[i / 8][i % 8] = pk[0];
-      pb[i / 8][i % 8 + 1] = pk[1];
-    }
-    if (st == qtile && a == p) {  // the tile that holds this pair's own keys (uniform per wavefront)
-      float pe = pv[0];
-#pragma unroll
-      for (int i = 1; i < 16; ++i) pe = (i == istar) ? pv[i] : pe;
-      if (h == hstar) {
-        pd_exact = pe;
-        pd_round = (float)(__bf16)pe;
+      for (int e = 0; e < EPS; ++e) {
+        const int i = step * EPS + e;
+        pv[i] = fast_exp2(fmaf(sacc[i], sc_i, -scale2));
+        pe = (i == istar) ? pv[i] : pe;
+        if (i & 1) {
+          const bf16x2 pk = {(__bf16)pv[i - 1], (__bf16)pv[i]};
+          lsum = __builtin_amdgcn_fdot2_f32_bf16(pk, ones, lsum, false);
+          pb[i / 8][(i - 1) % 8] = pk[0];
+          pb[i / 8][i % 8] = pk[1];
+        }
       }
+    };
+    if (FIRST) {
+#pragma unroll
+      for (int step = 0; step < NSTEP; ++step) softmax_slice(step);
+    } else {
+      second_product(prev, (st - 1) & 1, softmax_slice);
     }
-    // hand this tile's P to the partner (and to the second product below)
+    if (st == diag_stage && diag_wave && h == hstar) {  // the tile that holds this pair's own keys
+      pd_exact = pe;
+      pd_round = (float)(__bf16)pe;
+    }
+    // hand this tile's P to the partner (and to this wavefront's own second product)
 #pragma unroll
     for (int t2 = 0; t2 < 2; ++t2) {
       u32x4 raw;
       __builtin_memcpy(&raw, &pb[t2], 16);
-      *reinterpret_cast<u32x4*>(&xch[p][a][t2][lane * 16]) = raw;
+      *reinterpret_cast<u32x4*>(xch0 + (st & 1) * XPAR + xlane + a * 2048 + t2 * 1024) = raw;
     }
-    // the first Kh^T fragments do not depend on the exchange: on their way during the barrier
-    bf16x8 tr[RING];
-#pragma unroll
-    for (int i = 0; i < RING; ++i) tr[i] = read_t(i);
-    // barrier without waiting for the global -> LDS fetches of the next stage
-    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the P written above is in LDS
+    // After this barrier: P(st) is visible, stage st+1 is complete in LDS (every
+    // wavefront waited for its own pieces) and everybody has finished reading
+    // stage st-1 and P(st-1).
+    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) and lgkmcnt(0)
     __builtin_amdgcn_s_barrier();
-    // O^T[f][q] += sum_key Kh^T[f][key] P[key][q] over both tiles, for this
-    // wavefront's half of the features; contraction slot 8h + 4r + j of step
-    // T is key 16T + 8r + 4h + j on both operands.
-    bf16x8 pbT[4];
-#pragma unroll
-    for (int T = 0; T < 4; ++T) {
-      const u32x4 praw = *reinterpret_cast<const u32x4*>(&xch[p][T >> 1][T & 1][lane * 16]);
-      __builtin_memcpy(&pbT[T], &praw, 16);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int step = 0; step < NSTEP; ++step) {
-      oacc[step % FBH] =
-          __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr[step % RING], pbT[step / FBH], oacc[step % FBH], 0, 0, 0);
-      if (step + RING < NSTEP) tr[step % RING] = read_t(step + RING);
-      __builtin_amdgcn_sched_barrier(0);
-    }
   };
 
-  // two stages per trip, so that the buffer index is a compile-time constant
-  for (int64_t st = s0; st < s1; st += 2) {
-    one_stage(st, std::integral_constant<int, 0>{});
-    if (st + 1 < s1) one_stage(st + 1, std::integral_constant<int, 1>{});
+  if (s0 < s1) {
+    __builtin_amdgcn_s_waitcnt(0x0070);  // stage s0 has landed
+    __builtin_amdgcn_s_barrier();
+    int cur = 0, prev = 2 * STAGE, nxt = STAGE;
+    one_stage(s0, cur, prev, nxt, std::true_type{});
+    for (int st = s0 + 1; st < s1; ++st) {
+      const int t = prev;
+      prev = cur;
+      cur = nxt;
+      nxt = t;
+      one_stage(st, cur, prev, nxt, std::false_type{});
+    }
+    // the second product of the last stage
+    second_product(cur, (s1 - 1) & 1, [](int) {});
   }
-
-  // The last trip fetched a stage nobody reads; it must have landed before
-  // this workgroup's LDS can be handed to another one.
-  __builtin_amdgcn_s_waitcnt(0x0f70);
 
   // Padded keys (zero rows of Kh) took part in the row sums with the same
   // term for every row, the rounded 2^(0 - x_max); take this lane's share out.
   {
     int cnt = 0;
-    const int64_t st_pad = n / kStageKeys;
-    for (int64_t st = (s0 > st_pad ? s0 : st_pad); st < s1; ++st)
+    const int st_pad = (int)(n / kStageKeys);
+    for (int st = (s0 > st_pad ? s0 : st_pad); st < s1; ++st)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) cnt += (st * kStageKeys + 32 * a + 4 * h + 8 * (i / 4) + (i % 4) >= n) ? 1 : 0;
+      for (int i = 0; i < 16; ++i) cnt += ((int64_t)st * kStageKeys + 32 * a + 4 * h + 8 * (i / 4) + (i % 4) >= n) ? 1 : 0;
     const float c0 = (float)(__bf16)fast_exp2(fmaf(0.f, sc_i, -scale2));
     lsum -= (float)cnt * c0;
   }
 
   // row sums: the two halves of a lane pair, then the two wavefronts of the pair (through LDS);
   // the same exchange hands P~_ii to every lane of the q row's column
-  const bool has_diag = qtile >= s0 && qtile < s1;  // this split met the pair's own keys (uniform)
+  const bool has_diag = diag_stage >= s0 && diag_stage < s1;  // this split met the pair's own keys (uniform)
   float ltot = lsum + __shfl_xor(lsum, 32, kWave);
   __syncthreads();  // everybody is done with xch
-  float* lx = reinterpret_cast<float*>(&xch[0][0][0][0]);
+  float* lx = reinterpret_cast<float*>(&xch[0][0][0][0][0]);
   if (a == 1 && h == 0) lx[p * 32 + col] = ltot;
-  if (has_diag && a == p && h == hstar) lx[64 + p * 32 + col] = pd_round;
+  if (has_diag && diag_wave && h == hstar) lx[kQTile + p * 32 + col] = pd_round;
   __syncthreads();
   if (a == 0 && h == 0) {
     ltot += lx[p * 32 + col];
     pr.lpart[(int64_t)split * npad + qrow] = ltot;
   }
   if (has_diag) {
-    if (a == p && h == hstar) {
+    if (diag_wave && h == hstar) {
       const f32x2 v = {pd_exact, pd_round};
       *reinterpret_cast<f32x2*>(pr.pdiag + 2 * qrow) = v;
     }
     // The positive key's own term P~_ii kh~_i leaves the sum here, where it is
     // known to the last bit; the combine puts (1 - P~_ii / l~) kh_i in fp32 in
     // its place.  What is stored is the negatives' sum, which may be rounded.
-    const float prr = lx[64 + p * 32 + col];
+    const float prr = lx[kQTile + p * 32 + col];
     const uint16_t* krow = pr.khat + qrow * C + a * (C / 2) + 4 * h;
 #pragma unroll
     for (int fb = 0; fb < FBH; ++fb)
@@ -751,7 +806,7 @@ int nce_run(const NceArgs& args, int pairs, int64_t n, float tau, const NceLayou
                                      : dim3((unsigned)L.splits, (unsigned)(L.npad / kQTile), z);
   // fp32 inputs keep fp32 partial sums; the 2-byte types, whose gradient is rounded to 2^-9 anyway, bf16 ones
   constexpr bool HP = sizeof(T) == 2;
-  hipLaunchKernelGGL((nce_main_kernel<C, HP>), main_grid, dim3(kNceBlock), 0, stream, args, n, L.npad, L.splits, scale2,
+  hipLaunchKernelGGL((nce_main_kernel<C, HP>), main_grid, dim3(kNceMainBlock), 0, stream, args, n, L.npad, L.splits, scale2,
                      qtile_major ? 1 : 0);
   rc = check_launch();
   if (rc) return rc;
