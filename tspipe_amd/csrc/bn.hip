@@ -432,7 +432,7 @@ int ts_bn_stats(const float* x, int64_t N, int64_t C, int64_t HW, float* ws, flo
   const int64_t slab = ts::bn_slab(N, HW, 16384);
   dim3 grid((unsigned)((N + slab - 1) / slab), (unsigned)C);
   hipLaunchKernelGGL(ts::bn_stats_kernel<true>, grid, dim3(ts::kBnBlock), 0, st, x, N, C, HW, slab,
-                     (float)((double)N * (double)HW), ws, sum, sum_squares, ub_mean, ub_invstd, eps);
+                     cnt, ws, sum, sum_squares, ub_mean, ub_invstd, eps);
   return ts::check_launch();
 }
 

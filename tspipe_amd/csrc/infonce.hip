@@ -307,6 +307,19 @@ __global__ __launch_bounds__(kNceMainBlock) void nce_main_kernel(NceArgs args, i
   const int stages = (int)(npad / kStageKeys);
   const int s0 = (int)((int64_t)stages * split / splits), s1 = (int)((int64_t)stages * (split + 1) / splits);
 
+  // Every field of the pair that the prologue needs, requested in one go: one
+  // scalar-load latency instead of one per use.
+  const uint16_t* const khat_p = pr.khat;
+  const uint16_t* const qb = pr.qb;
+  const void* const q_single = pr.q;
+  const float* const rq_p = pr.rq;
+  const int n_pieces = pr.n_pieces;
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("" : : "s"(khat_p), "s"(qb), "s"(q_single), "s"(rq_p), "s"(n_pieces));
+#else
+  (void)khat_p, (void)qb, (void)q_single, (void)n_pieces;
+#endif
+
   // Global -> LDS without passing through registers: lane L's 16 bytes land
   // at (LDS base) + 16 L, so the swizzle is applied on the global side: the
   // lane that fills slot (row, c') loads chunk c' ^ swz(row) of that row.
@@ -326,7 +339,7 @@ __global__ __launch_bounds__(kNceMainBlock) void nce_main_kernel(NceArgs args, i
     // explicitly (vmcnt(0) in front of the stage barrier).  M0 carries the LDS
     // destination; nothing else in this kernel uses it.
 #if defined(__HIP_DEVICE_COMPILE__)
-    const uint8_t* src = reinterpret_cast<const uint8_t*>(pr.khat) + (int64_t)st * STAGE + goff[u];
+    const uint8_t* src = reinterpret_cast<const uint8_t*>(khat_p) + (int64_t)st * STAGE + goff[u];
     const uint32_t lds = (uint32_t)(uintptr_t)(nce_lds_void*)sm + (uint32_t)(base + (w * NU + u) * 1024);
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
                  :
@@ -339,22 +352,61 @@ __global__ __launch_bounds__(kNceMainBlock) void nce_main_kernel(NceArgs args, i
     for (int u = 0; u < NU; ++u) fetch_piece(s0, 0, u);
   }
 
-  // Q fragments: B operand of S^T, resident for the whole kernel.
-  const uint16_t* qg;
-  if (pr.qb) {
-    qg = pr.qb + qrow * C;
-  } else {
-    qg = (const uint16_t*)nce_row<bf16_t>(pr, qrow < n ? qrow : 0, C).q;
-  }
-  bf16x8 qf[KK];
-#pragma unroll
-  for (int kk = 0; kk < KK; ++kk) {
-    u32x4 raw = {0u, 0u, 0u, 0u};
-    if (qrow < n) raw = *reinterpret_cast<const u32x4*>(qg + kk * 16 + h * 8);
-    __builtin_memcpy(&qf[kk], &raw, 16);
-  }
-  const float rq_i = (qrow < n) ? pr.rq[qrow] : 0.f;
+  const float rq_i = (qrow < n) ? rq_p[qrow] : 0.f;  // on its way while the tiles are fetched
   const float sc_i = rq_i * scale2;
+
+  // Q fragments: B operand of S^T, resident for the whole kernel.  The q tile
+  // (kQTile rows, exactly two stage buffers) comes in through LDS with the
+  // same swizzled, coalesced fetch as the keys; read straight from global
+  // memory, a fragment load would touch 64 different cache lines.
+  // Rows beyond the batch fetch the last row instead; their fragments are
+  // zeroed below.  One decision up front (a single matrix, or row blocks), so
+  // that the pair's fields are read once and the eight fetches go out back to
+  // back.
+#if defined(__HIP_DEVICE_COMPILE__)
+  {
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(nce_lds_void*)sm + (uint32_t)(STAGE + w * 2 * NU * 1024);
+    auto fetch_q = [&](auto&& row_ptr, uint32_t lds_base) {
+      const uint8_t* qsrc[2 * NU];
+#pragma unroll
+      for (int u = 0; u < 2 * NU; ++u) {
+        const int slot = (w * 2 * NU + u) * kWave + lane;
+        const int row = slot / CPR, cs = slot % CPR;
+        int64_t grow = qtile * kQTile + row;
+        grow = grow < n ? grow : n - 1;
+        qsrc[u] = reinterpret_cast<const uint8_t*>(row_ptr(grow)) + ((cs ^ nce_swz<CPR>(row)) << 4);
+      }
+#pragma unroll
+      for (int u = 0; u < 2 * NU; ++u) {
+        asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                     :
+                     : "v"(qsrc[u]), "s"(__builtin_amdgcn_readfirstlane(lds_base + u * 1024))
+                     : "memory");
+      }
+    };
+    if (qb != nullptr || n_pieces == 0) {
+      const uint16_t* base = qb ? qb : (const uint16_t*)q_single;
+      fetch_q([&](int64_t grow) { return base + grow * C; }, lds0);
+    } else {
+      fetch_q([&](int64_t grow) { return (const uint16_t*)nce_row<bf16_t>(pr, grow, C).q; }, lds0);
+    }
+  }
+#endif
+  __builtin_amdgcn_s_waitcnt(0x0070);
+  __builtin_amdgcn_s_barrier();  // the q tile and stage s0 are in LDS
+  bf16x8 qf[KK];
+  {
+    const int row = p * 32 + col;
+    const int sw = nce_swz<CPR>(row);
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      u32x4 raw = *reinterpret_cast<const u32x4*>(sm + STAGE + row * ROWB + (((2 * kk + h) ^ sw) << 4));
+      if (qrow >= n) raw = u32x4{0u, 0u, 0u, 0u};  // rows beyond the batch were not fetched
+      __builtin_memcpy(&qf[kk], &raw, 16);
+    }
+  }
+  __builtin_amdgcn_s_waitcnt(0xc07f);  // the fragments have left LDS ...
+  __builtin_amdgcn_s_barrier();        // ... in every wavefront: the two buffers may be fetched into
 
   // LDS byte offsets of this lane's operand reads within a stage (the parts
   // that depend on a compile-time index only through an addition are left to
@@ -401,70 +453,72 @@ __global__ __launch_bounds__(kNceMainBlock) void nce_main_kernel(NceArgs args, i
   const bool diag_wave = a == (p & 1);
 
   // Software pipeline, one barrier per stage.  In stage st a wavefront issues
+  //   the last MFMAs of O^T(st-2), whose operands it kept in registers,
   //   16 MFMAs of S^T(st)                     (+ the fetches of stage st+1),
-  //   16 MFMAs of O^T += Kh^T(st-1) P(st-1)   with the soft-max of S^T(st)
-  //                                           between them on the vector unit,
+  //   the first MFMAs of O^T += Kh^T(st-1) P(st-1), with the soft-max of
+  //   S^T(st) between them on the vector unit,
   // then writes P(st) for its partner and meets the others at the barrier.  A
   // SIMD holds two wavefronts of the workgroup, so the vector work of one runs
   // under the MFMAs of the other.
   //
   // Operand fragments are read from LDS four MFMAs ahead of their use, into a
-  // ring of four registers sets; the order is pinned with scheduling barriers,
-  // because left to itself the compiler reads every fragment right in front of
-  // its MFMA and the LDS latency is paid sixteen times per phase.
+  // ring of four register sets, and the read-ahead runs across the phases: the
+  // first operands of the second product are requested during the last steps
+  // of the first, and the MFMAs held back over the barrier cover the latency
+  // of the first reads of the next stage.  The order is pinned with scheduling
+  // barriers, because left to itself the compiler reads every fragment right
+  // in front of its MFMA and the LDS latency is paid at every step.
   constexpr int RING = 4;
-  constexpr int NSTEP = 4 * FBH;      // MFMAs of the second product per stage (== KK)
-  constexpr int EPS = 16 / NSTEP;     // soft-max elements handled between two of them
-  static_assert(NSTEP == KK && EPS >= 1, "feature width");
+  constexpr int NSTEP = 4 * FBH;                 // MFMAs of the second product per stage (== KK)
+  constexpr int TAIL = NSTEP >= 8 ? RING : 0;    // of which held back over the barrier
+  constexpr int BODY = NSTEP - TAIL;             // the others carry the soft-max
+  static_assert(NSTEP == KK && BODY >= 1 && BODY <= 16, "feature width");
   const uint32_t xlane = (uint32_t)(p * 4096 + lane * 16);
   uint8_t* const xch0 = &xch[0][0][0][0][0];
-  // O^T[f][q] += sum_key Kh^T[f][key] P[key][q] over both tiles of the stage in
-  // the buffer at `base`, for this wavefront's half of the features;
-  // contraction slot 8h + 4r + j of step T is key 16T + 8r + 4h + j on both
-  // operands.  `between(step)` runs after the MFMA of each step.
-  auto second_product = [&](int base, int parity, auto&& between) {
-    uint32_t atc[FBH][2];
+  // Second product: O^T[f][q] += sum_key Kh^T[f][key] P[key][q] over both tiles
+  // of a stage, for this wavefront's half of the features; contraction slot
+  // 8h + 4r + j of step T is key 16T + 8r + 4h + j on both operands.
+  // step s: key step T = s / FBH (16 keys), feature block s % FBH.
+  auto read_t = [&](const uint32_t (&atc)[FBH][2], int step) {
+    const int T = step / FBH, fbl = step % FBH;
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((nce_lds_s16x4*)(sm + atc[fbl][0] + T * 16 * ROWB));
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((nce_lds_s16x4*)(sm + atc[fbl][1] + T * 16 * ROWB));
+    bf16x8 v;
+    __builtin_memcpy(&v, &lo, 8);
+    __builtin_memcpy(reinterpret_cast<char*>(&v) + 8, &hi, 8);
+    return v;
+  };
+  auto read_p = [&](int parity, int T) {
+    const u32x4 praw = *reinterpret_cast<const u32x4*>(xch0 + parity * XPAR + xlane + T * 1024);
+    bf16x8 v;
+    __builtin_memcpy(&v, &praw, 16);
+    return v;
+  };
+  // operands of the held-back steps BODY .. NSTEP-1 of the previous stage's second product
+  bf16x8 trH[RING], pbH[4];
+  auto tail_steps = [&]() {
 #pragma unroll
-    for (int fbl = 0; fbl < FBH; ++fbl) {
-      atc[fbl][0] = at[fbl][0] + (uint32_t)base;
-      atc[fbl][1] = at[fbl][1] + (uint32_t)base;
-    }
-    auto read_t = [&](int step) {
-      // step s: key step T = s / FBH (16 keys), feature block s % FBH
-      const int T = step / FBH, fbl = step % FBH;
-      const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((nce_lds_s16x4*)(sm + atc[fbl][0] + T * 16 * ROWB));
-      const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((nce_lds_s16x4*)(sm + atc[fbl][1] + T * 16 * ROWB));
-      bf16x8 v;
-      __builtin_memcpy(&v, &lo, 8);
-      __builtin_memcpy(reinterpret_cast<char*>(&v) + 8, &hi, 8);
-      return v;
-    };
-    bf16x8 pbT[4];
-#pragma unroll
-    for (int T = 0; T < 4; ++T) {
-      const u32x4 praw = *reinterpret_cast<const u32x4*>(xch0 + parity * XPAR + xlane + T * 1024);
-      __builtin_memcpy(&pbT[T], &praw, 16);
-    }
-    bf16x8 tr[RING];
-#pragma unroll
-    for (int i = 0; i < RING; ++i) tr[i] = read_t(i);
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int step = 0; step < NSTEP; ++step) {
-      oacc[step % FBH] =
-          __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr[step % RING], pbT[step / FBH], oacc[step % FBH], 0, 0, 0);
-      if (step + RING < NSTEP) tr[step % RING] = read_t(step + RING);
-      between(step);
+    for (int j = 0; j < TAIL; ++j) {
+      const int step = BODY + j;
+      oacc[step % FBH] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(trH[j], pbH[step / FBH], oacc[step % FBH], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
 
-  // cur / prev / nxt: byte offsets of the buffers of stages st, st-1, st+1
-  auto one_stage = [&](int st, int cur, int prev, int nxt, auto first_tag) {
-    constexpr bool FIRST = decltype(first_tag)::value;
+  // MODE 0: the split's first stage (no second product yet), 1: its second
+  // stage (nothing held back yet), 2: any later stage.
+  // cur / prev / nxt: byte offsets of the buffers of stages st, st-1, st+1.
+  auto one_stage = [&](int st, int cur, int prev, int nxt, auto mode_tag) {
+    constexpr int MODE = decltype(mode_tag)::value;
     uint32_t akc[KL];
 #pragma unroll
     for (int kl = 0; kl < KL; ++kl) akc[kl] = ak[kl] + (uint32_t)cur;
+    uint32_t atc[FBH][2];
+#pragma unroll
+    for (int fbl = 0; fbl < FBH; ++fbl) {
+      atc[fbl][0] = at[fbl][0] + (uint32_t)prev;
+      atc[fbl][1] = at[fbl][1] + (uint32_t)prev;
+    }
     auto read_k = [&](int kk) {
       const u32x4 raw = *reinterpret_cast<const u32x4*>(sm + akc[kk % KL] + (kk / KL) * (KL * 32));
       bf16x8 v;
@@ -473,6 +527,13 @@ __global__ __launch_bounds__(kNceMainBlock) void nce_main_kernel(NceArgs args, i
     };
     // near the end the fetch repeats the last stage into the idle buffer (no branch)
     const int st_next = st + 1 < s1 ? st + 1 : s1 - 1;
+    const int par_prev = (st - 1) & 1;
+
+    bf16x8 kr[RING];
+#pragma unroll
+    for (int i = 0; i < RING; ++i) kr[i] = read_k(i);
+    __builtin_amdgcn_sched_barrier(0);
+    if (MODE == 2) tail_steps();
 
     // S^T[key][q] = sum_f Kh[key][f] Q[q][f] for tile a of the stage; the
     // next stage's fetches are issued between the MFMAs, into the buffer that
@@ -481,14 +542,19 @@ __global__ __launch_bounds__(kNceMainBlock) void nce_main_kernel(NceArgs args, i
     f32x16 sacc;
 #pragma unroll
     for (int i = 0; i < 16; ++i) sacc[i] = 0.f;
-    bf16x8 kr[RING];
-#pragma unroll
-    for (int i = 0; i < RING; ++i) kr[i] = read_k(i);
-    __builtin_amdgcn_sched_barrier(0);
+    bf16x8 pbT[4], tr[RING];
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) {
       sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kr[kk % RING], qf[kk], sacc, 0, 0, 0);
       if (kk + RING < KK) kr[kk % RING] = read_k(kk + RING);
+      if (MODE >= 1 && kk >= KK - RING) {  // first operands of the second product
+        const int j = kk - (KK - RING);
+        if (j < 2) {
+          pbT[2 * j] = read_p(par_prev, 2 * j);
+          pbT[2 * j + 1] = read_p(par_prev, 2 * j + 1);
+        }
+        tr[j] = read_t(atc, j);
+      }
       if (kk < NU) fetch_piece(st_next, nxt, kk);
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -498,10 +564,9 @@ __global__ __launch_bounds__(kNceMainBlock) void nce_main_kernel(NceArgs args, i
     float pv[16];
     float pe = 0.f;
     bf16x8 pb[2];
-    auto softmax_slice = [&](int step) {
+    auto softmax_elems = [&](int i0, int i1) {
 #pragma unroll
-      for (int e = 0; e < EPS; ++e) {
-        const int i = step * EPS + e;
+      for (int i = i0; i < i1; ++i) {
         pv[i] = fast_exp2(fmaf(sacc[i], sc_i, -scale2));
         pe = (i == istar) ? pv[i] : pe;
         if (i & 1) {
@@ -512,11 +577,21 @@ __global__ __launch_bounds__(kNceMainBlock) void nce_main_kernel(NceArgs args, i
         }
       }
     };
-    if (FIRST) {
-#pragma unroll
-      for (int step = 0; step < NSTEP; ++step) softmax_slice(step);
+    if (MODE == 0) {
+      softmax_elems(0, 16);
     } else {
-      second_product(prev, (st - 1) & 1, softmax_slice);
+#pragma unroll
+      for (int step = 0; step < BODY; ++step) {
+        oacc[step % FBH] =
+            __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr[step % RING], pbT[step / FBH], oacc[step % FBH], 0, 0, 0);
+        if (step + RING < NSTEP) tr[step % RING] = read_t(atc, step + RING);
+        softmax_elems(16 * step / BODY, 16 * (step + 1) / BODY);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+#pragma unroll
+      for (int j = 0; j < TAIL; ++j) trH[j] = tr[(BODY + j) % RING];
+#pragma unroll
+      for (int T = 0; T < 4; ++T) pbH[T] = pbT[T];
     }
     if (st == diag_stage && diag_wave && h == hstar) {  // the tile that holds this pair's own keys
       pd_exact = pe;
@@ -537,19 +612,47 @@ __global__ __launch_bounds__(kNceMainBlock) void nce_main_kernel(NceArgs args, i
   };
 
   if (s0 < s1) {
-    __builtin_amdgcn_s_waitcnt(0x0070);  // stage s0 has landed
-    __builtin_amdgcn_s_barrier();
     int cur = 0, prev = 2 * STAGE, nxt = STAGE;
-    one_stage(s0, cur, prev, nxt, std::true_type{});
-    for (int st = s0 + 1; st < s1; ++st) {
+    auto rotate = [&]() {
       const int t = prev;
       prev = cur;
       cur = nxt;
       nxt = t;
-      one_stage(st, cur, prev, nxt, std::false_type{});
+    };
+    one_stage(s0, cur, prev, nxt, std::integral_constant<int, 0>{});
+    if (s0 + 1 < s1) {
+      rotate();
+      one_stage(s0 + 1, cur, prev, nxt, std::integral_constant<int, 1>{});
+      for (int st = s0 + 2; st < s1; ++st) {
+        rotate();
+        one_stage(st, cur, prev, nxt, std::integral_constant<int, 2>{});
+      }
     }
-    // the second product of the last stage
-    second_product(cur, (s1 - 1) & 1, [](int) {});
+    // the second product of the last stage, its first reads ahead of the
+    // held-back steps of the one before
+    {
+      uint32_t atc[FBH][2];
+#pragma unroll
+      for (int fbl = 0; fbl < FBH; ++fbl) {
+        atc[fbl][0] = at[fbl][0] + (uint32_t)cur;
+        atc[fbl][1] = at[fbl][1] + (uint32_t)cur;
+      }
+      const int parity = (s1 - 1) & 1;
+      bf16x8 pbT[4], tr[RING];
+#pragma unroll
+      for (int T = 0; T < 4; ++T) pbT[T] = read_p(parity, T);
+#pragma unroll
+      for (int i = 0; i < RING; ++i) tr[i] = read_t(atc, i);
+      __builtin_amdgcn_sched_barrier(0);
+      if (s0 + 1 < s1) tail_steps();
+#pragma unroll
+      for (int step = 0; step < NSTEP; ++step) {
+        oacc[step % FBH] =
+            __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr[step % RING], pbT[step / FBH], oacc[step % FBH], 0, 0, 0);
+        if (step + RING < NSTEP) tr[step % RING] = read_t(atc, step + RING);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
   }
 
   // Padded keys (zero rows of Kh) took part in the row sums with the same
