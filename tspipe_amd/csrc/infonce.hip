@@ -35,13 +35,14 @@
 //            MFMAs of the second product of stage st-1.  Kh^T operands are
 //            read from the same row-major LDS tile as the Kh operands, with
 //            the transposing LDS read of gfx950 (ds_read_b64_tr_b16).
-//   combine  per 32 q rows: adds the key splits, forms dq; its first
+//   combine  per 16 q rows: adds the key splits, forms dq; one more
 //            workgroup adds up the loss from the split row sums.
 //
 // Accuracy: the row sum l is taken over the bf16-rounded P that the second
-// product uses, so O / l is an exact convex combination of the rounded keys,
-// and the positive key's own term is taken out of O again (by the main kernel,
-// which knows P_ii as it rounded it) and replaced by the fp32 kh_i.  The
+// product uses, so O / l is an exact convex combination of the rounded keys.
+// The positive key's own term never enters O (the main kernel feeds P_ii to
+// the second product as zero, while the row sum keeps it as it was rounded);
+// the combine adds it with the fp32 kh_i.  The
 // projection <qh, dqh> is formed from dqh itself.  The gradient then carries
 // the bf16 rounding of the NEGATIVE keys only, weighted by their
 // probabilities, also when P_ii -> 1.
@@ -593,9 +594,17 @@ __global__ __launch_bounds__(kNceMainBlock) void nce_main_kernel(NceArgs args, i
 #pragma unroll
       for (int T = 0; T < 4; ++T) pbH[T] = pbT[T];
     }
-    if (st == diag_stage && diag_wave && h == hstar) {  // the tile that holds this pair's own keys
-      pd_exact = pe;
-      pd_round = (float)(__bf16)pe;
+    if (st == diag_stage && diag_wave) {  // the tile that holds this pair's own keys (uniform)
+      // The positive key's own term leaves the second product here: P~_ii stays
+      // in the row sum above but goes to the MFMA as zero, so O^T is the
+      // negatives' sum and the combine adds (1 - P~_ii / l~) kh_i in fp32.
+      if (h == hstar) {
+        pd_exact = pe;
+        pd_round = (float)(__bf16)pe;
+      }
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+        if (i == istar && h == hstar) pb[i / 8][i % 8] = (__bf16)0.0f;
     }
     // hand this tile's P to the partner (and to this wavefront's own second product)
 #pragma unroll
@@ -667,38 +676,20 @@ __global__ __launch_bounds__(kNceMainBlock) void nce_main_kernel(NceArgs args, i
     lsum -= (float)cnt * c0;
   }
 
-  // row sums: the two halves of a lane pair, then the two wavefronts of the pair (through LDS);
-  // the same exchange hands P~_ii to every lane of the q row's column
+  // row sums: the two halves of a lane pair, then the two wavefronts of the pair (through LDS)
   const bool has_diag = diag_stage >= s0 && diag_stage < s1;  // this split met the pair's own keys (uniform)
   float ltot = lsum + __shfl_xor(lsum, 32, kWave);
   __syncthreads();  // everybody is done with xch
   float* lx = reinterpret_cast<float*>(&xch[0][0][0][0][0]);
   if (a == 1 && h == 0) lx[p * 32 + col] = ltot;
-  if (has_diag && diag_wave && h == hstar) lx[kQTile + p * 32 + col] = pd_round;
   __syncthreads();
   if (a == 0 && h == 0) {
     ltot += lx[p * 32 + col];
     pr.lpart[(int64_t)split * npad + qrow] = ltot;
   }
-  if (has_diag) {
-    if (diag_wave && h == hstar) {
-      const f32x2 v = {pd_exact, pd_round};
-      *reinterpret_cast<f32x2*>(pr.pdiag + 2 * qrow) = v;
-    }
-    // The positive key's own term P~_ii kh~_i leaves the sum here, where it is
-    // known to the last bit; the combine puts (1 - P~_ii / l~) kh_i in fp32 in
-    // its place.  What is stored is the negatives' sum, which may be rounded.
-    const float prr = lx[kQTile + p * 32 + col];
-    const uint16_t* krow = pr.khat + qrow * C + a * (C / 2) + 4 * h;
-#pragma unroll
-    for (int fb = 0; fb < FBH; ++fb)
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        uint16_t kb4[4];
-        __builtin_memcpy(kb4, krow + 32 * fb + 8 * g, 8);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) oacc[fb][4 * g + j] = fmaf(-prr, bf16_bits_to_f32(kb4[j]), oacc[fb][4 * g + j]);
-      }
+  if (has_diag && diag_wave && h == hstar) {
+    const f32x2 v = {pd_exact, pd_round};
+    *reinterpret_cast<f32x2*>(pr.pdiag + 2 * qrow) = v;
   }
   // partial O^T in register-native order, [split][tile of 32 q rows][feature half a][fb] and then
   //   fp32: [i/4][lane][i%4]      (16 bytes per lane and store)
@@ -731,11 +722,11 @@ __global__ __launch_bounds__(kNceMainBlock) void nce_main_kernel(NceArgs args, i
 }
 
 // ---------------------------------------------------------------------------
-// combine: one workgroup per 32 q rows, two wavefronts per 32-feature block.
-// Lane (col = row, h) of wavefront (fb, g2) holds features
+// combine: one workgroup per 16 q rows, one wavefront per 32-feature block.
+// Lane (row = lane % 16, h, g2) of wavefront fb holds features
 // 32 fb + 8 g + 4 h + j for g = 2 g2, 2 g2 + 1 and j = 0..3, the order the
 // partial O^T was stored in.  With O'_i the negatives' sum (the main kernel
-// took the positive key's term out):
+// kept the positive key's term out):
 //   dqh_i = (2/N) [ O'_i / l~_i  -  (1 - P~_ii / l~_i) kh_i ]
 // (~: rounded to bf16 as the MFMA saw it; kh_i: fp32), then the projection
 // with <qh_i, dqh_i>, summed over the row through LDS.
@@ -792,24 +783,39 @@ __device__ __forceinline__ void nce_loss_block(const NceArgs& args, int pairs, i
 }
 
 template <typename T, int C, bool HP>
-__global__ __launch_bounds__(4 * C) void nce_combine_kernel(NceArgs args, int64_t n, int64_t npad, int splits,
-                                                            float loss_scale, float* __restrict__ loss_out) {
-  constexpr int NW = C / 16;  // wavefronts: two per 32-feature block
+__global__ __launch_bounds__(2 * C) void nce_combine_kernel(NceArgs args, int64_t n, int64_t npad, int splits,
+                                                            float loss_scale, float* __restrict__ loss_out,
+                                                            int xcd_map) {
+  constexpr int NW = C / 32;  // wavefronts: one per 32-feature block
   constexpr int FBH = C / 64;
-  // workgroup 0 of the first pair computes the loss; the 32-row tiles start at workgroup 1
-  if (blockIdx.x == 0) {
-    if (blockIdx.z == 0) nce_loss_block<4 * C>(args, (int)gridDim.z, n, npad, splits, loss_scale, loss_out);
+  // The grid is the 16-row units, then 8 more workgroups of which the first
+  // computes the loss (for the first pair only) and the others have nothing to do.
+  const int64_t units = npad / 16;
+  if (blockIdx.x >= units) {
+    if (blockIdx.x == units && blockIdx.z == 0)
+      nce_loss_block<2 * C>(args, (int)gridDim.z, n, npad, splits, loss_scale, loss_out);
     return;
   }
+  // Workgroup ids are dealt round-robin to the 8 XCDs and the grid's width is
+  // a multiple of 8.  With xcd_map, the main kernel ran all key splits of q
+  // tile t on XCD t % 8; a unit is taken by a workgroup of that XCD, which
+  // finds the partial sums in its own L2.
+  int64_t unit = blockIdx.x;
+  if (xcd_map) {
+    const int64_t x = blockIdx.x % 8, j = blockIdx.x / 8;
+    constexpr int UPT = kQTile / 16;  // units per q tile
+    unit = (x + 8 * (j / UPT)) * UPT + j % UPT;
+  }
   const NcePair& pr = args.p[blockIdx.z];
-  __shared__ float dots[NW][32];
-  const int lane = threadIdx.x % kWave, wv = threadIdx.x / kWave;
-  const int fb = wv >> 1, g2 = wv & 1;
-  const int col = lane % 32, h = lane / 32;
-  const int64_t tile32 = (int64_t)blockIdx.x - 1;
-  const int64_t row = tile32 * 32 + col;
+  __shared__ float dots[NW][16];
+  const int lane = threadIdx.x % kWave, fb = threadIdx.x / kWave;
+  const int col16 = lane & 15, h = (lane >> 4) & 1, g2 = lane >> 5;
+  const int64_t tile32 = unit >> 1;
+  const int half = (int)(unit & 1);
+  const int64_t row = unit * 16 + col16;
   const bool live = row < n;
   const int a = fb / FBH, fbl = fb % FBH;
+  const int slot = h * 32 + half * 16 + col16;  // the main kernel's lane that held this row and feature group
 
   // Bound by memory latency, not arithmetic: every load is issued before the
   // first use of any of them (up to 8 splits; more come in further rounds).
@@ -841,11 +847,11 @@ __global__ __launch_bounds__(4 * C) void nce_combine_kernel(NceArgs args, int64_
       lv[u] = pr.lpart[(int64_t)sp * npad + row];
       const int64_t b = (int64_t)sp * split_blocks + blk;
       if (HP) {
-        vh[u] = reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(pr.opart) + b * 16 * kWave)[g2 * kWave + lane];
+        vh[u] = reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(pr.opart) + b * 16 * kWave)[g2 * kWave + slot];
       } else {
         const f32x4* src = reinterpret_cast<const f32x4*>(pr.opart + b * 16 * kWave);
-        vf[u][0] = src[(2 * g2) * kWave + lane];
-        vf[u][1] = src[(2 * g2 + 1) * kWave + lane];
+        vf[u][0] = src[(2 * g2) * kWave + slot];
+        vf[u][1] = src[(2 * g2 + 1) * kWave + slot];
       }
     }
 #pragma unroll
@@ -874,13 +880,14 @@ __global__ __launch_bounds__(4 * C) void nce_combine_kernel(NceArgs args, int64_
     qh[e] = to_f32(qv[e / 4][e % 4]) * rq_i;
     dot = fmaf(qh[e], dqh[e], dot);
   }
+  dot += __shfl_xor(dot, 16, kWave);
   dot += __shfl_xor(dot, 32, kWave);
-  if (h == 0) dots[wv][col] = dot;
+  if (lane < 16) dots[fb][col16] = dot;
   __syncthreads();
   if (!live || !rp.dq) return;
   float total = 0.f;
 #pragma unroll
-  for (int x = 0; x < NW; ++x) total += dots[x][col];
+  for (int x = 0; x < NW; ++x) total += dots[x][col16];
   // below eps the norm is the constant eps and normalize() is linear: no projection
   if (rq_i >= 1.f / kNormEps) total = 0.f;
 #pragma unroll
@@ -913,8 +920,9 @@ int nce_run(const NceArgs& args, int pairs, int64_t n, float tau, const NceLayou
                      qtile_major ? 1 : 0);
   rc = check_launch();
   if (rc) return rc;
-  hipLaunchKernelGGL((nce_combine_kernel<T, C, HP>), dim3((unsigned)(L.npad / 32 + 1), 1, z), dim3(4 * C), 0, stream,
-                     args, n, L.npad, L.splits, 2.f * tau, loss_out);
+  const int xcd_map = qtile_major && (L.npad / kQTile) % 8 == 0 ? 1 : 0;
+  hipLaunchKernelGGL((nce_combine_kernel<T, C, HP>), dim3((unsigned)(L.npad / 16 + 8), 1, z), dim3(2 * C), 0, stream,
+                     args, n, L.npad, L.splits, 2.f * tau, loss_out, xcd_map);
   return check_launch();
 }
 
