@@ -293,6 +293,7 @@ __global__ __launch_bounds__(kNceMainBlock) void nce_main_kernel(NceArgs args, i
   // exchanged P, double-buffered by stage parity: [parity][pair][tile][step][lane * 16]
   __shared__ __attribute__((aligned(1024))) uint8_t xch[2][NW / 2][2][2][1024];
   constexpr int XPAR = (NW / 2) * 4096;  // bytes per parity
+  __shared__ __attribute__((aligned(256))) uint8_t dump[NW * 256];  // written by the L2 prefetch, never read
   const int tid = threadIdx.x, lane = tid % kWave;
   const int w = __builtin_amdgcn_readfirstlane(tid / kWave);
   const int col = lane % 32, h = lane / 32;
@@ -348,9 +349,32 @@ __global__ __launch_bounds__(kNceMainBlock) void nce_main_kernel(NceArgs args, i
                  : "memory");
 #endif
   };
+  // The stage after the next is requested into this XCD's L2 (one word per
+  // 128-byte line of this wavefront's share), so that the LDS fetch a stage
+  // later finds it there: a fetch that has to go to memory does not always
+  // land within one stage, and at the barrier every wavefront waits for the
+  // slowest fetch of the eight.  The words go to an LDS area nobody reads: a
+  // load into a register would write that register whenever it returns, long
+  // after the compiler has given it to something else.  Issued after the
+  // stage's fetches, so that vmcnt(1) awaits those and not this.
+  auto l2_prefetch = [&](int st) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    if (lane < 8 * NU) {
+      const uint8_t* src = reinterpret_cast<const uint8_t*>(khat_p) + (int64_t)st * STAGE + (w * NU * 8 + lane) * 128;
+      const uint32_t lds = (uint32_t)(uintptr_t)(nce_lds_void*)dump + (uint32_t)(w * 256);
+      asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off"
+                   :
+                   : "v"(src), "s"(__builtin_amdgcn_readfirstlane(lds))
+                   : "memory");
+    }
+#else
+    (void)st, (void)dump;
+#endif
+  };
   if (s0 < s1) {
 #pragma unroll
     for (int u = 0; u < NU; ++u) fetch_piece(s0, 0, u);
+    l2_prefetch(s0 + 1 < s1 ? s0 + 1 : s1 - 1);
   }
 
   const float rq_i = (qrow < n) ? rq_p[qrow] : 0.f;  // on its way while the tiles are fetched
@@ -557,6 +581,7 @@ __global__ __launch_bounds__(kNceMainBlock) void nce_main_kernel(NceArgs args, i
         tr[j] = read_t(atc, j);
       }
       if (kk < NU) fetch_piece(st_next, nxt, kk);
+      if (kk == NU) l2_prefetch(st + 2 < s1 ? st + 2 : s1 - 1);
       __builtin_amdgcn_sched_barrier(0);
     }
     // P = 2^(S * rq_i * log2e/tau - x_max), rounded to bf16; keys this lane
@@ -616,7 +641,7 @@ __global__ __launch_bounds__(kNceMainBlock) void nce_main_kernel(NceArgs args, i
     // After this barrier: P(st) is visible, stage st+1 is complete in LDS (every
     // wavefront waited for its own pieces) and everybody has finished reading
     // stage st-1 and P(st-1).
-    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) and lgkmcnt(0)
+    __builtin_amdgcn_s_waitcnt(0x0071);  // vmcnt(1): all but the L2 prefetch, which came last; lgkmcnt(0)
     __builtin_amdgcn_s_barrier();
   };
 
@@ -663,6 +688,10 @@ __global__ __launch_bounds__(kNceMainBlock) void nce_main_kernel(NceArgs args, i
       }
     }
   }
+
+  // The last L2 prefetch writes into this workgroup's LDS; it must have landed
+  // before the LDS can be handed to another workgroup.
+  __builtin_amdgcn_s_waitcnt(0x0f70);
 
   // Padded keys (zero rows of Kh) took part in the row sums with the same
   // term for every row, the rounded 2^(0 - x_max); take this lane's share out.
