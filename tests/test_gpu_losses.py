@@ -288,6 +288,24 @@ def test_infonce_bf16(device, n, c):
     assert (err <= 1e-3 * peak + gw.abs() * 2.0 ** -8).all() or peak < 1e-9
 
 
+def test_infonce_more_keys_than_an_l2_holds(device):
+    # above 8192 rows the launcher makes the key split the fastest grid index; 8330 is not a
+    # multiple of the 128-row q tile or the 64-key stage, so padded rows and keys are in play
+    n, c = 8330, 256
+    q, k = _nce_inputs(n, c, 17, torch.bfloat16)
+    want, (gw,) = _oracle_grad(lambda a, b: ts_oracle.infonce(a, b, 0.2), q, others=(k,))
+    qd = q.to(device).requires_grad_()
+    loss = ta.infonce_loss(qd, k.to(device), 0.2)
+    loss.backward()
+    assert rel_err(loss.item(), want) < 1e-3
+    peak = gw.abs().max().item()
+    err = (qd.grad.cpu().double() - gw).abs()
+    assert (err <= 1e-3 * peak + gw.abs() * 2.0 ** -8).all()
+    # the gradient is orthogonal to its row (normalize Jacobian), a size-independent identity
+    dots = (qd.grad.float() * qd.detach().float()).sum(dim=1).abs().max().item()
+    assert dots < 2e-2 * peak
+
+
 def test_infonce_unnormalised_inputs_and_pair(device):
     g = seeded(31)
     o1, o2, t1, t2 = [(torch.randn(512, 256, generator=g) * (0.5 + i)).to(torch.bfloat16) for i in range(4)]
