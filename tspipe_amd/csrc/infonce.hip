@@ -478,10 +478,9 @@ __global__ __launch_bounds__(kNceMainBlock) void nce_main_kernel(NceArgs args, i
   const bool diag_wave = a == (p & 1);
 
   // Software pipeline, one barrier per stage.  In stage st a wavefront issues
-  //   the last MFMAs of O^T(st-2), whose operands it kept in registers,
   //   16 MFMAs of S^T(st)                     (+ the fetches of stage st+1),
-  //   the first MFMAs of O^T += Kh^T(st-1) P(st-1), with the soft-max of
-  //   S^T(st) between them on the vector unit,
+  //   16 MFMAs of O^T += Kh^T(st-1) P(st-1)   with the soft-max of S^T(st)
+  //                                           between them on the vector unit,
   // then writes P(st) for its partner and meets the others at the barrier.  A
   // SIMD holds two wavefronts of the workgroup, so the vector work of one runs
   // under the MFMAs of the other.
@@ -489,15 +488,14 @@ __global__ __launch_bounds__(kNceMainBlock) void nce_main_kernel(NceArgs args, i
   // Operand fragments are read from LDS four MFMAs ahead of their use, into a
   // ring of four register sets, and the read-ahead runs across the phases: the
   // first operands of the second product are requested during the last steps
-  // of the first, and the MFMAs held back over the barrier cover the latency
-  // of the first reads of the next stage.  The order is pinned with scheduling
-  // barriers, because left to itself the compiler reads every fragment right
-  // in front of its MFMA and the LDS latency is paid at every step.
+  // of the first.  The order is pinned with scheduling barriers, because left
+  // to itself the compiler reads every fragment right in front of its MFMA
+  // and the LDS latency is paid at every step.  (Holding the last MFMAs of the
+  // second product back over the barrier, to cover the first reads of the next
+  // stage, was measured: no gain.)
   constexpr int RING = 4;
-  constexpr int NSTEP = 4 * FBH;                 // MFMAs of the second product per stage (== KK)
-  constexpr int TAIL = NSTEP >= 8 ? RING : 0;    // of which held back over the barrier
-  constexpr int BODY = NSTEP - TAIL;             // the others carry the soft-max
-  static_assert(NSTEP == KK && BODY >= 1 && BODY <= 16, "feature width");
+  constexpr int NSTEP = 4 * FBH;  // MFMAs of the second product per stage (== KK), which also carry the soft-max
+  static_assert(NSTEP == KK && NSTEP <= 16, "feature width");
   const uint32_t xlane = (uint32_t)(p * 4096 + lane * 16);
   uint8_t* const xch0 = &xch[0][0][0][0][0];
   // Second product: O^T[f][q] += sum_key Kh^T[f][key] P[key][q] over both tiles
@@ -519,19 +517,7 @@ __global__ __launch_bounds__(kNceMainBlock) void nce_main_kernel(NceArgs args, i
     __builtin_memcpy(&v, &praw, 16);
     return v;
   };
-  // operands of the held-back steps BODY .. NSTEP-1 of the previous stage's second product
-  bf16x8 trH[RING], pbH[4];
-  auto tail_steps = [&]() {
-#pragma unroll
-    for (int j = 0; j < TAIL; ++j) {
-      const int step = BODY + j;
-      oacc[step % FBH] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(trH[j], pbH[step / FBH], oacc[step % FBH], 0, 0, 0);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-  };
-
-  // MODE 0: the split's first stage (no second product yet), 1: its second
-  // stage (nothing held back yet), 2: any later stage.
+  // MODE 0: the split's first stage (no second product yet), 1: any later stage.
   // cur / prev / nxt: byte offsets of the buffers of stages st, st-1, st+1.
   auto one_stage = [&](int st, int cur, int prev, int nxt, auto mode_tag) {
     constexpr int MODE = decltype(mode_tag)::value;
@@ -558,7 +544,6 @@ __global__ __launch_bounds__(kNceMainBlock) void nce_main_kernel(NceArgs args, i
 #pragma unroll
     for (int i = 0; i < RING; ++i) kr[i] = read_k(i);
     __builtin_amdgcn_sched_barrier(0);
-    if (MODE == 2) tail_steps();
 
     // S^T[key][q] = sum_f Kh[key][f] Q[q][f] for tile a of the stage; the
     // next stage's fetches are issued between the MFMAs, into the buffer that
@@ -607,17 +592,13 @@ __global__ __launch_bounds__(kNceMainBlock) void nce_main_kernel(NceArgs args, i
       softmax_elems(0, 16);
     } else {
 #pragma unroll
-      for (int step = 0; step < BODY; ++step) {
+      for (int step = 0; step < NSTEP; ++step) {
         oacc[step % FBH] =
             __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr[step % RING], pbT[step / FBH], oacc[step % FBH], 0, 0, 0);
         if (step + RING < NSTEP) tr[step % RING] = read_t(atc, step + RING);
-        softmax_elems(16 * step / BODY, 16 * (step + 1) / BODY);
+        softmax_elems(16 * step / NSTEP, 16 * (step + 1) / NSTEP);
         __builtin_amdgcn_sched_barrier(0);
       }
-#pragma unroll
-      for (int j = 0; j < TAIL; ++j) trH[j] = tr[(BODY + j) % RING];
-#pragma unroll
-      for (int T = 0; T < 4; ++T) pbH[T] = pbT[T];
     }
     if (st == diag_stage && diag_wave) {  // the tile that holds this pair's own keys (uniform)
       // The positive key's own term leaves the second product here: P~_ii stays
@@ -654,16 +635,11 @@ __global__ __launch_bounds__(kNceMainBlock) void nce_main_kernel(NceArgs args, i
       nxt = t;
     };
     one_stage(s0, cur, prev, nxt, std::integral_constant<int, 0>{});
-    if (s0 + 1 < s1) {
+    for (int st = s0 + 1; st < s1; ++st) {
       rotate();
-      one_stage(s0 + 1, cur, prev, nxt, std::integral_constant<int, 1>{});
-      for (int st = s0 + 2; st < s1; ++st) {
-        rotate();
-        one_stage(st, cur, prev, nxt, std::integral_constant<int, 2>{});
-      }
+      one_stage(st, cur, prev, nxt, std::integral_constant<int, 1>{});
     }
-    // the second product of the last stage, its first reads ahead of the
-    // held-back steps of the one before
+    // the second product of the last stage
     {
       uint32_t atc[FBH][2];
 #pragma unroll
@@ -678,7 +654,6 @@ __global__ __launch_bounds__(kNceMainBlock) void nce_main_kernel(NceArgs args, i
 #pragma unroll
       for (int i = 0; i < RING; ++i) tr[i] = read_t(atc, i);
       __builtin_amdgcn_sched_barrier(0);
-      if (s0 + 1 < s1) tail_steps();
 #pragma unroll
       for (int step = 0; step < NSTEP; ++step) {
         oacc[step % FBH] =
