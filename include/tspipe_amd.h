@@ -97,6 +97,21 @@ int64_t ts_ema_plan(const void* const* t, const void* const* s, void* const* out
 int ts_ema_multi(const ts_ema_chunk* table_dev, int64_t n_chunks, int64_t chunk_elems, float m32,
                  float c32, ts_stream_t stream);
 
+/* The same two calls for parameter lists in another floating type (the
+ * reference's per-tensor expression works on whatever dtype the parameters
+ * have): dtype TS_F32, TS_BF16 or TS_F16, the same for t, s and out.  The
+ * table's pointers are then element pointers of that type (for TS_F32 the
+ * calls are ts_ema_plan / ts_ema_multi themselves).  Arithmetic as the eager
+ * ops do it for a 2-byte type: each product and the sum are formed in fp32 and
+ * rounded to the type, out = r(r(t*m32) + r(s*c32)).  Pointers must be aligned
+ * to the element size; chunk_elems is a positive multiple of 2048 for the
+ * 2-byte types (or 0 = automatic). */
+int64_t ts_ema_plan_dtype(const void* const* t, const void* const* s, void* const* out,
+                          const int64_t* numel, int64_t n_tensors, int64_t chunk_elems, int dtype,
+                          ts_ema_chunk* table, int64_t capacity);
+int ts_ema_multi_dtype(const ts_ema_chunk* table_dev, int64_t n_chunks, int64_t chunk_elems, float m32,
+                       float c32, int dtype, ts_stream_t stream);
+
 /* The same launch, also writing a clone of the student values: for every
  * chunk, s is copied to (char*)out + clone_offset_bytes.  Fuses the pipeline's
  * `online_new_param = [t.detach().clone() for t in online_prev_param]`

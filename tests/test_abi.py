@@ -105,6 +105,30 @@ def test_ema_plan_alignment_flags_and_errors():
     assert rc == (100000 + 4095) // 4096
 
 
+def test_ema_plan_for_two_byte_types():
+    lib = _lib.lib()
+    numels = [5000, 3, 4096]
+    t, s, o = _u64([0x10000, 0x20002, 0x30000]), _u64([0x50000, 0x60002, 0x70000]), _u64([0x90000, 0xa0002, 0xb0000])
+    n = np.asarray(numels, dtype=np.int64)
+    for dtype in (1, 2):  # TS_BF16, TS_F16
+        args = (t.ctypes.data, s.ctypes.data, o.ctypes.data, n.ctypes.data, 3, 2048, dtype)
+        count = lib.ts_ema_plan_dtype(*args, None, 0)
+        assert count == 3 + 1 + 2
+        table = (EmaChunk * count)()
+        assert lib.ts_ema_plan_dtype(*args, ctypes.addressof(table), count) == count
+        # element pointers advance by 2 bytes per element; the 2-byte aligned tensor is flagged
+        assert [(c.t - 0x10000, c.n) for c in table[:3]] == [(0, 2048), (4096, 2048), (8192, 904)]
+        assert table[3].t == 0x20002 and table[3].n == 3 and table[3].flags == 0
+        assert [c.flags for c in table[:3]] == [1, 1, 1] and table[5].out == 0xb0000 + 4096
+    bad = (t.ctypes.data, s.ctypes.data, o.ctypes.data, n.ctypes.data, 3)
+    assert lib.ts_ema_plan_dtype(*bad, 1024, 1, None, 0) == -1   # 2-byte chunks are multiples of 2048
+    assert lib.ts_ema_plan_dtype(*bad, 2048, 7, None, 0) == -1   # unknown dtype
+    odd = _u64([0x10001])
+    assert lib.ts_ema_plan_dtype(odd.ctypes.data, s.ctypes.data, o.ctypes.data, n.ctypes.data, 1, 2048, 1, None, 0) == -4
+    # dtype 0 is ts_ema_plan itself
+    assert lib.ts_ema_plan_dtype(*bad, 4096, 0, None, 0) == lib.ts_ema_plan(*bad, 4096, None, 0)
+
+
 def _plan_copy(src, dst, nbytes, chunk, cap=None):
     lib = _lib.lib()
     src, dst, nbytes = _u64(src), _u64(dst), np.asarray(nbytes, dtype=np.int64)

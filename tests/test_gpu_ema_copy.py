@@ -74,10 +74,48 @@ def test_ema_in_place_form(device):
         assert bits_equal(t, w) and t.data_ptr() == p
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_ema_two_byte_parameter_lists(device, dtype):
+    # the reference's expression runs on whatever dtype the parameters have
+    # (benchmarks/byol/trainer.py:209): each product and the sum rounded to the type
+    g = seeded(21)
+    shapes = [(64, 3, 7, 7), (64,), (1000, 512), (3,), (1,), (17, 5), (2048 * 3 + 5,)]
+    teacher = [(torch.randn(s, generator=g) * 0.3).to(dtype) for s in shapes]
+    student = [(torch.randn(s, generator=g) * 0.3).to(dtype) for s in shapes]
+    t_dev, s_dev = [t.to(device) for t in teacher], [s.to(device) for s in student]
+    for m in (0.99, 0.996, 0.5):
+        got = ta.calculate_target_network_parameters(m, s_dev, t_dev)
+        want = ts_oracle.ema_update(m, student, teacher)
+        for a, b, t in zip(got, want, t_dev):
+            assert a.dtype == dtype and a.shape == b.shape and bits_equal(a, b)
+    # views that are only 2-byte aligned, and the in-place form
+    base_t, base_s = torch.randn(5000, generator=g).to(dtype), torch.randn(5000, generator=g).to(dtype)
+    bt, bs = base_t.to(device), base_s.to(device)
+    got = ta.momentum_update(0.9, [bs[1:4098], bs[4099:4100]], [bt[3:4100], bt[4101:4102]])
+    want = ts_oracle.ema_update(0.9, [base_s[1:4098], base_s[4099:4100]], [base_t[3:4100], base_t[4101:4102]])
+    for a, b in zip(got, want):
+        assert bits_equal(a, b)
+    params_t = [torch.nn.Parameter(t.clone()) for t in t_dev]
+    ta.update_target_network_parameters_(s_dev, params_t, 0.99)
+    for p, w in zip(params_t, ts_oracle.ema_update(0.99, student, teacher)):
+        assert bits_equal(p, w)
+    # chained: the rounding of every step is the reference's
+    t_cpu, cur = teacher, t_dev
+    for _ in range(20):
+        cur = ta.momentum_update(0.99, s_dev, cur)
+        t_cpu = ts_oracle.ema_update(0.99, student, t_cpu)
+    for a, b in zip(cur, t_cpu):
+        assert bits_equal(a, b)
+
+
 def test_ema_rejects_bad_inputs(device):
     a = torch.zeros(8, device=device)
     with pytest.raises(TypeError):
-        ta.momentum_update(0.9, [a.half()], [a.half()])
+        ta.momentum_update(0.9, [a.half()], [a])          # mixed types
+    with pytest.raises(TypeError):
+        ta.momentum_update(0.9, [a.double()], [a.double()])
+    with pytest.raises(TypeError):
+        ta.clone_and_update(0.9, [a.half()], [a.half()])  # the fused form is fp32
     with pytest.raises(ValueError):
         ta.momentum_update(0.9, [a], [torch.zeros(9, device=device)])
     with pytest.raises(TypeError):

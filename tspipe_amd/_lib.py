@@ -27,6 +27,9 @@ SIGNATURES = {
     "ts_ema_auto_chunk": (c_int64, [c_int64]),
     "ts_ema_plan": (c_int64, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_int64]),
     "ts_ema_multi": (c_int, [c_void_p, c_int64, c_int64, c_float, c_float, c_void_p]),
+    "ts_ema_plan_dtype": (c_int64, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int, c_void_p,
+                                    c_int64]),
+    "ts_ema_multi_dtype": (c_int, [c_void_p, c_int64, c_int64, c_float, c_float, c_int, c_void_p]),
     "ts_ema_clone_multi": (c_int, [c_void_p, c_int64, c_int64, c_float, c_float, c_int64, c_void_p]),
     "ts_copy_auto_chunk": (c_int64, [c_int64]),
     "ts_copy_plan": (c_int64, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_int64]),

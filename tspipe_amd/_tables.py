@@ -132,7 +132,7 @@ def clear_table_cache() -> None:
 
 
 def stage_ema(t_ptrs: np.ndarray, s_ptrs: np.ndarray, o_ptrs: np.ndarray, numels: np.ndarray,
-              device: torch.device, chunk_elems: int = 0):
+              device: torch.device, chunk_elems: int = 0, dtype: int = 0):
     """Plans the chunk table of one EMA launch and puts it on the device.
 
     A training loop presents the same few (teacher, student, output) pointer
@@ -147,21 +147,22 @@ def stage_ema(t_ptrs: np.ndarray, s_ptrs: np.ndarray, o_ptrs: np.ndarray, numels
         chunk_elems = lib.ts_ema_auto_chunk(int(numels.sum()))
     stream_id = torch.cuda.current_stream(device).cuda_stream
     key = b"".join((t_ptrs[:n].tobytes(), s_ptrs[:n].tobytes(), o_ptrs[:n].tobytes(), numels[:n].tobytes(),
-                    int(chunk_elems).to_bytes(8, "little"), int(stream_id).to_bytes(8, "little")))
+                    int(chunk_elems).to_bytes(8, "little"), int(stream_id).to_bytes(8, "little"),
+                    bytes((dtype,))))
     cache = _table_cache(device)
     with _table_lock:
         hit = cache.get(key)
         if hit is not None:
             cache.move_to_end(key)
             return hit
-    args = (t_ptrs.ctypes.data, s_ptrs.ctypes.data, o_ptrs.ctypes.data, numels.ctypes.data, n, chunk_elems)
+    args = (t_ptrs.ctypes.data, s_ptrs.ctypes.data, o_ptrs.ctypes.data, numels.ctypes.data, n, chunk_elems, dtype)
     ring = _ring(device)
     slot = ring.acquire(0)
-    count = lib.ts_ema_plan(*args, slot.pinned.data_ptr(), slot.capacity)
+    count = lib.ts_ema_plan_dtype(*args, slot.pinned.data_ptr(), slot.capacity)
     if count == -2:  # TS_ERR_CAPACITY: count, grow the slot, plan again
-        count = _lib.check(lib.ts_ema_plan(*args, None, 0), "ts_ema_plan(count)")
+        count = _lib.check(lib.ts_ema_plan_dtype(*args, None, 0), "ts_ema_plan(count)")
         slot = ring.grow(slot, count)
-        count = lib.ts_ema_plan(*args, slot.pinned.data_ptr(), slot.capacity)
+        count = lib.ts_ema_plan_dtype(*args, slot.pinned.data_ptr(), slot.capacity)
     _lib.check(count, "ts_ema_plan")
     nbytes = count * ENTRY_BYTES
     dev = torch.empty(max(nbytes, ENTRY_BYTES), dtype=torch.uint8, device=device)

@@ -81,6 +81,72 @@ __global__ __launch_bounds__(kEmaBlock) void ema_multi_kernel(const ts_ema_chunk
   }
 }
 
+// The same update for parameter lists kept in a 2-byte floating type.  The
+// eager ops the reference runs on such tensors form each product and the sum
+// in fp32 and round every result to the type: out = r(r(t*m) + r(s*c)).
+constexpr int kSubElems2 = kEmaBlock * 8;  // one 16-byte vector per thread and operand
+
+// Every fp32 intermediate is pinned in a register before it is narrowed:
+// otherwise the compiler folds the widening, the fp32 operation and the
+// narrowing into one mixed-precision instruction that rounds once, which
+// differs from the two roundings of the eager ops whenever the fp32 result
+// lands on a tie of the narrow type.
+__device__ __forceinline__ float ema_pin(float x) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("" : "+v"(x));
+#endif
+  return x;
+}
+
+template <typename T>
+__device__ __forceinline__ T ema1_t(T t, T s, float m, float c) {
+#pragma clang fp contract(off)
+  const float a = to_f32(from_f32<T>(ema_pin(to_f32(t) * m)));
+  const float b = to_f32(from_f32<T>(ema_pin(to_f32(s) * c)));
+  return from_f32<T>(ema_pin(a + b));
+}
+
+template <typename T>
+__global__ __launch_bounds__(kEmaBlock) void ema_multi_kernel_2byte(const ts_ema_chunk* __restrict__ table,
+                                                                    uint32_t subs, float m, float c) {
+  const uint32_t chunk = blockIdx.x / subs, sub = blockIdx.x % subs;
+  const ts_ema_chunk ch = table[chunk];
+  const uint32_t begin = sub * kSubElems2;
+  if (begin >= ch.n) return;
+  const uint32_t n = (ch.n - begin < (uint32_t)kSubElems2) ? ch.n - begin : (uint32_t)kSubElems2;
+  const T* __restrict__ tp = reinterpret_cast<const T*>(ch.t) + begin;
+  const T* __restrict__ sp = reinterpret_cast<const T*>(ch.s) + begin;
+  T* __restrict__ op = reinterpret_cast<T*>(ch.out) + begin;
+  const uint32_t tid = threadIdx.x;
+  if (ch.flags & 1u) {
+    const uint32_t n8 = n >> 3;
+    if (tid < n8) {
+      const u32x4 ra = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(tp) + tid);
+      const u32x4 rb = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(sp) + tid);
+      T a[8], b[8], r[8];
+      __builtin_memcpy(a, &ra, 16);
+      __builtin_memcpy(b, &rb, 16);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) r[e] = ema1_t<T>(a[e], b[e], m, c);
+      u32x4 rr;
+      __builtin_memcpy(&rr, r, 16);
+      __builtin_nontemporal_store(rr, reinterpret_cast<u32x4*>(op) + tid);
+    }
+    const uint32_t rem = n & 7u;
+    if (tid < rem) {
+      const uint32_t i = (n8 << 3) + tid;
+      op[i] = ema1_t<T>(tp[i], sp[i], m, c);
+    }
+  } else {
+    // storage offsets that break 16-byte alignment: 2-byte accesses, coalesced
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const uint32_t i = u * kEmaBlock + tid;
+      if (i < n) op[i] = ema1_t<T>(tp[i], sp[i], m, c);
+    }
+  }
+}
+
 constexpr int kCopyBlock = 256;
 constexpr int kSubBytes = kCopyBlock * 16;
 
@@ -144,6 +210,25 @@ int ts_ema_multi(const ts_ema_chunk* table_dev, int64_t n_chunks, int64_t chunk_
   if (subs > 0x7fffffffLL || n_chunks * subs > 0x7fffffffLL) return TS_ERR_RANGE;
   TS_LAUNCH_TIMED(ts::ema_multi_kernel<false>, dim3((unsigned)(n_chunks * subs)), dim3(ts::kEmaBlock),
                   (hipStream_t)stream, table_dev, (uint32_t)subs, m32, c32, (int64_t)0);
+  return ts::check_launch();
+}
+
+int ts_ema_multi_dtype(const ts_ema_chunk* table_dev, int64_t n_chunks, int64_t chunk_elems, float m32,
+                       float c32, int dtype, ts_stream_t stream) {
+  if (dtype == TS_F32) return ts_ema_multi(table_dev, n_chunks, chunk_elems, m32, c32, stream);
+  if (dtype != TS_BF16 && dtype != TS_F16) return TS_ERR_ARG;
+  if (n_chunks < 0 || chunk_elems <= 0 || chunk_elems % ts::kSubElems2 != 0) return TS_ERR_ARG;
+  if (n_chunks == 0) return TS_OK;
+  if (!table_dev) return TS_ERR_ARG;
+  const int64_t subs = chunk_elems / ts::kSubElems2;
+  if (subs > 0x7fffffffLL || n_chunks * subs > 0x7fffffffLL) return TS_ERR_RANGE;
+  const dim3 grid((unsigned)(n_chunks * subs));
+  if (dtype == TS_BF16)
+    TS_LAUNCH_TIMED(ts::ema_multi_kernel_2byte<ts::bf16_t>, grid, dim3(ts::kEmaBlock), (hipStream_t)stream,
+                    table_dev, (uint32_t)subs, m32, c32);
+  else
+    TS_LAUNCH_TIMED(ts::ema_multi_kernel_2byte<ts::f16_t>, grid, dim3(ts::kEmaBlock), (hipStream_t)stream,
+                    table_dev, (uint32_t)subs, m32, c32);
   return ts::check_launch();
 }
 

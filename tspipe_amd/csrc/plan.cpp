@@ -27,11 +27,15 @@ int64_t ts_ema_auto_chunk(int64_t total_elems) {
   return c;
 }
 
-int64_t ts_ema_plan(const void* const* t, const void* const* s, void* const* out,
-                    const int64_t* numel, int64_t n_tensors, int64_t chunk_elems,
-                    ts_ema_chunk* table, int64_t capacity) {
+int64_t ts_ema_plan_dtype(const void* const* t, const void* const* s, void* const* out,
+                          const int64_t* numel, int64_t n_tensors, int64_t chunk_elems, int dtype,
+                          ts_ema_chunk* table, int64_t capacity) {
+  if (dtype != TS_F32 && dtype != TS_BF16 && dtype != TS_F16) return TS_ERR_ARG;
+  const int64_t esize = dtype == TS_F32 ? 4 : 2;
+  // elements in one workgroup's share: 256 threads x 16 bytes
+  const int64_t sub = 4096 / esize;
   if (n_tensors < 0 || (n_tensors > 0 && (!t || !s || !out || !numel))) return TS_ERR_ARG;
-  if (chunk_elems < 0 || chunk_elems % 1024 != 0 || chunk_elems > ((int64_t)1 << 30))
+  if (chunk_elems < 0 || chunk_elems % sub != 0 || chunk_elems > ((int64_t)1 << 30))
     return TS_ERR_ARG;
   if (chunk_elems == 0) {
     int64_t total = 0;
@@ -47,17 +51,17 @@ int64_t ts_ema_plan(const void* const* t, const void* const* s, void* const* out
     if (n < 0) return TS_ERR_ARG;
     if (n == 0) continue;
     if (!t[i] || !s[i] || !out[i]) return TS_ERR_ARG;
-    if (!aligned(t[i], 4) || !aligned(s[i], 4) || !aligned(out[i], 4)) return TS_ERR_ALIGN;
-    // chunk_elems*4 is a multiple of 16, so every chunk of a tensor shares
-    // the 16-byte alignment of the tensor's base pointers.
+    if (!aligned(t[i], esize) || !aligned(s[i], esize) || !aligned(out[i], esize)) return TS_ERR_ALIGN;
+    // chunk_elems * esize is a multiple of 16, so every chunk of a tensor
+    // shares the 16-byte alignment of the tensor's base pointers.
     const uint32_t flags = (aligned(t[i], 16) && aligned(s[i], 16) && aligned(out[i], 16)) ? 1u : 0u;
     for (int64_t off = 0; off < n; off += chunk_elems) {
       if (table) {
         if (count >= capacity) return TS_ERR_CAPACITY;
         ts_ema_chunk& c = table[count];
-        c.t = (const float*)t[i] + off;
-        c.s = (const float*)s[i] + off;
-        c.out = (float*)out[i] + off;
+        c.t = (const float*)((const char*)t[i] + off * esize);
+        c.s = (const float*)((const char*)s[i] + off * esize);
+        c.out = (float*)((char*)out[i] + off * esize);
         c.n = (uint32_t)((n - off < chunk_elems) ? (n - off) : chunk_elems);
         c.flags = flags;
       }
@@ -65,6 +69,12 @@ int64_t ts_ema_plan(const void* const* t, const void* const* s, void* const* out
     }
   }
   return count;
+}
+
+int64_t ts_ema_plan(const void* const* t, const void* const* s, void* const* out,
+                    const int64_t* numel, int64_t n_tensors, int64_t chunk_elems,
+                    ts_ema_chunk* table, int64_t capacity) {
+  return ts_ema_plan_dtype(t, s, out, numel, n_tensors, chunk_elems, TS_F32, table, capacity);
 }
 
 int64_t ts_copy_auto_chunk(int64_t total_bytes) {

@@ -26,6 +26,8 @@ kernel_events = None
 
 
 _F32 = torch.float32
+# the dtype codes of the C ABI (ts_dtype)
+_DTYPE_CODES = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
 _shape_of = operator.attrgetter("shape")
 _dtype_of = operator.attrgetter("dtype")
 _device_of = operator.attrgetter("device")
@@ -56,8 +58,8 @@ def _prepare(online: Iterable[Optional[torch.Tensor]], target: Iterable[torch.Te
     if next(iter(devices)).type != "cuda":
         raise TypeError("EMA kernel needs device tensors (the pipeline asserts the same, tspipe/gpu_task.py:407)")
     dtypes = set(map(_dtype_of, teachers)) | set(map(_dtype_of, students))
-    if dtypes != {_F32}:
-        raise TypeError(f"EMA kernel is fp32 (got {sorted(map(str, dtypes))})")
+    if len(dtypes) != 1 or next(iter(dtypes)) not in _DTYPE_CODES:
+        raise TypeError(f"EMA kernel takes one of fp32 / bf16 / fp16 for all tensors (got {sorted(map(str, dtypes))})")
     shapes = tuple(map(_shape_of, teachers))
     if shapes != tuple(map(_shape_of, students)):
         bad = next((tuple(t.shape), tuple(s.shape)) for s, t in pairs if t.shape != s.shape)
@@ -75,15 +77,21 @@ def _ptrs(tensors: Sequence[torch.Tensor]) -> np.ndarray:
 def _launch(m: float, students: Sequence[torch.Tensor], teachers: Sequence[torch.Tensor],
             out_ptrs: np.ndarray, numels: np.ndarray) -> None:
     device = teachers[0].device
+    code = _DTYPE_CODES[teachers[0].dtype]
     with torch.cuda.device(device):
-        table = _tables.stage_ema(_ptrs(teachers), _ptrs(students), out_ptrs, numels, device)
+        table = _tables.stage_ema(_ptrs(teachers), _ptrs(students), out_ptrs, numels, device, dtype=code)
         timed = kernel_events is not None
         if timed:
             start, end = _lib.time_next_launch(device)
         # the reference multiplies by the Python doubles m and (1. - m); torch
-        # rounds each to fp32 before the fp32 multiply, and so does ctypes here
-        status = _lib.lib().ts_ema_multi(table.dev_ptr, table.n_chunks, table.chunk, float(m), 1.0 - float(m),
-                                        _lib.current_stream_ptr(device))
+        # rounds each to fp32 before the multiply (also for 2-byte tensors,
+        # whose products are formed in fp32), and so does ctypes here
+        if code == 0:
+            status = _lib.lib().ts_ema_multi(table.dev_ptr, table.n_chunks, table.chunk, float(m), 1.0 - float(m),
+                                            _lib.current_stream_ptr(device))
+        else:
+            status = _lib.lib().ts_ema_multi_dtype(table.dev_ptr, table.n_chunks, table.chunk, float(m),
+                                                  1.0 - float(m), code, _lib.current_stream_ptr(device))
         _lib.check(status, "ts_ema_multi")
         if timed:
             kernel_events.append((start, end))
@@ -147,14 +155,16 @@ class _Arena:
         # stream it was made on and is only handed out again on that stream
         self.stream = torch.cuda.current_stream(device).cuda_stream if device.type == "cuda" else None
         numels = np.array(list(map(torch.Tensor.numel, teachers)), dtype=np.int64)
-        if not (numels & 3).any():
-            # every size is a multiple of 4 elements: pieces sit back to back,
+        dtype = teachers[0].dtype
+        mask = 16 // teachers[0].element_size() - 1  # elements per 16 bytes, minus one
+        if not (numels & mask).any():
+            # every size is a multiple of 16 bytes: pieces sit back to back,
             # each on a 16-byte boundary, and torch's C++ unflatten makes the views
-            self.flat = torch.empty(int(numels.sum()), dtype=_F32, device=device)
+            self.flat = torch.empty(int(numels.sum()), dtype=dtype, device=device)
             self.views = list(torch._C._nn.unflatten_dense_tensors(self.flat, teachers))
         else:
-            padded = ((numels + 3) & ~3).tolist()
-            self.flat = torch.empty(sum(padded), dtype=_F32, device=device)
+            padded = ((numels + mask) & ~mask).tolist()
+            self.flat = torch.empty(sum(padded), dtype=dtype, device=device)
             pieces = self.flat.split(padded)
             self.views = [p[:t.numel()].view(t.shape) for p, t in zip(pieces, teachers)]
         self.ptrs = _ptrs(self.views)
@@ -275,6 +285,8 @@ def momentum_update(m: float, online_new_param: Iterable[Optional[torch.Tensor]]
     students, teachers, shapes = _prepare(online_new_param, target_param, skip_none)
     if not teachers:
         return []
+    if teachers[0].dtype is not _F32:
+        shapes = (shapes, teachers[0].dtype)  # arenas of another type are another pool entry
     arena, views = _acquire_arena(teachers, shapes)
     _launch(m, students, teachers, arena.ptrs, arena.numels)
     return views
@@ -316,6 +328,8 @@ def clone_and_update(m: float, online_param: Iterable[torch.Tensor], target_para
     students, teachers, shapes = _prepare(online_param, target_param, skip_none=False)
     if not teachers:
         return [], []
+    if teachers[0].dtype is not _F32:
+        raise TypeError("the fused clone + EMA launch is fp32 (use clone_params and momentum_update for other types)")
     ema_arena, views = _acquire_arena(teachers, shapes)  # views held: the second acquire cannot hand the same arena out
     clone_arena, clone_views = _acquire_arena(teachers, shapes)
     offset = clone_arena.flat.data_ptr() - ema_arena.flat.data_ptr()
