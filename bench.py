@@ -229,22 +229,36 @@ def run_step_benchmark(steps, warmup, dev):
     }
 
 
-def _time_stream(fn, iters, warmup=5):
-    """Average milliseconds per call of fn() over `iters` back-to-back calls,
-    one pair of HIP events around the whole batch on the current stream.  The
-    calls go straight to the C ABI with preallocated buffers (about 10 us of
-    host time each), so for kernels longer than that the figure is device time."""
+def _time_stream(fn, iters=50, warmup=10, batch=1):
+    """Median milliseconds per call of fn(): `warmup` untimed calls (at least
+    10), then `iters` samples (at least 50), each sample being `batch`
+    back-to-back calls between one pair of HIP events on the current stream
+    (an event pair around every single call would add its own marker packets
+    to a kernel of a few microseconds).  Callers that rotate through several
+    buffer sets pass the number of sets as `batch`, so every sample touches
+    each set once.  The calls go straight to the C ABI with preallocated
+    buffers (about 10 us of host time each); for kernels longer than that the
+    figure is device time."""
     import torch
-    for _ in range(warmup):
+    for _ in range(max(warmup, 10)):
         fn()
     torch.cuda.synchronize()
-    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    a.record()
-    for _ in range(iters):
-        fn()
-    b.record()
+    pairs = []
+    for _ in range(max(iters, 50)):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(batch):
+            fn()
+        b.record()
+        pairs.append((a, b))
     torch.cuda.synchronize()
-    return a.elapsed_time(b) / iters
+    return statistics.median(_event_ms(pairs)) / batch
+
+
+TIMING_NOTE = ("ms: median over >=50 samples after >=10 warm-up calls; a sample is one HIP-event pair around "
+               "`calls_per_sample` back-to-back calls, one per rotating buffer set")
+MALL_BYTES = 256 << 20  # Infinity Cache: a working set below this is not an HBM measurement
+KD_MASKED_LAUNCHES = 3   # counting + compaction, row kernel (selected rows, then zero-fill), final reduction
 
 
 def _cpu_ms(fn, budget_s=1.2, max_iters=20):
@@ -305,15 +319,38 @@ def run_kernel_table(dev, with_cpu=True):
                 ts_oracle.distil_ce(s_c, t_c, m_c, T).backward()
         return f
 
-    def entry(nbytes, ms, note=None, launches=None):
+    def entry(nbytes, ms, note=None, launches=None, working_set=None, sets=1, resident_ms=None):
+        """working_set: bytes the timed calls touch between two visits of the
+        same address (all rotating sets together); sets: buffer sets rotated
+        through; resident_ms: the same call looping on ONE set, when that set
+        is smaller than the Infinity Cache."""
         gbs = nbytes / (ms * 1e-3) / 1e9
         e = {"ms": round(ms, 4), "GB/s": round(gbs, 1), "frac_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
              "algorithmic_bytes": nbytes}
         if launches:
             e["kernel_launches"] = launches
+        if working_set is not None:
+            e["working_set_bytes"] = int(working_set)
+            e["calls_per_sample"] = sets
+            if working_set < MALL_BYTES:
+                e["cache_note"] = "working set below the 256 MB Infinity Cache: not an HBM figure"
+        if resident_ms is not None:
+            e["infinity_cache_resident"] = {"ms": round(resident_ms, 4),
+                                            "GB/s": round(nbytes / (resident_ms * 1e-3) / 1e9, 1),
+                                            "note": "the same call looping on one buffer set that fits the Infinity Cache"}
         if note:
             e["note"] = note
         return e
+
+    def rotate(fns):
+        """One callable that runs fns[0], fns[1], ... in turn."""
+        state = {"i": 0}
+
+        def f():
+            fns[state["i"] % len(fns)]()
+            state["i"] += 1
+        f.keep = fns
+        return f
 
     # EMA, stand-alone (no concurrent loss), both parameter lists; kernel-only events
     for name, shapes, m in (("ema_vit_base", vit, 0.99), ("ema_resnet18", r18, 0.996)):
@@ -376,23 +413,36 @@ def run_kernel_table(dev, with_cpu=True):
         f.keep = (ws, loss)
         return f
 
-    # KD small (cfg2) and a scaled shape for a bandwidth figure
-    for name, rows in (("kd_256x100_f32", 256), ("kd_65536x100_f32", 65536)):
-        s = (torch.randn(rows, 100, generator=g) * 3).to(dev)
-        t = (torch.randn(rows, 100, generator=g) * 3).to(dev)
-        f = kd_call(s, t, None, 4.0, torch.empty_like(s))
-        out[name] = entry(3 * rows * 100 * 4, _time_stream(f, 50),
-                          "latency-bound: 2 launches of a few us each" if rows == 256 else None, 2)
-        cpu(name, kd_cpu(s, t, 4.0))
+    # KD small (cfg2, latency) and the same row width at 65536 rows for a bandwidth figure: 8 buffer
+    # sets of 78.6 MB each in turn, so that no call finds its operands in the Infinity Cache
+    s = (torch.randn(256, 100, generator=g) * 3).to(dev)
+    t = (torch.randn(256, 100, generator=g) * 3).to(dev)
+    f = kd_call(s, t, None, 4.0, torch.empty_like(s))
+    out["kd_256x100_f32"] = entry(3 * 256 * 100 * 4, _time_stream(f), "latency-bound: one launch of a few us", 1)
+    cpu("kd_256x100_f32", kd_cpu(s, t, 4.0))
+
+    def kd_sets(rows, V, n_sets):
+        fns = []
+        for _ in range(n_sets):
+            s_ = (torch.randn(rows, V, generator=g) * 3).to(dev)
+            t_ = (torch.randn(rows, V, generator=g) * 3).to(dev)
+            fns.append(kd_call(s_, t_, None, 4.0, torch.empty_like(s_)))
+            fns[-1].operands = (s_, t_)
+        return fns
+    fns = kd_sets(65536, 100, 8)
+    one = 3 * 65536 * 100 * 4
+    out["kd_65536x100_f32"] = entry(one, _time_stream(rotate(fns), batch=8), None, 1, working_set=8 * one, sets=8,
+                                    resident_ms=_time_stream(fns[0]))
+    cpu("kd_65536x100_f32", kd_cpu(*fns[0].operands, 4.0))
+    del fns
 
     # an ImageNet-sized class count (not one of the benchmark configurations): rows long enough to stream
-    s = (torch.randn(32768, 1000, generator=g) * 3).to(dev)
-    t = (torch.randn(32768, 1000, generator=g) * 3).to(dev)
-    f = kd_call(s, t, None, 4.0, torch.empty_like(s))
-    out["kd_32768x1000_f32"] = entry(3 * 32768 * 1000 * 4, _time_stream(f, 30),
-                                     "not one of the benchmark configurations", 2)
-    cpu("kd_32768x1000_f32", kd_cpu(s, t, 4.0))
-    del s, t, f
+    fns = kd_sets(32768, 1000, 2)
+    one = 3 * 32768 * 1000 * 4
+    out["kd_32768x1000_f32"] = entry(one, _time_stream(rotate(fns), batch=2), "not one of the benchmark configurations", 1,
+                                     working_set=2 * one, sets=2)
+    cpu("kd_32768x1000_f32", kd_cpu(*fns[0].operands, 4.0))
+    del fns, s, t, f
 
     # DistilBERT-shaped masked KD (cfg3) after a gather of 4 micro-batches
     pieces_s = [(torch.randn(8, 128, 30522, generator=g) * 2).to(torch.bfloat16).to(dev) for _ in range(4)]
@@ -430,13 +480,15 @@ def run_kernel_table(dev, with_cpu=True):
         _lib.check(lib.ts_kdce_pieces_fwd_bwd(a_s, a_t, a_g, a_r, 4, mptr, None, 0, 30522, 0.5, 4.0, 0.0, ws_p.data_ptr(),
                                               loss_p.data_ptr(), _lib.TS_BF16, stream), "ts_kdce_pieces_fwd_bwd")
     out["kd_masked_4_pieces_8x128x30522_bf16"] = entry(
-        3 * n_sel * row_b + (4096 - n_sel) * row_b, _time_stream(f_pieces, 30),
-        "same loss read from the 4 micro-batch outputs in place: replaces 2 gathers (2 x ~77 us) + the call below", 3)
+        3 * n_sel * row_b + (4096 - n_sel) * row_b, _time_stream(f_pieces),
+        "same loss read from the 4 micro-batch outputs in place: replaces 2 gathers (2 x ~77 us) + the call below",
+        KD_MASKED_LAUNCHES, working_set=3 * 4096 * row_b)
     del pieces_s, pieces_t, flat_s, flat_t, grads, ws_p
     f = kd_call(s_full, t_full, mask, 2.0, torch.empty_like(s_full))
-    out["kd_masked_32x128x30522_bf16"] = entry(3 * n_sel * row_b + (4096 - n_sel) * row_b, _time_stream(f, 30),
+    out["kd_masked_32x128x30522_bf16"] = entry(3 * n_sel * row_b + (4096 - n_sel) * row_b, _time_stream(f),
                                                f"n_sel={n_sel}; bytes = read s,t + write grad for selected rows, "
-                                               f"zero-fill of the other rows", 3)
+                                               f"zero-fill of the other rows", KD_MASKED_LAUNCHES,
+                                               working_set=3 * 4096 * row_b)
     if with_cpu:
         s_c, t_c, m_c = s_full.cpu(), t_full.cpu(), mask.cpu()
         sp_c, tp_c = list(s_c.chunk(4)), list(t_c.chunk(4))
@@ -451,7 +503,7 @@ def run_kernel_table(dev, with_cpu=True):
 
     # InfoNCE: cfg4 (single pair), the symmetric two-pair call of MoCo-v3's contrastive_loss, and a
     # batch four times as large, where the fixed costs of the three launches weigh less
-    def nce_entry(name, n, pairs, iters, note=None):
+    def nce_entry(name, n, pairs, note=None):
         mk = lambda: torch.nn.functional.normalize(torch.randn(n, 256, generator=g), dim=1).to(torch.bfloat16).to(dev)
         q1, k1 = mk(), mk()
         q2, k2 = (mk(), mk()) if pairs == 2 else (None, None)
@@ -464,7 +516,7 @@ def run_kernel_table(dev, with_cpu=True):
             _lib.check(lib.ts_infonce_fwd_bwd(ptr(q1), ptr(k1), ptr(q2), ptr(k2), n, 256, 0.2, ws.data_ptr(),
                                               loss.data_ptr(), ptr(d1), ptr(d2), _lib.TS_BF16, stream),
                        "ts_infonce_fwd_bwd")
-        ms = _time_stream(f, iters)
+        ms = _time_stream(f)
         flops = pairs * 2 * 2 * n * n * 256
         e = {"ms": round(ms, 4), "TFLOP/s": round(flops / (ms * 1e-3) / 1e12, 1),
              "frac_mfma_bf16_peak": round(flops / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
@@ -480,9 +532,9 @@ def run_kernel_table(dev, with_cpu=True):
                 t.grad = None
             sum(ts_oracle.infonce(a, b, 0.2) for a, b in zip(qc, kc)).backward()
         cpu(name, f_cpu)
-    nce_entry("infonce_4096x256_bf16", 4096, 1, 50)
-    nce_entry("infonce_2_pairs_4096x256_bf16", 4096, 2, 50, "both directions of the symmetric loss in one call")
-    nce_entry("infonce_16384x256_bf16", 16384, 1, 20,
+    nce_entry("infonce_4096x256_bf16", 4096, 1)
+    nce_entry("infonce_2_pairs_4096x256_bf16", 4096, 2, "both directions of the symmetric loss in one call")
+    nce_entry("infonce_16384x256_bf16", 16384, 1,
               "not one of the benchmark configurations: the same kernels at 16x the work")
 
     # BYOL loss (latency only)
@@ -495,7 +547,7 @@ def run_kernel_table(dev, with_cpu=True):
         _lib.check(lib.ts_byol_fwd_bwd(o[0].data_ptr(), o[3].data_ptr(), o[1].data_ptr(), o[2].data_ptr(), 256, 128,
                                        wsb.data_ptr(), loss.data_ptr(), g1.data_ptr(), g2.data_ptr(), _lib.TS_F32,
                                        stream), "ts_byol_fwd_bwd")
-    out["byol_256x128_f32"] = {"ms": round(_time_stream(f, 50), 4), "note": "latency-bound", "kernel_launches": 2}
+    out["byol_256x128_f32"] = {"ms": round(_time_stream(f), 4), "note": "latency-bound", "kernel_launches": 2}
     oc = [t.cpu() for t in o]
     oc[0].requires_grad_()
     oc[1].requires_grad_()
@@ -505,44 +557,100 @@ def run_kernel_table(dev, with_cpu=True):
         ts_oracle.byol_contrastive_loss(*oc).backward()
     cpu("byol_256x128_f32", byol_cpu)
 
-    # DeferredBatchNorm (cfg5): statistics only, statistics + normalise, backward
-    x = (torch.randn(32, 256, 56, 56, generator=g) * 1.5 + 0.5).to(dev)
-    y = torch.empty_like(x)
+    # DeferredBatchNorm (cfg5): 8 different micro-batches of [32, 256, 56, 56] (822 MB of inputs, and as much
+    # again of outputs) taken in turn, as the configuration has them: no call finds its micro-batch in the
+    # Infinity Cache.  Statistics only, statistics + normalise, backward, and the configuration's whole sequence.
+    MB = 8
+    dgen = torch.Generator(device=dev).manual_seed(5)
+    xs = [torch.randn(32, 256, 56, 56, generator=dgen, device=dev) * 1.5 + 0.5 for _ in range(MB)]
+    ys = [torch.empty_like(xs[0]) for _ in range(MB)]
+    x, y = xs[0], ys[0]
     z = lambda n: torch.zeros(n, device=dev)  # noqa: E731
     wsn, acc_s, acc_q, mean_b, inv_b = z(768), z(256), z(256), z(256), z(256)
+    run_m, run_v, nbt = z(256), torch.ones(256, device=dev), torch.zeros((), dtype=torch.int64, device=dev)
     gamma, beta = torch.rand(256, generator=g).to(dev) + 0.5, (torch.randn(256, generator=g) * 0.1).to(dev)
+    one_x = x.numel() * 4
 
-    def stats():
-        _lib.check(lib.ts_bn_stats(x.data_ptr(), 32, 256, 3136, wsn.data_ptr(), acc_s.data_ptr(), acc_q.data_ptr(),
-                                   mean_b.data_ptr(), inv_b.data_ptr(), 1e-5, stream), "ts_bn_stats")
+    def stats_of(xi):
+        def f():
+            _lib.check(lib.ts_bn_stats(xi.data_ptr(), 32, 256, 3136, wsn.data_ptr(), acc_s.data_ptr(), acc_q.data_ptr(),
+                                       mean_b.data_ptr(), inv_b.data_ptr(), 1e-5, stream), "ts_bn_stats")
+        return f
 
-    def apply():
-        _lib.check(lib.ts_bn_apply(x.data_ptr(), y.data_ptr(), mean_b.data_ptr(), inv_b.data_ptr(), gamma.data_ptr(),
-                                   beta.data_ptr(), 32, 256, 3136, 0, 1e-5, stream), "ts_bn_apply")
+    def apply_of(xi, yi):
+        def f():
+            _lib.check(lib.ts_bn_apply(xi.data_ptr(), yi.data_ptr(), mean_b.data_ptr(), inv_b.data_ptr(), gamma.data_ptr(),
+                                       beta.data_ptr(), 32, 256, 3136, 0, 1e-5, stream), "ts_bn_apply")
+        return f
 
-    def both():
-        stats()
-        apply()
-    out["bn_stats_32x256x56x56_f32"] = entry(x.numel() * 4, _time_stream(stats, 50), None, 1)
-    out["bn_stats_normalise_32x256x56x56_f32"] = entry(x.numel() * 12, _time_stream(both, 50), None, 2)
+    def both_of(xi, yi):
+        st_, ap_ = stats_of(xi), apply_of(xi, yi)
+
+        def f():
+            st_()
+            ap_()
+        return f
+    out["bn_stats_32x256x56x56_f32"] = entry(one_x, _time_stream(rotate([stats_of(xi) for xi in xs]), batch=MB), None, 1,
+                                             working_set=MB * one_x, sets=MB, resident_ms=_time_stream(stats_of(x)))
+    out["bn_stats_normalise_32x256x56x56_f32"] = entry(
+        3 * one_x, _time_stream(rotate([both_of(xi, yi) for xi, yi in zip(xs, ys)]), batch=MB), None, 2,
+        working_set=2 * MB * one_x, sets=MB, resident_ms=_time_stream(both_of(x, y)))
     ws4, par = z(4 * 256), {"p": 0}
 
-    def fused():
-        _lib.check(lib.ts_bn_forward_train(x.data_ptr(), y.data_ptr(), gamma.data_ptr(), beta.data_ptr(), 32, 256, 3136,
-                                           acc_s.data_ptr(), acc_q.data_ptr(), mean_b.data_ptr(), inv_b.data_ptr(),
-                                           ws4.data_ptr(), par["p"], 1e-5, stream), "ts_bn_forward_train")
-        par["p"] ^= 1
+    def fused_of(xi, yi):
+        def f():
+            _lib.check(lib.ts_bn_forward_train(xi.data_ptr(), yi.data_ptr(), gamma.data_ptr(), beta.data_ptr(), 32, 256,
+                                               3136, acc_s.data_ptr(), acc_q.data_ptr(), mean_b.data_ptr(),
+                                               inv_b.data_ptr(), ws4.data_ptr(), par["p"], 1e-5, stream),
+                       "ts_bn_forward_train")
+            par["p"] ^= 1
+        return f
     out["bn_forward_train_32x256x56x56_f32"] = entry(
-        x.numel() * 12, _time_stream(fused, 50), "the same work in 2 launches (what DeferredBatchNorm.forward runs)", 2)
-    dy, dx, dgam, dbet = torch.randn_like(x), torch.empty_like(x), z(256), z(256)
+        3 * one_x, _time_stream(rotate([fused_of(xi, yi) for xi, yi in zip(xs, ys)]), batch=MB),
+        "the same work in 2 launches (what DeferredBatchNorm.forward runs)", 2,
+        working_set=2 * MB * one_x, sets=MB, resident_ms=_time_stream(fused_of(x, y)))
 
-    def bwd():
-        _lib.check(lib.ts_bn_backward(x.data_ptr(), dy.data_ptr(), mean_b.data_ptr(), inv_b.data_ptr(), gamma.data_ptr(),
-                                      dx.data_ptr(), dgam.data_ptr(), dbet.data_ptr(), ws4.data_ptr(), par["p"], 32, 256,
-                                      3136, 1, stream), "ts_bn_backward")
-        par["p"] ^= 1
-    out["bn_backward_32x256x56x56_f32"] = entry(x.numel() * 20, _time_stream(bwd, 30),
-                                                "bytes = read x,dy twice + write dx", 2)
+    def commit():
+        _lib.check(lib.ts_bn_commit(acc_s.data_ptr(), acc_q.data_ptr(), run_m.data_ptr(), run_v.data_ptr(), nbt.data_ptr(),
+                                    256, float(MB * 32 * 3136), 0.1, stream), "ts_bn_commit")
+
+    # the configuration's own sequence: 8 micro-batches tracked (and normalised), then one commit
+    track8 = [stats_of(xi) for xi in xs]
+    fwd8 = [fused_of(xi, yi) for xi, yi in zip(xs, ys)]
+
+    def cfg5_track():
+        for f_ in track8:
+            f_()
+        commit()
+
+    def cfg5_forward():
+        for f_ in fwd8:
+            f_()
+        commit()
+    out["bn_cfg5_track_x8_commit"] = entry(MB * one_x, _time_stream(cfg5_track), "8 x _track over 8 different "
+                                           "micro-batches + _commit (momentum 0.1): one mini-batch of the configuration",
+                                           MB + 2, working_set=MB * one_x, sets=1)
+    out["bn_cfg5_forward_x8_commit"] = entry(3 * MB * one_x, _time_stream(cfg5_forward), "8 x training forward "
+                                             "(statistics + normalise with gamma, beta) + _commit: what DeferredBatchNorm "
+                                             "runs for one mini-batch of the configuration", 2 * MB + 2,
+                                             working_set=2 * MB * one_x, sets=1)
+    del ys, y
+    dys = [torch.randn(32, 256, 56, 56, generator=dgen, device=dev) for _ in range(4)]
+    dxs = [torch.empty_like(xs[0]) for _ in range(4)]
+    dy = dys[0]
+    dgam, dbet = z(256), z(256)
+
+    def bwd_of(xi, dyi, dxi):
+        def f():
+            _lib.check(lib.ts_bn_backward(xi.data_ptr(), dyi.data_ptr(), mean_b.data_ptr(), inv_b.data_ptr(),
+                                          gamma.data_ptr(), dxi.data_ptr(), dgam.data_ptr(), dbet.data_ptr(), ws4.data_ptr(),
+                                          par["p"], 32, 256, 3136, 1, stream), "ts_bn_backward")
+            par["p"] ^= 1
+        return f
+    out["bn_backward_32x256x56x56_f32"] = entry(
+        5 * one_x, _time_stream(rotate([bwd_of(xi, dyi, dxi) for xi, dyi, dxi in zip(xs, dys, dxs)]), batch=4),
+        "bytes = read x,dy twice + write dx", 2, working_set=3 * 4 * one_x, sets=4)
+    del dxs
     if with_cpu:
         x_c, dy_c, gamma_c, beta_c = x.cpu(), dy.cpu(), gamma.cpu(), beta.cpu()
         ora = ts_oracle.DeferredBNOracle(256, chunks=1 << 30, weight=gamma_c, bias=beta_c)
@@ -635,6 +743,7 @@ def main():
     }
     if not args.no_kernels:
         line["kernels"] = run_kernel_table(dev, with_cpu=not args.no_cpu)
+        line["kernels_timing_note"] = TIMING_NOTE
         line["kernels_cpu_note"] = ("cpu_ms: the oracle's eager PyTorch chain for the same operation and shape on "
                                     f"{min(os.cpu_count() or 1, int(os.environ.get('OMP_NUM_THREADS', os.cpu_count() or 1)))} "
                                     "host threads, median of up to 20 calls within ~1.2 s (a single call when one takes longer)")

@@ -272,6 +272,13 @@ def test_a_refused_call_leaves_the_next_forward_correct(device, monkeypatch):
     _check_workspace(bn)
     # a cast of the module takes the workspace along; it comes back as fp32 zeros
     bn.half()
+    # fp16 buffers under an fp32 input: refused on the host, before any kernel writes floats into them
+    with pytest.raises(TypeError, match="fp32"):
+        bn(xs[0].to(device))
+    with pytest.raises(TypeError, match="fp32"):
+        bn._track(xs[0].to(device))
+    with pytest.raises(TypeError, match="fp32"):
+        bn._commit()
     bn.float()
     assert bn._workspace(xs[0].to(device)).dtype == torch.float32
     y = bn(xs[0].to(device))

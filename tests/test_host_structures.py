@@ -189,3 +189,18 @@ def test_bind_params_repoints_without_copy():
     with pytest.raises(ValueError):
         ta.bind_params_(model.parameters(), [v.double() for v in version])
 
+
+
+def test_deferred_bn_refuses_cast_state_on_the_host():
+    # module.half() casts the accumulators, running statistics and affine parameters; the kernels
+    # read and write C floats, so the mismatch is an error raised before anything is launched
+    bn = ta.DeferredBatchNorm(4, chunks=2)
+    x = torch.zeros(2, 4, 3, 3)
+    bn._require_state(x)
+    bn.half()
+    with pytest.raises(TypeError, match="sum is torch.float16"):
+        bn._require_state(x)
+    bn.float()
+    bn.weight.data = bn.weight.data.double()
+    with pytest.raises(TypeError, match="weight is torch.float64"):
+        bn._require_state(x)

@@ -153,6 +153,27 @@ class DeferredBatchNorm(_BatchNorm):
         if input.dim() <= 2:
             raise ValueError("expected at least 3D input (got %dD input)" % input.dim())
 
+    def _require_state(self, x: Tensor) -> None:
+        """The kernels read and write the accumulators, the running statistics
+        and the affine parameters as C floats on x's device.  A module cast
+        with ``.half()`` / ``.double()`` or left on another device is refused
+        here, as ``F.batch_norm`` refuses mixed types, instead of letting a
+        kernel write 4-byte values into narrower buffers."""
+        state = [("sum", self.sum), ("sum_squares", self.sum_squares), ("running_mean", self.running_mean),
+                 ("running_var", self.running_var)]
+        if self.affine:
+            state += [("weight", self.weight), ("bias", self.bias)]
+        for name, t in state:
+            if t is None:
+                continue
+            if t.dtype != torch.float32:
+                raise TypeError(f"DeferredBatchNorm kernels are fp32: {name} is {t.dtype} (input {x.dtype})")
+            if t.device != x.device:
+                raise TypeError(f"DeferredBatchNorm: {name} is on {t.device}, the input on {x.device}")
+        nbt = self.num_batches_tracked
+        if nbt is not None and (nbt.dtype != torch.int64 or nbt.device != x.device):
+            raise TypeError(f"DeferredBatchNorm: num_batches_tracked must be int64 on {x.device}")
+
     def _workspace(self, x: Tensor) -> Tensor:
         """The layer's reduction workspace, on x's device.  Its alternating
         halves assume that the layer's calls run one after the other on the
@@ -198,6 +219,7 @@ class DeferredBatchNorm(_BatchNorm):
         Returns True once ``chunks`` micro-batches have been seen."""
         x = input.detach()
         _require_fp32_cuda(x)
+        self._require_state(x)
         x = x if x.is_contiguous() else x.contiguous()
         self._last_stats = self._stats(x, accumulate=True)
         self.counter += input.size().numel() // input.size(1)
@@ -208,6 +230,9 @@ class DeferredBatchNorm(_BatchNorm):
         """Folds the accumulated sums into the running statistics
         (tspipe/batchnorm.py:61-85)."""
         dev = self.sum.device
+        if not self.sum.is_cuda:
+            raise TypeError("DeferredBatchNorm kernels need device buffers (no host fallback)")
+        self._require_state(self.sum)
         with torch.cuda.device(dev):
             status = _lib.lib().ts_bn_commit(
                 self.sum.data_ptr(), self.sum_squares.data_ptr(), self.running_mean.data_ptr(),
@@ -221,6 +246,7 @@ class DeferredBatchNorm(_BatchNorm):
     def forward(self, input: Tensor) -> Tensor:  # type: ignore[override]
         self._check_input_dim(input)
         _require_fp32_cuda(input)
+        self._require_state(input)
         if input.size(1) != self.num_features:
             raise ValueError(f"expected {self.num_features} channels, got {input.size(1)}")
         x = input if input.is_contiguous() else input.contiguous()

@@ -58,6 +58,12 @@
 
 #include "common.h"
 
+// The LDS-DMA loads below set M0 from inline assembly and name it as
+// clobbered, so that the compiler does not assume a value of its own survives
+// them.  M0 is a register the compiler reserves, and it warns about any
+// clobber of such a register; nothing here needs M0 preserved.
+#pragma clang diagnostic ignored "-Winline-asm"
+
 namespace ts {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -339,14 +345,14 @@ __global__ __launch_bounds__(kNceMainBlock) void nce_main_kernel(NceArgs args, i
     // LDS read into a wait for ALL of them, which would undo the read-ahead of
     // the operand rings below.  Completion of these fetches is awaited
     // explicitly (vmcnt(0) in front of the stage barrier).  M0 carries the LDS
-    // destination; nothing else in this kernel uses it.
+    // destination and is named as clobbered.
 #if defined(__HIP_DEVICE_COMPILE__)
     const uint8_t* src = reinterpret_cast<const uint8_t*>(khat_p) + (int64_t)st * STAGE + goff[u];
     const uint32_t lds = (uint32_t)(uintptr_t)(nce_lds_void*)sm + (uint32_t)(base + (w * NU + u) * 1024);
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
                  :
                  : "v"(src), "s"(__builtin_amdgcn_readfirstlane(lds))
-                 : "memory");
+                 : "memory", "m0");
 #endif
   };
   // The stage after the next is requested into this XCD's L2 (one word per
@@ -365,7 +371,7 @@ __global__ __launch_bounds__(kNceMainBlock) void nce_main_kernel(NceArgs args, i
       asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off"
                    :
                    : "v"(src), "s"(__builtin_amdgcn_readfirstlane(lds))
-                   : "memory");
+                   : "memory", "m0");
     }
 #else
     (void)st, (void)dump;
@@ -406,7 +412,7 @@ __global__ __launch_bounds__(kNceMainBlock) void nce_main_kernel(NceArgs args, i
         asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
                      :
                      : "v"(qsrc[u]), "s"(__builtin_amdgcn_readfirstlane(lds_base + u * 1024))
-                     : "memory");
+                     : "memory", "m0");
       }
     };
     if (qb != nullptr || n_pieces == 0) {
