@@ -173,8 +173,8 @@ def test_device_entry_points_validate_before_launching():
     assert lib.ts_kd_fwd_bwd(p + 1, p, None, 4, 10, 10, 10, 1.0, 1.0, p, p, None, 10, 0, None) == -4
     assert lib.ts_kd_fwd_bwd(p, p, None, 1 << 25, 10, 10, 10, 1.0, 1.0, p, p, None, 10, 0, None) == -5
     assert lib.ts_byol_fwd_bwd(p, p, p, None, 4, 8, p, p, None, None, 0, None) == -1              # x2 without y2
-    assert lib.ts_infonce_fwd_bwd(p, p, None, None, 16, 100, 0.2, p, p, None, None, 1, None) == -1   # c not 64/128/256
-    assert lib.ts_infonce_fwd_bwd(p, p, None, None, 16, 64, 0.001, 0x1000, p, None, None, 1, None) == -5  # tau too small
+    assert lib.ts_infonce_fwd_bwd(p, p, None, None, 16, 600, 0.2, 0x1000, p, None, None, 1, None) == -5  # wider than 512
+    assert lib.ts_infonce_fwd_bwd(p, p, None, None, 16, 64, 0.0, 0x1000, p, None, None, 1, None) == -1   # temperature
     assert lib.ts_infonce_fwd_bwd(p, p, None, None, 16, 64, 0.2, 0x1010, p, None, None, 1, None) == -4   # workspace alignment
     assert lib.ts_infonce_fwd_bwd(p, p, None, None, 16, 64, 0.2, 0x1000, p, None, None, 7, None) == -1   # dtype
     assert lib.ts_bn_stats(None, 2, 3, 4, p, None, None, None, None, 1e-5, None) == -1

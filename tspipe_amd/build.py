@@ -12,7 +12,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ_DIR = os.path.join(HERE, "build")
 LIB_PATH = os.path.join(HERE, "libtspipe_amd.so")
-SOURCES = ["misc.cpp", "plan.cpp", "ema_copy.hip", "losses.hip", "kd.hip", "bn.hip", "infonce.hip"]
+SOURCES = ["misc.cpp", "plan.cpp", "ema_copy.hip", "losses.hip", "kd.hip", "bn.hip", "infonce.hip", "infonce_general.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # -packed-fp32-ops off: the compiler's automatic v_pk_*_f32 forms are not

@@ -56,7 +56,7 @@
 //   D[i]: row (i%4) + 4h + 8(i/4), column l%32.
 #include <type_traits>
 
-#include "common.h"
+#include "infonce_common.h"
 
 // The LDS-DMA loads below set M0 from inline assembly and name it as
 // clobbered, so that the compiler does not assume a value of its own survives
@@ -68,22 +68,15 @@ namespace ts {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 
-constexpr float kNceLog2e = 1.4426950408889634f;
-constexpr float kNceLn2 = 0.6931471805599453f;
-constexpr float kNormEps = 1e-12f;  // F.normalize's eps
 constexpr int kQTile = 128;         // q rows per workgroup of the main kernel (32 per wavefront pair)
 constexpr int kStageKeys = 64;      // keys per LDS stage (two tiles of 32)
 constexpr int kNceBlock = 256;      // prep kernel
 constexpr int kNceMainBlock = 512;  // main kernel: 8 wavefronts, two per SIMD
-constexpr int kNceMaxPieces = 8;
 
 // defined in losses.hip
 int launch_sum_scale(const float* v, int64_t n, float scale, float denom, float* out, hipStream_t stream);
-
-__host__ __device__ inline int64_t nce_round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
 
 // Workspace carve-up (all offsets multiples of 256 bytes): a small head, then
 // one region per pair.
@@ -93,65 +86,6 @@ struct NceLayout {
   size_t head_bytes;
   size_t off_rq, off_rk, off_pdiag, off_lpart, off_khat, off_qb, off_opart, pair_bytes;
 };
-
-// One (q, k) pair's pointers; the kernels pick theirs by blockIdx.z, so the two
-// pairs of the symmetric loss share every launch.  q, k and dq may come as up
-// to kNceMaxPieces row blocks (micro-batch outputs that were never
-// concatenated): piece i holds rows row0[i] .. row0[i+1]-1.  n_pieces == 0
-// means the single matrices q / k / dq.
-struct NcePair {
-  const void* q;
-  const void* k;
-  void* dq;
-  float *rq, *rk, *pdiag, *lpart, *opart;
-  uint16_t* khat;  // normalised keys, bf16, [npad][C]
-  uint16_t* qb;    // bf16 copy of the queries for fp32 / fp16 inputs, else null
-  int n_pieces;
-  int64_t row0[kNceMaxPieces];
-  const void* qp[kNceMaxPieces];
-  const void* kp[kNceMaxPieces];
-  void* dqp[kNceMaxPieces];
-};
-struct NceArgs {
-  NcePair p[2];
-};
-
-struct NceRow {
-  const void* q;
-  const void* k;
-  void* dq;
-};
-
-// Pointers to one batch row of q, k and dq (T: the storage type).
-template <typename T>
-__device__ __forceinline__ NceRow nce_row(const NcePair& pr, int64_t row, int C) {
-  NceRow r;
-  if (pr.n_pieces == 0) {
-    r.q = (const T*)pr.q + row * C;
-    r.k = (const T*)pr.k + row * C;
-    r.dq = pr.dq ? (T*)pr.dq + row * C : nullptr;
-    return r;
-  }
-  const void* qb = pr.qp[0];
-  const void* kb = pr.kp[0];
-  void* db = pr.dqp[0];
-  int64_t r0 = 0;
-#pragma unroll
-  for (int i = 1; i < kNceMaxPieces; ++i) {
-    const bool ge = i < pr.n_pieces && row >= pr.row0[i];
-    qb = ge ? pr.qp[i] : qb;
-    kb = ge ? pr.kp[i] : kb;
-    db = ge ? pr.dqp[i] : db;
-    r0 = ge ? pr.row0[i] : r0;
-  }
-  const int64_t local = row - r0;
-  r.q = (const T*)qb + local * C;
-  r.k = (const T*)kb + local * C;
-  r.dq = db ? (T*)db + local * C : nullptr;
-  return r;
-}
-
-inline size_t nce_align(size_t x) { return (x + 255) & ~(size_t)255; }
 
 // Key splits: enough workgroups for one per CU (a workgroup is 4 wavefronts,
 // one per SIMD, each with its own software pipeline; its three stage buffers
@@ -975,6 +909,8 @@ int nce_launch(NceArgs& args, int pairs, int64_t n, int64_t c, float tau, void* 
 inline void nce_clear_pieces(NcePair& P) {
   P.q = P.k = nullptr;
   P.dq = nullptr;
+  P.rq = P.rk = P.pdiag = P.lpart = P.opart = P.stat = nullptr;
+  P.khat = P.qb = nullptr;
   P.n_pieces = 0;
   for (int i = 0; i < kNceMaxPieces; ++i) {
     P.row0[i] = 0;
@@ -983,14 +919,28 @@ inline void nce_clear_pieces(NcePair& P) {
   }
 }
 
+// The bf16-MFMA path takes 2-byte inputs of width 64 / 128 / 256 at
+// temperatures its fixed soft-max reference point can represent
+// (2^(-2 log2(e)/tau) must stay a normal fp32); everything else -- fp32 inputs,
+// other widths, smaller temperatures -- goes to the fp32-MFMA path.
+inline bool nce_bf16_path(int64_t c, float tau, int dtype) {
+  return dtype != TS_F32 && (c == 64 || c == 128 || c == 256) && tau >= 0.03f;
+}
+
 }  // namespace ts
 
 extern "C" {
 
 size_t ts_infonce_workspace_bytes(int64_t n, int64_t c, int n_pairs) {
-  if (n < 0 || c <= 0 || n_pairs < 1 || n_pairs > 2) return 0;
-  const ts::NceLayout L = ts::nce_layout(n, c, n_pairs);
-  return L.head_bytes + L.pair_bytes * (size_t)n_pairs;
+  if (n < 0 || c <= 0 || c > 512 || n_pairs < 1 || n_pairs > 2) return 0;
+  // dtype and temperature decide the path at call time: room for either
+  size_t bytes = ts::nce_general_workspace_bytes(n, c, n_pairs);
+  if (c == 64 || c == 128 || c == 256) {
+    const ts::NceLayout L = ts::nce_layout(n, c, n_pairs);
+    const size_t b16 = L.head_bytes + L.pair_bytes * (size_t)n_pairs;
+    if (b16 > bytes) bytes = b16;
+  }
+  return bytes;
 }
 
 int ts_infonce_fwd_bwd(const void* q1, const void* k1, const void* q2, const void* k2, int64_t n, int64_t c,
@@ -998,15 +948,14 @@ int ts_infonce_fwd_bwd(const void* q1, const void* k1, const void* q2, const voi
                        ts_stream_t stream) {
   if (!q1 || !k1 || !workspace || !loss_out) return TS_ERR_ARG;
   if ((q2 == nullptr) != (k2 == nullptr)) return TS_ERR_ARG;
-  if (n < 0 || !(tau > 0.f)) return TS_ERR_ARG;
-  if (c != 64 && c != 128 && c != 256) return TS_ERR_ARG;
+  if (n < 0 || !(tau > 0.f) || c < 1) return TS_ERR_ARG;
   if (dtype != TS_F32 && dtype != TS_BF16 && dtype != TS_F16) return TS_ERR_ARG;
-  // fixed soft-max reference point: 2^(-2 log2(e)/tau) must stay a normal fp32
-  if (tau < 0.03f) return TS_ERR_RANGE;
-  if (n > (1 << 24)) return TS_ERR_RANGE;
+  if (c > 512 || n > (1 << 24)) return TS_ERR_RANGE;
   if ((uintptr_t)workspace & 255u) return TS_ERR_ALIGN;
-  // rows are read as 16-byte vectors
-  if (((uintptr_t)q1 | (uintptr_t)k1 | (uintptr_t)q2 | (uintptr_t)k2) & 15u) return TS_ERR_ALIGN;
+  const uintptr_t ptr_bits = (uintptr_t)q1 | (uintptr_t)k1 | (uintptr_t)q2 | (uintptr_t)k2 | (uintptr_t)dq1 | (uintptr_t)dq2;
+  if (ptr_bits & (dtype == TS_F32 ? 3u : 1u)) return TS_ERR_ALIGN;
+  // the bf16 path reads rows as 16-byte vectors; rows that are not aligned for that take the other path
+  const bool fast = ts::nce_bf16_path(c, tau, dtype) && (ptr_bits & 15u) == 0;
   hipStream_t st = (hipStream_t)stream;
   const int pairs = q2 ? 2 : 1;
   if (n == 0) {
@@ -1021,6 +970,7 @@ int ts_infonce_fwd_bwd(const void* q1, const void* k1, const void* q2, const voi
     args.p[p].k = src ? k2 : k1;
     args.p[p].dq = src ? dq2 : dq1;
   }
+  if (!fast) return ts::nce_general_launch(args, pairs, n, c, tau, workspace, loss_out, dtype, st);
   return ts::nce_launch(args, pairs, n, c, tau, workspace, loss_out, dtype, st);
 }
 
@@ -1031,12 +981,13 @@ int ts_infonce_pieces_fwd_bwd(const void* const* q1_pieces, const void* const* k
   if (!q1_pieces || !k1_pieces || !piece_rows || !workspace || !loss_out) return TS_ERR_ARG;
   if ((q2_pieces == nullptr) != (k2_pieces == nullptr)) return TS_ERR_ARG;
   if (n_pieces < 1 || n_pieces > ts::kNceMaxPieces) return TS_ERR_RANGE;
-  if (!(tau > 0.f)) return TS_ERR_ARG;
-  if (c != 64 && c != 128 && c != 256) return TS_ERR_ARG;
+  if (!(tau > 0.f) || c < 1) return TS_ERR_ARG;
   if (dtype != TS_F32 && dtype != TS_BF16 && dtype != TS_F16) return TS_ERR_ARG;
-  if (tau < 0.03f) return TS_ERR_RANGE;
+  if (c > 512) return TS_ERR_RANGE;
   if ((uintptr_t)workspace & 255u) return TS_ERR_ALIGN;
   const int pairs = q2_pieces ? 2 : 1;
+  bool fast = ts::nce_bf16_path(c, tau, dtype);
+  const uintptr_t elem_mask = dtype == TS_F32 ? 3u : 1u;
   ts::NceArgs args;
   int64_t n = 0;
   for (int p = 0; p < 2; ++p) {
@@ -1051,7 +1002,9 @@ int ts_infonce_pieces_fwd_bwd(const void* const* q1_pieces, const void* const* k
     for (int i = 0; i < n_pieces; ++i) {
       if (piece_rows[i] <= 0 || !qs[i] || !ks[i]) return TS_ERR_ARG;
       if (want != (ds && ds[i] != nullptr)) return TS_ERR_ARG;
-      if (((uintptr_t)qs[i] | (uintptr_t)ks[i] | (uintptr_t)(want ? ds[i] : nullptr)) & 15u) return TS_ERR_ALIGN;
+      const uintptr_t bits = (uintptr_t)qs[i] | (uintptr_t)ks[i] | (uintptr_t)(want ? ds[i] : nullptr);
+      if (bits & elem_mask) return TS_ERR_ALIGN;
+      if (bits & 15u) fast = false;  // the bf16 path reads rows as 16-byte vectors
       P.row0[i] = rows;
       P.qp[i] = qs[i];
       P.kp[i] = ks[i];
@@ -1062,6 +1015,7 @@ int ts_infonce_pieces_fwd_bwd(const void* const* q1_pieces, const void* const* k
     n = rows;
   }
   if (n > (1 << 24)) return TS_ERR_RANGE;
+  if (!fast) return ts::nce_general_launch(args, pairs, n, c, tau, workspace, loss_out, dtype, (hipStream_t)stream);
   return ts::nce_launch(args, pairs, n, c, tau, workspace, loss_out, dtype, (hipStream_t)stream);
 }
 

@@ -438,15 +438,20 @@ class _InfoNCEFn(torch.autograd.Function):
         if any(t.shape != q1.shape or t.dtype != q1.dtype for t in tensors):
             raise ValueError("InfoNCE inputs must agree in shape and dtype")
         n, c_in = int(q1.shape[0]), int(q1.shape[1])
-        if c_in > 256:
-            raise ValueError(f"InfoNCE kernels take embeddings of up to 256 features, got {c_in}")
-        if not tau >= 0.03:
-            raise ValueError(f"InfoNCE kernels need a temperature of at least 0.03, got {tau}")
-        # the kernels come in widths 64, 128 and 256; zero features change neither norms nor products
-        c = 64 if c_in <= 64 else 128 if c_in <= 128 else 256
+        if c_in > 512:
+            raise ValueError(f"InfoNCE kernels take embeddings of up to 512 features, got {c_in}")
+        if not tau > 0:
+            raise ValueError(f"InfoNCE needs a positive temperature, got {tau}")
         prep = [t.detach() if t.is_contiguous() else t.detach().contiguous() for t in tensors]
-        if c != c_in:
-            prep = [torch.nn.functional.pad(t, (0, c - c_in)) for t in prep]
+        # bf16 / fp16 embeddings at temperatures of 0.03 and above run on the bf16 matrix cores, whose
+        # kernels come in widths 64, 128 and 256: narrower rows are padded (zero features change neither
+        # norms nor products).  fp32 embeddings, wider rows and smaller temperatures take the fp32
+        # kernels, which accept any width as it is.
+        c = c_in
+        if q1.dtype != torch.float32 and tau >= 0.03 and c_in <= 256:
+            c = 64 if c_in <= 64 else 128 if c_in <= 128 else 256
+            if c != c_in:
+                prep = [torch.nn.functional.pad(t, (0, c - c_in)) for t in prep]
         dev = q1.device
         lib = _lib.lib()
         pairs = 2 if q2 is not None else 1
@@ -543,10 +548,10 @@ class _PairPiecesFn(torch.autograd.Function):
         with torch.cuda.device(dev):
             stream = _lib.current_stream_ptr(dev)
             if kind == "infonce":
-                if c not in (64, 128, 256):
-                    raise ValueError(f"InfoNCE on pieces takes 64, 128 or 256 features, got {c} (gather and pad instead)")
-                if not tau >= 0.03:
-                    raise ValueError(f"InfoNCE kernels need a temperature of at least 0.03, got {tau}")
+                if c > 512:
+                    raise ValueError(f"InfoNCE kernels take embeddings of up to 512 features, got {c}")
+                if not tau > 0:
+                    raise ValueError(f"InfoNCE needs a positive temperature, got {tau}")
                 ws = torch.empty(lib.ts_infonce_workspace_bytes(total, c, 2), dtype=torch.uint8, device=dev)
                 status = lib.ts_infonce_pieces_fwd_bwd(ptrs(dense[0]), ptrs(dense[1]), ptrs(g1), ptrs(dense[2]),
                                                        ptrs(dense[3]), ptrs(g2), rows_arr, n, c, tau, ws.data_ptr(),
