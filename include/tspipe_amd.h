@@ -287,6 +287,19 @@ int ts_mse_fwd_bwd(const void* s, const void* t, const uint8_t* row_mask, int64_
                    void* workspace, float* loss_out, void* grad, int64_t ld_g, int dtype,
                    ts_stream_t stream);
 
+/* The same term on logits that were never concatenated (the micro-batch
+ * outputs that tspipe/gpu_task.py:188-191 concatenates before calling loss_fn;
+ * the term itself is benchmarks/distilbert/distiller.py:751-755): host arrays
+ * of n_pieces device pointers, piece p being a contiguous [piece_rows[p], V]
+ * matrix; row_mask covers all rows in order; grad_pieces may be NULL (or hold
+ * NULLs) for loss only.  workspace: ts_mse_workspace_bytes(sum of piece_rows, V).
+ * More than 8 pieces: TS_ERR_RANGE. */
+int ts_mse_pieces_fwd_bwd(const void* const* s_pieces, const void* const* t_pieces,
+                          void* const* grad_pieces, const int64_t* piece_rows, int n_pieces,
+                          const uint8_t* row_mask, int64_t V, float weight, int per_element,
+                          int accumulate, void* workspace, float* loss_out, int dtype,
+                          ts_stream_t stream);
+
 /* Cosine embedding loss with target +1, forward and backward: the hidden-state
  * term of DistilBERT's loss (benchmarks/distilbert/distiller.py:756-770,
  * nn.CosineEmbeddingLoss(reduction="mean") on the rows the attention mask keeps):
@@ -301,6 +314,17 @@ int ts_cosine_fwd_bwd(const void* x, const void* y, const uint8_t* row_mask, int
                       float weight, void* workspace, float* loss_out, void* gx, int dtype,
                       ts_stream_t stream);
 
+/* The same loss on hidden states that were never concatenated
+ * (tspipe/gpu_task.py:188-191; the term is distiller.py:756-770): host arrays
+ * of n_pieces device pointers, piece p being a contiguous [piece_rows[p], c]
+ * matrix; row_mask covers all rows in order; gx_pieces may be NULL (or hold
+ * NULLs) for loss only.  workspace: ts_cosine_workspace_bytes(sum of
+ * piece_rows).  More than 8 pieces: TS_ERR_RANGE. */
+int ts_cosine_pieces_fwd_bwd(const void* const* x_pieces, const void* const* y_pieces,
+                             void* const* gx_pieces, const int64_t* piece_rows, int n_pieces,
+                             const uint8_t* row_mask, int64_t c, float weight, void* workspace,
+                             float* loss_out, int dtype, ts_stream_t stream);
+
 /* ------------------------------------------------------------------------ */
 /* MoCo-v3 InfoNCE loss, forward and backward, logits never stored.      */
 /*                                                                          */
@@ -310,10 +334,17 @@ int ts_cosine_fwd_bwd(const void* x, const void* y, const uint8_t* row_mask, int
 /*   loss = CrossEntropy(logits, arange(N)) * 2 tau   (mean over rows)       */
 /*   dq   = d loss / d q  (k is the detached teacher output)                 */
 /* Up to two (q,k) pairs are summed into one loss (main.py:162); q2,k2,dq2   */
-/* may be NULL.  q*, k*: [n, c] contiguous bf16 (TS_BF16), or fp32 / fp16     */
-/* (TS_F32 / TS_F16, rounded to bf16 for the MFMA contraction; dq comes back */
-/* in the input type); c = 64, 128 or 256.                                   */
-/* workspace: ts_infonce_workspace_bytes(n, c, n_pairs) bytes, 256-aligned.  */
+/* may be NULL.  q*, k*: [n, c] contiguous, 1 <= c <= 512 (--moco-dim,        */
+/* main.py:98), any tau > 0 (--moco-t, main.py:107); dq comes back in the     */
+/* input type.  Two implementations, chosen per call:                        */
+/*   bf16 MFMA: TS_BF16 / TS_F16 inputs (fp16 rounded to bf16 for the         */
+/*     contraction) with c = 64, 128 or 256, tau >= 0.03 and rows on 16-byte  */
+/*     boundaries;                                                            */
+/*   fp32 MFMA: everything else -- TS_F32 inputs (the reference's TSPipe run  */
+/*     is fp32, main.py:151-160), other widths, smaller temperatures; every   */
+/*     product and sum in fp32, running row maximum.                          */
+/* workspace: ts_infonce_workspace_bytes(n, c, n_pairs) bytes, 256-aligned    */
+/* (covers either implementation).                                           */
 /* ------------------------------------------------------------------------ */
 
 size_t ts_infonce_workspace_bytes(int64_t n, int64_t c, int n_pairs);
@@ -328,7 +359,8 @@ int ts_infonce_fwd_bwd(const void* q1, const void* k1, const void* q2, const voi
  * loss_fn; the gradient goes straight into one buffer per piece).
  *   q1_pieces, k1_pieces, dq1_pieces (and the second pair's, or NULLs): host
  *     arrays of n_pieces device pointers, piece p being a contiguous
- *     [piece_rows[p], c] matrix, 16-byte aligned; the dq arrays may be NULL
+ *     [piece_rows[p], c] matrix (16-byte aligned for the bf16 implementation,
+ *     element-aligned otherwise); the dq arrays may be NULL
  *     (or hold NULLs) for loss only.  Both pairs share piece_rows.
  * workspace: ts_infonce_workspace_bytes(sum of piece_rows, c, n_pairs).
  * More than 8 pieces: TS_ERR_RANGE. */

@@ -639,7 +639,10 @@ def test_kd_pieces_equal_gathered(device, rows, V, dtype, with_ce):
     assert ((got - gw).abs() <= tol * gw.abs().max().item() + slack).all()
 
 
-def test_distil_loss_fn_pieces_matches_gathered_plugin(device):
+@pytest.mark.parametrize("a_mse,restrict", [(0.0, True), (0.25, True), (0.25, False)])
+def test_distil_loss_fn_pieces_matches_gathered_plugin(device, a_mse, restrict):
+    # every term reads the micro-batch outputs where they lie (KD, CE and squared error on the logits,
+    # cosine on the hidden states): bit-equal to the same plug-in on the concatenated tensors
     from argparse import Namespace
     g = seeded(260)
     chunks, bs, seq, V, H = 4, 2, 16, 30522, 32
@@ -651,8 +654,8 @@ def test_distil_loss_fn_pieces_matches_gathered_plugin(device):
     pick = torch.rand(chunks * bs, seq, generator=g) < 0.15
     lm[pick] = torch.randint(0, V, (int(pick.sum()),), generator=g)
     att = torch.rand(chunks * bs, seq, generator=g) < 0.8
-    params = Namespace(alpha_ce=0.5, alpha_mlm=2.0, alpha_clm=0.0, alpha_mse=0.0, alpha_cos=1.0, temperature=2.0,
-                       restrict_ce_to_mask=True)
+    params = Namespace(alpha_ce=0.5, alpha_mlm=2.0, alpha_clm=0.0, alpha_mse=a_mse, alpha_cos=1.0, temperature=2.0,
+                       restrict_ce_to_mask=restrict)
     labels = (lm.to(device), att.to(device))
     loss = ta.distil_loss_fn_pieces([{"logits": a, "hidden_states": (b,)} for a, b in zip(s, sh)],
                                     [{"logits": a, "hidden_states": (b,)} for a, b in zip(t, th)], labels, None, params, 0)
@@ -665,6 +668,21 @@ def test_distil_loss_fn_pieces_matches_gathered_plugin(device):
     assert loss.item() == ref.item()
     assert torch.equal(torch.cat([p.grad for p in s]), s_cat.grad)
     assert torch.equal(torch.cat([p.grad for p in sh]), sh_cat.grad)
+    # and the gathered plug-in against the oracle on a slice the fp64 evaluation can afford is
+    # test_distil_loss_fn_plugin's job; here the cosine and squared-error pieces alone, against it
+    x = [p.detach().float().cpu() for p in sh]
+    y = [p.float().cpu() for p in th]
+    xc = torch.cat(x).double().requires_grad_()
+    keep = att.reshape(-1)
+    cosv = torch.nn.functional.cosine_similarity(xc.reshape(-1, H)[keep], torch.cat(y).double().reshape(-1, H)[keep], dim=1)
+    want = (1.0 - cosv).mean()
+    want.backward()
+    xs = [p.detach().clone().requires_grad_() for p in sh]
+    got = ta.cosine_embedding_loss_pieces(xs, th, att.to(device))
+    got.backward()
+    assert rel_err(got.item(), want.item()) < 1e-3
+    gp = torch.cat([p.grad for p in xs]).double().cpu()
+    assert ((gp - xc.grad).abs() <= 1e-3 * xc.grad.abs().max() + xc.grad.abs() * 2.0 ** -8).all()
 
 
 def test_kd_pieces_argument_errors(device):

@@ -8,7 +8,7 @@ from .batch_ops import (Batch, ScatterGatherFn, batch_size, check, defaultScatte
 from .batchnorm import DeferredBatchNorm
 from .ema import (bind_params_, calculate_target_network_parameters, calculate_updated_momentum_encoder,
                   clone_and_update, clone_params, copy_params_, momentum_update, update_target_network_parameters_)
-from .losses import (Logits, SoftTarget, byol_contrastive_loss, byol_contrastive_loss_pieces, byol_loss, cosine_embedding_loss, distil_ce_loss,
+from .losses import (Logits, SoftTarget, byol_contrastive_loss, byol_contrastive_loss_pieces, byol_loss, cosine_embedding_loss, cosine_embedding_loss_pieces, distil_ce_loss,
                      distil_loss_fn, distil_loss_fn_pieces, infonce_loss, kd_ce_loss, kd_ce_loss_pieces,
                      kd_soft_target_loss, logits_mse_loss, moco_contrastive_loss, moco_contrastive_loss_pair,
                      moco_contrastive_loss_pieces,

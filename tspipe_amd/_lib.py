@@ -47,6 +47,10 @@ SIGNATURES = {
     "ts_cosine_workspace_bytes": (c_size_t, [c_int64]),
     "ts_cosine_fwd_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_float, c_void_p, c_void_p,
                                   c_void_p, c_int, c_void_p]),
+    "ts_cosine_pieces_fwd_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int64, c_float,
+                                         c_void_p, c_void_p, c_int, c_void_p]),
+    "ts_mse_pieces_fwd_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int64, c_float, c_int,
+                                      c_int, c_void_p, c_void_p, c_int, c_void_p]),
     "ts_mse_workspace_bytes": (c_size_t, [c_int64, c_int64]),
     "ts_mse_fwd_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_float, c_int, c_int,
                                c_void_p, c_void_p, c_void_p, c_int64, c_int, c_void_p]),

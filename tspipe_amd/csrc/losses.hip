@@ -112,22 +112,117 @@ __global__ __launch_bounds__(1024) void mask_count_kernel(const uint8_t* __restr
   if (threadIdx.x == 0) *out = (int)tot;
 }
 
+// Two row-wise operands and an optional gradient as up to kRowMaxPieces row
+// blocks each (micro-batch outputs that were never concatenated): piece i
+// holds rows row0[i] .. row0[i+1]-1, contiguous rows of the common width.
+// n_pieces == 0 means the single matrices a / b / g with leading dimensions.
+constexpr int kRowMaxPieces = 8;
+struct RowPieces {
+  const void* a;
+  const void* b;
+  void* g;
+  int64_t ld_a, ld_b, ld_g;
+  int n_pieces;
+  int64_t row0[kRowMaxPieces];
+  const void* ap[kRowMaxPieces];
+  const void* bp[kRowMaxPieces];
+  void* gp[kRowMaxPieces];  // all null or all set
+};
+
+template <typename T>
+struct RowPtrs {
+  const T* a;
+  const T* b;
+  T* g;
+};
+
+// Pointers to one batch row (the piece is found with a chain of selects,
+// uniform for a wavefront or workgroup that shares a row).
+template <typename T>
+__device__ __forceinline__ RowPtrs<T> row_ptrs(const RowPieces& t, int64_t row) {
+  RowPtrs<T> r;
+  if (t.n_pieces == 0) {
+    r.a = (const T*)t.a + row * t.ld_a;
+    r.b = (const T*)t.b + row * t.ld_b;
+    r.g = t.g ? (T*)t.g + row * t.ld_g : nullptr;
+    return r;
+  }
+  const void* ab = t.ap[0];
+  const void* bb = t.bp[0];
+  void* gb = t.gp[0];
+  int64_t r0 = 0;
+#pragma unroll
+  for (int i = 1; i < kRowMaxPieces; ++i) {
+    const bool ge = i < t.n_pieces && row >= t.row0[i];
+    ab = ge ? t.ap[i] : ab;
+    bb = ge ? t.bp[i] : bb;
+    gb = ge ? t.gp[i] : gb;
+    r0 = ge ? t.row0[i] : r0;
+  }
+  const int64_t local = row - r0;
+  r.a = (const T*)ab + local * t.ld_a;
+  r.b = (const T*)bb + local * t.ld_b;
+  r.g = gb ? (T*)gb + local * t.ld_g : nullptr;
+  return r;
+}
+
+inline RowPieces row_single(const void* a, const void* b, void* g, int64_t ld_a, int64_t ld_b, int64_t ld_g) {
+  RowPieces t;
+  t.a = a;
+  t.b = b;
+  t.g = g;
+  t.ld_a = ld_a;
+  t.ld_b = ld_b;
+  t.ld_g = ld_g;
+  t.n_pieces = 0;
+  for (int i = 0; i < kRowMaxPieces; ++i) {
+    t.row0[i] = 0;
+    t.ap[i] = t.bp[i] = nullptr;
+    t.gp[i] = nullptr;
+  }
+  return t;
+}
+
+// Fills a piece table from host arrays of device pointers; returns a status
+// and the total number of rows.
+inline int row_pieces(const void* const* a, const void* const* b, void* const* g, const int64_t* piece_rows,
+                      int n_pieces, int64_t width, size_t elem, RowPieces* out, int64_t* total) {
+  if (!a || !b || !piece_rows) return TS_ERR_ARG;
+  if (n_pieces < 1 || n_pieces > kRowMaxPieces) return TS_ERR_RANGE;
+  RowPieces t = row_single(nullptr, nullptr, nullptr, width, width, width);
+  const bool want = g && g[0];
+  int64_t rows = 0;
+  for (int i = 0; i < n_pieces; ++i) {
+    if (piece_rows[i] <= 0 || !a[i] || !b[i]) return TS_ERR_ARG;
+    if (want != (g && g[i] != nullptr)) return TS_ERR_ARG;
+    if (((uintptr_t)a[i] | (uintptr_t)b[i] | (uintptr_t)(want ? g[i] : nullptr)) & (elem - 1)) return TS_ERR_ALIGN;
+    t.row0[i] = rows;
+    t.ap[i] = a[i];
+    t.bp[i] = b[i];
+    t.gp[i] = want ? g[i] : nullptr;
+    rows += piece_rows[i];
+  }
+  t.n_pieces = n_pieces;
+  *out = t;
+  *total = rows;
+  return TS_OK;
+}
+
 // ---- cosine embedding loss with target +1 ----------------------------------
 //   cos_i = <x_i, y_i> / sqrt((|x_i|^2 + eps)(|y_i|^2 + eps)),  eps = 1e-12
 //   loss  = weight * mean over selected rows of (1 - cos_i);  gradient to x only.
 template <typename T>
-__global__ __launch_bounds__(256) void cosine_rows_kernel(const T* __restrict__ x, const T* __restrict__ y,
-                                                          const uint8_t* __restrict__ mask,
+__global__ __launch_bounds__(256) void cosine_rows_kernel(const RowPieces tab, const uint8_t* __restrict__ mask,
                                                           const int* __restrict__ n_sel_dev, int64_t n, int64_t c,
-                                                          float weight, float* __restrict__ row_loss,
-                                                          T* __restrict__ gx) {
+                                                          float weight, float* __restrict__ row_loss) {
   constexpr float kEps = 1e-12f;
   const int lane = threadIdx.x % kWave;
   const int64_t row = (int64_t)blockIdx.x * (256 / kWave) + threadIdx.x / kWave;
   if (row >= n) return;
-  const T* xr = x + row * c;
-  const T* yr = y + row * c;
-  T* gr = gx ? gx + row * c : nullptr;
+  const RowPtrs<T> rp = row_ptrs<T>(tab, row);
+  const T* xr = rp.a;
+  const T* yr = rp.b;
+  T* gr = rp.g;
   if (mask && mask[row] == 0) {
     if (lane == 0) row_loss[row] = 0.f;
     if (gr)
@@ -166,12 +261,10 @@ constexpr int kMseBlock = 256;
 constexpr int kMseSpan = 2048;
 
 template <typename T>
-__global__ __launch_bounds__(kMseBlock) void mse_rows_kernel(const T* __restrict__ s, const T* __restrict__ t,
-                                                              const uint8_t* __restrict__ mask,
+__global__ __launch_bounds__(kMseBlock) void mse_rows_kernel(const RowPieces tab, const uint8_t* __restrict__ mask,
                                                               const int* __restrict__ n_sel_dev, int64_t n_rows,
-                                                              int64_t V, int64_t ld_s, int64_t ld_t, int64_t ld_g,
-                                                              float weight, int per_element, int accumulate,
-                                                              float* __restrict__ partial, T* __restrict__ grad) {
+                                                              int64_t V, float weight, int per_element, int accumulate,
+                                                              float* __restrict__ partial) {
   __shared__ float lds[kMseBlock / kWave];
   const int64_t parts = gridDim.x;
   const float rows_sel = n_sel_dev ? (float)(*n_sel_dev) : (float)n_rows;
@@ -181,10 +274,11 @@ __global__ __launch_bounds__(kMseBlock) void mse_rows_kernel(const T* __restrict
     const bool sel = !mask || mask[row] != 0;
     const int64_t i0 = (int64_t)blockIdx.x * kMseSpan + threadIdx.x;  // consecutive lanes, consecutive elements
     float acc = 0.f;
+    const RowPtrs<T> rp = row_ptrs<T>(tab, row);
     if (sel) {
-      const T* sr = s + row * ld_s;
-      const T* tr = t + row * ld_t;
-      T* gr = grad ? grad + row * ld_g : nullptr;
+      const T* sr = rp.a;
+      const T* tr = rp.b;
+      T* gr = rp.g;
 #pragma unroll
       for (int j = 0; j < kMseSpan / kMseBlock; ++j) {
         const int64_t i = i0 + j * kMseBlock;
@@ -194,8 +288,8 @@ __global__ __launch_bounds__(kMseBlock) void mse_rows_kernel(const T* __restrict
           if (gr) gr[i] = from_f32<T>(accumulate ? to_f32(gr[i]) + k * d : k * d);
         }
       }
-    } else if (grad && !accumulate) {
-      T* gr = grad + row * ld_g;
+    } else if (rp.g && !accumulate) {
+      T* gr = rp.g;
 #pragma unroll
       for (int j = 0; j < kMseSpan / kMseBlock; ++j)
         if (i0 + j * kMseBlock < V) gr[i0 + j * kMseBlock] = from_f32<T>(0.f);
@@ -226,9 +320,8 @@ __global__ __launch_bounds__(1024) void mse_finalize_kernel(const float* __restr
 inline int64_t mse_parts(int64_t V) { return (V + kMseSpan - 1) / kMseSpan; }
 
 template <typename T>
-int launch_mse(const void* s, const void* t, const uint8_t* mask, int64_t n_rows, int64_t V, int64_t ld_s,
-               int64_t ld_t, float weight, int per_element, int accumulate, void* ws, float* loss_out, void* grad,
-               int64_t ld_g, hipStream_t stream) {
+int launch_mse(const RowPieces& tab, const uint8_t* mask, int64_t n_rows, int64_t V, float weight, int per_element,
+               int accumulate, void* ws, float* loss_out, hipStream_t stream) {
   int* n_sel = reinterpret_cast<int*>(ws);
   float* partial = reinterpret_cast<float*>(reinterpret_cast<char*>(ws) + 16);
   if (mask) {
@@ -238,9 +331,8 @@ int launch_mse(const void* s, const void* t, const uint8_t* mask, int64_t n_rows
   }
   const int64_t parts = mse_parts(V);
   const int64_t gy = n_rows < 65535 ? n_rows : 65535;
-  hipLaunchKernelGGL((mse_rows_kernel<T>), dim3((unsigned)parts, (unsigned)gy), dim3(kMseBlock), 0, stream,
-                     (const T*)s, (const T*)t, mask, mask ? n_sel : (const int*)nullptr, n_rows, V, ld_s, ld_t, ld_g,
-                     weight, per_element, accumulate, partial, (T*)grad);
+  hipLaunchKernelGGL((mse_rows_kernel<T>), dim3((unsigned)parts, (unsigned)gy), dim3(kMseBlock), 0, stream, tab, mask,
+                     mask ? n_sel : (const int*)nullptr, n_rows, V, weight, per_element, accumulate, partial);
   int rc = check_launch();
   if (rc) return rc;
   hipLaunchKernelGGL(mse_finalize_kernel, dim3(1), dim3(1024), 0, stream, partial, n_rows * parts,
@@ -249,8 +341,8 @@ int launch_mse(const void* s, const void* t, const uint8_t* mask, int64_t n_rows
 }
 
 template <typename T>
-int launch_cosine(const void* x, const void* y, const uint8_t* mask, int64_t n, int64_t c, float weight, void* ws,
-                  float* loss_out, void* gx, hipStream_t stream) {
+int launch_cosine(const RowPieces& tab, const uint8_t* mask, int64_t n, int64_t c, float weight, void* ws,
+                  float* loss_out, hipStream_t stream) {
   int* n_sel = reinterpret_cast<int*>(ws);
   float* row_loss = reinterpret_cast<float*>(reinterpret_cast<char*>(ws) + 16);
   if (mask) {
@@ -258,8 +350,8 @@ int launch_cosine(const void* x, const void* y, const uint8_t* mask, int64_t n, 
     int rc = check_launch();
     if (rc) return rc;
   }
-  hipLaunchKernelGGL((cosine_rows_kernel<T>), dim3((unsigned)((n + 3) / 4)), dim3(256), 0, stream, (const T*)x,
-                     (const T*)y, mask, mask ? n_sel : (const int*)nullptr, n, c, weight, row_loss, (T*)gx);
+  hipLaunchKernelGGL((cosine_rows_kernel<T>), dim3((unsigned)((n + 3) / 4)), dim3(256), 0, stream, tab, mask,
+                     mask ? n_sel : (const int*)nullptr, n, c, weight, row_loss);
   int rc = check_launch();
   if (rc) return rc;
   hipLaunchKernelGGL(sum_scale_kernel, dim3(1), dim3(1024), 0, stream, row_loss, n, weight,
@@ -298,6 +390,34 @@ int launch_sum_scale(const float* v, int64_t n, float scale, float denom, float*
   return check_launch();
 }
 
+int cosine_dispatch(const RowPieces& tab, const uint8_t* mask, int64_t n, int64_t c, float weight, void* ws,
+                    float* loss_out, int dtype, hipStream_t st) {
+  if (n == 0) {
+    hipLaunchKernelGGL(sum_scale_kernel, dim3(1), dim3(1024), 0, st, (const float*)ws, (int64_t)0, weight,
+                       (const int*)nullptr, 0.f, loss_out);
+    return check_launch();
+  }
+  switch (dtype) {
+    case TS_F32: return launch_cosine<float>(tab, mask, n, c, weight, ws, loss_out, st);
+    case TS_BF16: return launch_cosine<bf16_t>(tab, mask, n, c, weight, ws, loss_out, st);
+    default: return launch_cosine<f16_t>(tab, mask, n, c, weight, ws, loss_out, st);
+  }
+}
+
+int mse_dispatch(const RowPieces& tab, const uint8_t* mask, int64_t n_rows, int64_t V, float weight, int per_element,
+                 int accumulate, void* ws, float* loss_out, int dtype, hipStream_t st) {
+  if (n_rows == 0) {
+    hipLaunchKernelGGL(mse_finalize_kernel, dim3(1), dim3(1024), 0, st, (const float*)ws, (int64_t)0,
+                       (const int*)nullptr, (int64_t)0, V, weight, per_element, accumulate, loss_out);
+    return check_launch();
+  }
+  switch (dtype) {
+    case TS_F32: return launch_mse<float>(tab, mask, n_rows, V, weight, per_element, accumulate, ws, loss_out, st);
+    case TS_BF16: return launch_mse<bf16_t>(tab, mask, n_rows, V, weight, per_element, accumulate, ws, loss_out, st);
+    default: return launch_mse<f16_t>(tab, mask, n_rows, V, weight, per_element, accumulate, ws, loss_out, st);
+  }
+}
+
 }  // namespace ts
 
 extern "C" {
@@ -314,19 +434,23 @@ int ts_cosine_fwd_bwd(const void* x, const void* y, const uint8_t* row_mask, int
   if (dtype != TS_F32 && dtype != TS_BF16 && dtype != TS_F16) return TS_ERR_ARG;
   if (n > (1 << 24)) return TS_ERR_RANGE;
   if ((uintptr_t)workspace & 15u) return TS_ERR_ALIGN;
-  hipStream_t st = (hipStream_t)stream;
-  if (n == 0) {
-    hipLaunchKernelGGL(ts::sum_scale_kernel, dim3(1), dim3(1024), 0, st, (const float*)workspace, (int64_t)0,
-                       weight, (const int*)nullptr, 0.f, loss_out);
-    return ts::check_launch();
-  }
-  switch (dtype) {
-    case TS_F32: return ts::launch_cosine<float>(x, y, row_mask, n, c, weight, workspace, loss_out, gx, st);
-    case TS_BF16: return ts::launch_cosine<ts::bf16_t>(x, y, row_mask, n, c, weight, workspace, loss_out, gx, st);
-    default: return ts::launch_cosine<ts::f16_t>(x, y, row_mask, n, c, weight, workspace, loss_out, gx, st);
-  }
+  const ts::RowPieces tab = ts::row_single(x, y, gx, c, c, c);
+  return ts::cosine_dispatch(tab, row_mask, n, c, weight, workspace, loss_out, dtype, (hipStream_t)stream);
 }
 
+int ts_cosine_pieces_fwd_bwd(const void* const* x_pieces, const void* const* y_pieces, void* const* gx_pieces,
+                             const int64_t* piece_rows, int n_pieces, const uint8_t* row_mask, int64_t c, float weight,
+                             void* workspace, float* loss_out, int dtype, ts_stream_t stream) {
+  if (!workspace || !loss_out || c <= 0) return TS_ERR_ARG;
+  if (dtype != TS_F32 && dtype != TS_BF16 && dtype != TS_F16) return TS_ERR_ARG;
+  if ((uintptr_t)workspace & 15u) return TS_ERR_ALIGN;
+  ts::RowPieces tab;
+  int64_t n = 0;
+  const int rc = ts::row_pieces(x_pieces, y_pieces, gx_pieces, piece_rows, n_pieces, c, ts::dtype_size(dtype), &tab, &n);
+  if (rc) return rc;
+  if (n > (1 << 24)) return TS_ERR_RANGE;
+  return ts::cosine_dispatch(tab, row_mask, n, c, weight, workspace, loss_out, dtype, (hipStream_t)stream);
+}
 
 size_t ts_mse_workspace_bytes(int64_t n_rows, int64_t V) {
   if (n_rows < 0) n_rows = 0;
@@ -344,23 +468,26 @@ int ts_mse_fwd_bwd(const void* s, const void* t, const uint8_t* row_mask, int64_
   if ((uintptr_t)workspace & 15u) return TS_ERR_ALIGN;
   const size_t es = ts::dtype_size(dtype);
   if (((uintptr_t)s | (uintptr_t)t | (uintptr_t)grad) & (es - 1)) return TS_ERR_ALIGN;
-  hipStream_t st = (hipStream_t)stream;
-  if (n_rows == 0) {
-    hipLaunchKernelGGL(ts::mse_finalize_kernel, dim3(1), dim3(1024), 0, st, (const float*)workspace, (int64_t)0,
-                       (const int*)nullptr, (int64_t)0, V, weight, per_element, accumulate, loss_out);
-    return ts::check_launch();
-  }
-  switch (dtype) {
-    case TS_F32:
-      return ts::launch_mse<float>(s, t, row_mask, n_rows, V, ld_s, ld_t, weight, per_element, accumulate, workspace,
-                                   loss_out, grad, ld_g, st);
-    case TS_BF16:
-      return ts::launch_mse<ts::bf16_t>(s, t, row_mask, n_rows, V, ld_s, ld_t, weight, per_element, accumulate,
-                                        workspace, loss_out, grad, ld_g, st);
-    default:
-      return ts::launch_mse<ts::f16_t>(s, t, row_mask, n_rows, V, ld_s, ld_t, weight, per_element, accumulate,
-                                       workspace, loss_out, grad, ld_g, st);
-  }
+  const ts::RowPieces tab = ts::row_single(s, t, grad, ld_s, ld_t, ld_g);
+  return ts::mse_dispatch(tab, row_mask, n_rows, V, weight, per_element, accumulate, workspace, loss_out, dtype,
+                          (hipStream_t)stream);
+}
+
+int ts_mse_pieces_fwd_bwd(const void* const* s_pieces, const void* const* t_pieces, void* const* grad_pieces,
+                          const int64_t* piece_rows, int n_pieces, const uint8_t* row_mask, int64_t V, float weight,
+                          int per_element, int accumulate, void* workspace, float* loss_out, int dtype,
+                          ts_stream_t stream) {
+  if (!workspace || !loss_out || V <= 0) return TS_ERR_ARG;
+  if (dtype != TS_F32 && dtype != TS_BF16 && dtype != TS_F16) return TS_ERR_ARG;
+  if ((uintptr_t)workspace & 15u) return TS_ERR_ALIGN;
+  ts::RowPieces tab;
+  int64_t n_rows = 0;
+  const int rc = ts::row_pieces(s_pieces, t_pieces, grad_pieces, piece_rows, n_pieces, V, ts::dtype_size(dtype), &tab,
+                                &n_rows);
+  if (rc) return rc;
+  if (n_rows > (1 << 24) || n_rows * ts::mse_parts(V) > 0x7fffffffLL) return TS_ERR_RANGE;
+  return ts::mse_dispatch(tab, row_mask, n_rows, V, weight, per_element, accumulate, workspace, loss_out, dtype,
+                          (hipStream_t)stream);
 }
 
 

@@ -178,7 +178,7 @@ class _KDPiecesFn(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, n: int, row_mask: Optional[Tensor], labels: Optional[Tensor], T: float, weight: float,
-                ce_weight: float, ignore_index: int, *pieces: Tensor):
+                ce_weight: float, ignore_index: int, mse_weight: float, mse_per_element: bool, *pieces: Tensor):
         import ctypes
         s_pieces, t_pieces = pieces[:n], pieces[n:]
         _require_cuda(row_mask, labels, *pieces)
@@ -208,7 +208,7 @@ class _KDPiecesFn(torch.autograd.Function):
                 raise ValueError(f"{lab.numel()} labels for {total} rows")
             lab = (lab if lab.dtype == torch.int64 else lab.to(torch.int64)).contiguous()
             label_ptr = lab.data_ptr()
-        need = [ctx.needs_input_grad[7 + i] for i in range(n)]
+        need = [ctx.needs_input_grad[9 + i] for i in range(n)]
         grads = [torch.empty_like(s2) for s2 in s_flat] if any(need) else None
         lib = _lib.lib()
         code = _lib.dtype_code(dtype)
@@ -221,6 +221,15 @@ class _KDPiecesFn(torch.autograd.Function):
                                                 V, 1.0 / T, T * T * weight, float(ce_weight), ws.data_ptr(),
                                                 loss.data_ptr(), code, _lib.current_stream_ptr(dev))
         _lib.check(status, "ts_kdce_pieces_fwd_bwd")
+        if mse_weight > 0.0:
+            # the squared-error term joins loss and gradient in place, piece by piece
+            ws2 = torch.empty(lib.ts_mse_workspace_bytes(total, V), dtype=torch.uint8, device=dev)
+            with torch.cuda.device(dev):
+                status = lib.ts_mse_pieces_fwd_bwd(ptrs(s_flat), ptrs(t_flat), None if grads is None else ptrs(grads),
+                                                   (ctypes.c_int64 * n)(*rows), n, mask_ptr, V, float(mse_weight),
+                                                   1 if mse_per_element else 0, 1, ws2.data_ptr(), loss.data_ptr(),
+                                                   code, _lib.current_stream_ptr(dev))
+            _lib.check(status, "ts_mse_pieces_fwd_bwd")
         ctx.grads, ctx.need, ctx.n = grads, need, n
         ctx.shapes = [sp.shape for sp in s_pieces]
         ctx.dims = [(r, V) for r in rows]
@@ -229,18 +238,19 @@ class _KDPiecesFn(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, grad_output: Tensor):
-        none7 = (None,) * 7
+        none9 = (None,) * 9
         if ctx.grads is None:
-            return none7 + (None,) * (2 * ctx.n)
+            return none9 + (None,) * (2 * ctx.n)
         _once(ctx)
         outs = []
         for g, need, shape, dims in zip(ctx.grads, ctx.need, ctx.shapes, ctx.dims):
             outs.append(_scale_saved_grad(g, grad_output, *dims).view(shape) if need else None)
-        return none7 + tuple(outs) + (None,) * ctx.n
+        return none9 + tuple(outs) + (None,) * ctx.n
 
 
 def kd_ce_loss_pieces(s_pieces, t_pieces, labels: Optional[Tensor], T: float, kd_weight: float = 1.0,
-                      ce_weight: float = 1.0, row_mask: Optional[Tensor] = None, ignore_index: int = -100) -> Tensor:
+                      ce_weight: float = 1.0, row_mask: Optional[Tensor] = None, ignore_index: int = -100,
+                      mse_weight: float = 0.0, mse_per_element: bool = False) -> Tensor:
     """``kd_ce_loss`` on lists of micro-batch outputs (split along dim 0) that
     were never concatenated: same value as
     ``kd_ce_loss(torch.cat(s_pieces), torch.cat(t_pieces), ...)`` without either
@@ -252,7 +262,8 @@ def kd_ce_loss_pieces(s_pieces, t_pieces, labels: Optional[Tensor], T: float, kd
         raise ValueError("need as many teacher pieces as student pieces, at least one")
     n = len(s_pieces)
     return _KDPiecesFn.apply(n, row_mask, labels, float(T), float(kd_weight),
-                             float(ce_weight) if labels is not None else 0.0, int(ignore_index), *s_pieces, *t_pieces)
+                             float(ce_weight) if labels is not None else 0.0, int(ignore_index),
+                             float(mse_weight), bool(mse_per_element), *s_pieces, *t_pieces)
 
 
 class _LogitsMSEFn(torch.autograd.Function):
@@ -364,6 +375,73 @@ def cosine_embedding_loss(x: Tensor, y: Tensor, row_mask: Optional[Tensor] = Non
     the rows (last dimension = features) kept by ``row_mask``; gradient to ``x``
     only (benchmarks/distilbert/distiller.py:756-770)."""
     return _CosineFn.apply(x, y, row_mask, float(weight))
+
+
+class _CosinePiecesFn(torch.autograd.Function):
+    """The cosine embedding loss on hidden states that were never concatenated."""
+
+    @staticmethod
+    def forward(ctx, n: int, row_mask: Optional[Tensor], weight: float, *pieces: Tensor):
+        import ctypes
+        x_pieces, y_pieces = pieces[:n], pieces[n:]
+        _require_cuda(row_mask, *pieces)
+        c = int(x_pieces[0].shape[-1])
+        dtype, dev = x_pieces[0].dtype, x_pieces[0].device
+        x_flat, y_flat, rows = [], [], []
+        for xp, yp in zip(x_pieces, y_pieces):
+            if xp.shape != yp.shape or xp.dtype != dtype or yp.dtype != dtype or int(xp.shape[-1]) != c:
+                raise ValueError("the pieces of both operands must agree in shape, dtype and width")
+            x2, y2 = xp.detach().reshape(-1, c), yp.detach().reshape(-1, c)
+            x_flat.append(x2 if x2.is_contiguous() else x2.contiguous())
+            y_flat.append(y2 if y2.is_contiguous() else y2.contiguous())
+            rows.append(int(x2.shape[0]))
+        total = sum(rows)
+        mask_ptr = None
+        if row_mask is not None:
+            m = row_mask.detach().reshape(-1)
+            if m.numel() != total:
+                raise ValueError(f"row mask has {m.numel()} entries for {total} rows")
+            if m.dtype != torch.bool:
+                m = m != 0
+            m = m.contiguous().view(torch.uint8)
+            mask_ptr = m.data_ptr()
+        need = [ctx.needs_input_grad[3 + i] for i in range(n)]
+        grads = [torch.empty_like(x2) for x2 in x_flat] if any(need) else None
+        lib = _lib.lib()
+        ws = torch.empty(lib.ts_cosine_workspace_bytes(total), dtype=torch.uint8, device=dev)
+        loss = torch.empty((), dtype=torch.float32, device=dev)
+        ptrs = lambda ts: (ctypes.c_void_p * n)(*[t.data_ptr() for t in ts])  # noqa: E731
+        with torch.cuda.device(dev):
+            status = lib.ts_cosine_pieces_fwd_bwd(ptrs(x_flat), ptrs(y_flat), None if grads is None else ptrs(grads),
+                                                  (ctypes.c_int64 * n)(*rows), n, mask_ptr, c, float(weight),
+                                                  ws.data_ptr(), loss.data_ptr(), _lib.dtype_code(dtype),
+                                                  _lib.current_stream_ptr(dev))
+        _lib.check(status, "ts_cosine_pieces_fwd_bwd")
+        ctx.grads, ctx.need, ctx.n = grads, need, n
+        ctx.shapes = [xp.shape for xp in x_pieces]
+        ctx.dims = [(r, c) for r in rows]
+        ctx.backward_done = False
+        return loss
+
+    @staticmethod
+    def backward(ctx, grad_output: Tensor):
+        if ctx.grads is None:
+            return (None,) * (3 + 2 * ctx.n)
+        _once(ctx)
+        outs = []
+        for g, need, shape, dims in zip(ctx.grads, ctx.need, ctx.shapes, ctx.dims):
+            outs.append(_scale_saved_grad(g, grad_output, *dims).view(shape) if need else None)
+        return (None,) * 3 + tuple(outs) + (None,) * ctx.n
+
+
+def cosine_embedding_loss_pieces(x_pieces, y_pieces, row_mask: Optional[Tensor] = None, weight: float = 1.0) -> Tensor:
+    """``cosine_embedding_loss`` on lists of micro-batch outputs (split along
+    dim 0) that were never concatenated; ``row_mask`` covers the whole batch.
+    Up to 8 pieces per call."""
+    x_pieces, y_pieces = list(x_pieces), list(y_pieces)
+    if len(x_pieces) != len(y_pieces) or not x_pieces:
+        raise ValueError("need as many teacher pieces as student pieces, at least one")
+    return _CosinePiecesFn.apply(len(x_pieces), row_mask, float(weight), *x_pieces, *y_pieces)
 
 
 # ---------------------------------------------------------------------------
@@ -688,27 +766,25 @@ def distil_loss_fn(student_outputs, teacher_outputs, labels, tspipe_args, params
 def distil_loss_fn_pieces(student_pieces, teacher_pieces, labels, tspipe_args, params, epoch: int) -> Tensor:
     """``distil_loss_fn`` for a pipeline that hands over the per-micro-batch
     output dicts instead of gathering them first (tspipe/gpu_task.py:147,
-    170-171, 188-191 is where the reference concatenates).  The logits, by far
-    the largest tensors, are read in place by ``kd_ce_loss_pieces``; the hidden
-    states of the cosine term are small and go through ``gather``.  ``labels``
-    is the whole batch's ``(lm_labels, attention_mask)`` as in ``distil_loss_fn``.
-    The ``alpha_mse`` term has no piece-wise kernel: use ``distil_loss_fn``."""
-    from .batch_ops import Batch, gather
+    170-171, 188-191 is where the reference concatenates).  Every term reads
+    the pieces where they lie: the logits through ``kd_ce_loss_pieces`` (KD,
+    cross entropy and the ``alpha_mse`` squared error), the last hidden states
+    through ``cosine_embedding_loss_pieces``.  ``labels`` is the whole batch's
+    ``(lm_labels, attention_mask)`` as in ``distil_loss_fn``."""
     lm_labels, attention_mask = labels
-    if float(getattr(params, "alpha_mse", 0.0)) > 0.0:
-        raise NotImplementedError("alpha_mse needs the gathered logits: call distil_loss_fn")
+    alpha_mse = float(getattr(params, "alpha_mse", 0.0))
     mask = (lm_labels > -1) if params.restrict_ce_to_mask else attention_mask
     terms = _ce_terms(lm_labels, params)
     ce_labels, ce_weight = terms[0] if terms else (None, 0.0)
     s_list, t_list = [p["logits"] for p in student_pieces], [p["logits"] for p in teacher_pieces]
     loss = kd_ce_loss_pieces(s_list, t_list, ce_labels, params.temperature, kd_weight=params.alpha_ce,
-                             ce_weight=ce_weight, row_mask=mask, ignore_index=-100)
+                             ce_weight=ce_weight, row_mask=mask, ignore_index=-100, mse_weight=alpha_mse)
     for ce_labels, ce_weight in terms[1:]:
         loss = loss + kd_ce_loss_pieces(s_list, t_list, ce_labels, params.temperature, kd_weight=0.0,
                                         ce_weight=ce_weight, row_mask=mask, ignore_index=-100)
     if getattr(params, "alpha_cos", 0.0) > 0.0:
-        s_hid = gather([Batch(p["hidden_states"][-1]) for p in student_pieces])
-        t_hid = gather([Batch(p["hidden_states"][-1]) for p in teacher_pieces])
-        loss = loss + cosine_embedding_loss(s_hid, t_hid, attention_mask, params.alpha_cos)
+        loss = loss + cosine_embedding_loss_pieces([p["hidden_states"][-1] for p in student_pieces],
+                                                   [p["hidden_states"][-1] for p in teacher_pieces],
+                                                   attention_mask, params.alpha_cos)
     return loss
 
