@@ -229,7 +229,7 @@ def run_step_benchmark(steps, warmup, dev):
     }
 
 
-def _time_stream(fn, iters=50, warmup=10, batch=1):
+def _time_stream(fn, iters=50, warmup=10, batch=4):
     """Median milliseconds per call of fn(): `warmup` untimed calls (at least
     10), then `iters` samples (at least 50), each sample being `batch`
     back-to-back calls between one pair of HIP events on the current stream
@@ -238,7 +238,8 @@ def _time_stream(fn, iters=50, warmup=10, batch=1):
     buffer sets pass the number of sets as `batch`, so every sample touches
     each set once.  The calls go straight to the C ABI with preallocated
     buffers (about 10 us of host time each); for kernels longer than that the
-    figure is device time."""
+    figure is device time.  Without rotation a sample is four calls on the same
+    buffers."""
     import torch
     for _ in range(max(warmup, 10)):
         fn()
@@ -256,7 +257,8 @@ def _time_stream(fn, iters=50, warmup=10, batch=1):
 
 
 TIMING_NOTE = ("ms: median over >=50 samples after >=10 warm-up calls; a sample is one HIP-event pair around "
-               "`calls_per_sample` back-to-back calls, one per rotating buffer set")
+               "`calls_per_sample` back-to-back calls, one per rotating buffer set (4 calls on the same buffers "
+               "where the entry names no buffer sets)")
 MALL_BYTES = 256 << 20  # Infinity Cache: a working set below this is not an HBM measurement
 KD_MASKED_LAUNCHES = 3   # counting + compaction, row kernel (selected rows, then zero-fill), final reduction
 
@@ -627,10 +629,10 @@ def run_kernel_table(dev, with_cpu=True):
         for f_ in fwd8:
             f_()
         commit()
-    out["bn_cfg5_track_x8_commit"] = entry(MB * one_x, _time_stream(cfg5_track), "8 x _track over 8 different "
+    out["bn_cfg5_track_x8_commit"] = entry(MB * one_x, _time_stream(cfg5_track, batch=1), "8 x _track over 8 different "
                                            "micro-batches + _commit (momentum 0.1): one mini-batch of the configuration",
                                            MB + 2, working_set=MB * one_x, sets=1)
-    out["bn_cfg5_forward_x8_commit"] = entry(3 * MB * one_x, _time_stream(cfg5_forward), "8 x training forward "
+    out["bn_cfg5_forward_x8_commit"] = entry(3 * MB * one_x, _time_stream(cfg5_forward, batch=1), "8 x training forward "
                                              "(statistics + normalise with gamma, beta) + _commit: what DeferredBatchNorm "
                                              "runs for one mini-batch of the configuration", 2 * MB + 2,
                                              working_set=2 * MB * one_x, sets=1)

@@ -11,10 +11,10 @@
 // last workgroup of a channel in the stand-alone statistics pass, the
 // normalising kernel in the fused passes) also clears it.
 //
-// Sums are taken about a per-channel shift k_c = x[0, c, 0] (the channel's
-// first value): S' = sum(x - k), Q' = sum((x - k)^2).  The variance
-// Q'/n - (S'/n)^2 then cancels against (mean - k)^2, which is of the order
-// of the variance itself, instead of against mean^2; the raw sums the
+// Sums are taken about a per-channel shift k_c (the mean of the channel's
+// first 64 values, bn_shift): S' = sum(x - k), Q' = sum((x - k)^2).  The
+// variance Q'/n - (S'/n)^2 then cancels against (mean - k)^2, which is far
+// below the variance itself, instead of against mean^2; the raw sums the
 // reference accumulates follow exactly as  sum x = S' + n k  and
 // sum x^2 = Q' + 2 k S' + n k^2.
 #include "common.h"
@@ -23,6 +23,20 @@ namespace ts {
 
 constexpr int kBnBlock = 256;
 constexpr int kBnUnroll = 4;
+
+// The per-channel shift the sums are taken about: the mean of the first (up
+// to) 64 values of the channel's first plane.  Every wavefront of every
+// workgroup of the channel computes it from the same loads in the same order,
+// so all agree to the bit.  A single sample as the shift can sit several
+// standard deviations from the mean, and (mean - k)^2, which the sums then
+// carry and the reconstruction takes out again, costs a digit of the
+// accumulated sum of squares; the mean of 64 samples is within sigma / 8.
+__device__ __forceinline__ float bn_shift(const float* __restrict__ x, int64_t c, int64_t HW) {
+  const int lane = threadIdx.x % kWave;
+  const int m = HW < kWave ? (int)HW : kWave;
+  const float v = lane < m ? x[c * HW + lane] : 0.f;
+  return wave_sum(v) / (float)m;
+}
 
 struct PlaneSplit {
   int64_t head, nvec, tail0;  // scalar head, 16-byte vectors, first tail element
@@ -38,76 +52,63 @@ __device__ __forceinline__ PlaneSplit split_plane(const float* p, int64_t HW) {
 }
 
 // Accumulates (a, b) over the slab's elements of x (and optionally a second
-// tensor y with the same layout) through a functor: f(xv, yv, a, b).
-// Planes are taken two at a time so that the loads of both are in flight
-// before either is consumed (a plane of a small feature map is only a few
-// vectors per thread).
+// tensor y with the same layout) through a functor: f(xv, yv, a, b), with a
+// wavefront per plane: wavefront w of the workgroup takes planes n0 + w,
+// n0 + w + NW, ...  A plane of a small feature map is a few hundred 16-byte
+// vectors; dealt to 64 lanes instead of a whole workgroup, nearly every load
+// instruction has all its lanes at work (a 56 x 56 plane is 784 vectors: 12.25
+// per lane, against 3.06 per thread of a 256-thread workgroup, whose fourth
+// load has 16 threads in it).  Four loads per lane and operand are in flight at
+// a time; more of them (8, 14: the whole plane) were measured slower.
+#ifndef TS_BN_WAVE_UNROLL
+#define TS_BN_WAVE_UNROLL 4
+#endif
 template <bool TWO, int BLOCK = 256, typename F>
-__device__ __forceinline__ void slab_reduce(const float* __restrict__ x, const float* __restrict__ y,
-                                            int64_t n0, int64_t n1, int64_t C, int64_t c, int64_t HW,
-                                            float& a, float& b, F f) {
-  constexpr int PL = 2;
-  const int tid = threadIdx.x;
-  for (int64_t n = n0; n < n1; n += PL) {
-    const float* px[PL];
-    const float* py[PL];
-    PlaneSplit sp[PL];
-    bool yvec[PL], live[PL];
-    int64_t maxvec = 0;
+__device__ __forceinline__ void slab_reduce_waves(const float* __restrict__ x, const float* __restrict__ y, int64_t n0,
+                                                  int64_t n1, int64_t C, int64_t c, int64_t HW, float& a, float& b,
+                                                  F f) {
+  constexpr int NW = BLOCK / kWave;
+  constexpr int U = TS_BN_WAVE_UNROLL;
+  const int lane = threadIdx.x % kWave, w = threadIdx.x / kWave;
+  for (int64_t n = n0 + w; n < n1; n += NW) {
+    const int64_t off = (n * C + c) * HW;
+    const float* px = x + off;
+    const float* py = TWO ? y + off : nullptr;
+    const PlaneSplit sp = split_plane(px, HW);
+    const bool yvec = !TWO || ((((uintptr_t)py) & 15u) == (((uintptr_t)px) & 15u));
+    const f32x4* px4 = reinterpret_cast<const f32x4*>(px + sp.head);
+    const f32x4* py4 = reinterpret_cast<const f32x4*>(py + sp.head);
+    for (int64_t base = 0; base < sp.nvec; base += kWave * U) {
+      f32x4 v[U], vy[U];
 #pragma unroll
-    for (int p = 0; p < PL; ++p) {
-      live[p] = n + p < n1;
-      const int64_t off = ((live[p] ? n + p : n) * C + c) * HW;
-      px[p] = x + off;
-      py[p] = TWO ? y + off : nullptr;
-      sp[p] = split_plane(px[p], HW);
-      yvec[p] = !TWO || ((((uintptr_t)py[p]) & 15u) == (((uintptr_t)px[p]) & 15u));
-      if (live[p] && sp[p].nvec > maxvec) maxvec = sp[p].nvec;
-    }
-#pragma unroll
-    for (int p = 0; p < PL; ++p) {
-      if (live[p]) {
-        if (tid < sp[p].head) f(px[p][tid], TWO ? py[p][tid] : 0.f, a, b);
-        const int64_t it = sp[p].tail0 + tid;
-        if (it < HW) f(px[p][it], TWO ? py[p][it] : 0.f, a, b);
-      }
-    }
-    for (int64_t base = 0; base < maxvec; base += BLOCK * kBnUnroll) {
-      f32x4 vx[PL][kBnUnroll], vy[PL][kBnUnroll];
-#pragma unroll
-      for (int p = 0; p < PL; ++p) {
-        const f32x4* px4 = reinterpret_cast<const f32x4*>(px[p] + sp[p].head);
-        const f32x4* py4 = reinterpret_cast<const f32x4*>(py[p] + sp[p].head);
-#pragma unroll
-        for (int u = 0; u < kBnUnroll; ++u) {
-          const int64_t i = base + u * BLOCK + tid;
-          if (live[p] && i < sp[p].nvec) {
-            vx[p][u] = px4[i];
-            if (TWO) {
-              if (yvec[p]) {
-                vy[p][u] = py4[i];
-              } else {
-                const float* q = py[p] + sp[p].head + (i << 2);
-                vy[p][u] = f32x4{q[0], q[1], q[2], q[3]};
-              }
+      for (int u = 0; u < U; ++u) {
+        const int64_t i = base + u * kWave + lane;
+        if (i < sp.nvec) {
+          v[u] = px4[i];
+          if (TWO) {
+            if (yvec) {
+              vy[u] = py4[i];
+            } else {
+              const float* q = py + sp.head + (i << 2);
+              vy[u] = f32x4{q[0], q[1], q[2], q[3]};
             }
           }
         }
       }
 #pragma unroll
-      for (int p = 0; p < PL; ++p) {
-#pragma unroll
-        for (int u = 0; u < kBnUnroll; ++u) {
-          const int64_t i = base + u * BLOCK + tid;
-          if (live[p] && i < sp[p].nvec) {
-            f(vx[p][u].x, TWO ? vy[p][u].x : 0.f, a, b);
-            f(vx[p][u].y, TWO ? vy[p][u].y : 0.f, a, b);
-            f(vx[p][u].z, TWO ? vy[p][u].z : 0.f, a, b);
-            f(vx[p][u].w, TWO ? vy[p][u].w : 0.f, a, b);
-          }
+      for (int u = 0; u < U; ++u) {
+        const int64_t i = base + u * kWave + lane;
+        if (i < sp.nvec) {
+          f(v[u].x, TWO ? vy[u].x : 0.f, a, b);
+          f(v[u].y, TWO ? vy[u].y : 0.f, a, b);
+          f(v[u].z, TWO ? vy[u].z : 0.f, a, b);
+          f(v[u].w, TWO ? vy[u].w : 0.f, a, b);
         }
       }
     }
+    if (lane < sp.head) f(px[lane], TWO ? py[lane] : 0.f, a, b);
+    const int64_t it = sp.tail0 + lane;
+    if (it < HW) f(px[it], TWO ? py[it] : 0.f, a, b);
   }
 }
 
@@ -132,9 +133,9 @@ __global__ __launch_bounds__(kBnBlock) void bn_stats_kernel(const float* __restr
   const int64_t c = blockIdx.y;
   const int64_t n0 = (int64_t)blockIdx.x * slab;
   const int64_t n1 = (n0 + slab < N) ? n0 + slab : N;
-  const float k = x[c * HW];  // shift: first value of the channel
+  const float k = bn_shift(x, c, HW);
   float S = 0.f, Q = 0.f;
-  slab_reduce<false>(x, nullptr, n0, n1, C, c, HW, S, Q, [k](float xv, float, float& a, float& b) {
+  slab_reduce_waves<false>(x, nullptr, n0, n1, C, c, HW, S, Q, [k](float xv, float, float& a, float& b) {
     const float d = xv - k;
     a += d;
     b += d * d;
@@ -158,8 +159,9 @@ __global__ __launch_bounds__(kBnBlock) void bn_stats_kernel(const float* __restr
     if (ticket == gridDim.x - 1) {
       const float St = atomicExch(ws + c, 0.f), Qt = atomicExch(ws + C + c, 0.f);
       atomicExch(tickets + c, 0u);
-      if (sum) sum[c] += St + cnt * k;
-      if (sum_squares) sum_squares[c] += Qt + 2.f * k * St + cnt * k * k;
+      // sum x = S' + n k and sum x^2 = Q' + k (2 S' + n k), each with one rounding per step
+      if (sum) sum[c] += fmaf(cnt, k, St);
+      if (sum_squares) sum_squares[c] += fmaf(k, fmaf(cnt, k, 2.f * St), Qt);
       const float dm = St / cnt;  // mean - k
       if (ub_mean) ub_mean[c] = k + dm;
       if (ub_invstd) ub_invstd[c] = 1.f / sqrtf(fmaxf(Qt / cnt - dm * dm, 0.f) + eps);
@@ -203,8 +205,11 @@ __device__ __forceinline__ void bn_apply_slab(const float* __restrict__ x, float
                                               float b) {
   const int64_t n0 = (int64_t)blockIdx.x * slab;
   const int64_t n1 = (n0 + slab < N) ? n0 + slab : N;
-  const int tid = threadIdx.x;
-  for (int64_t n = n0; n < n1; ++n) {
+  // a wavefront per plane, as in slab_reduce_waves
+  constexpr int kStep = kWave;
+  const int tid = threadIdx.x % kWave;
+  const int64_t nfirst = n0 + threadIdx.x / kWave, nstep = kBnBlock / kWave;
+  for (int64_t n = nfirst; n < n1; n += nstep) {
     const int64_t off = (n * C + c) * HW;
     const float* px = x + off;
     float* py = y + off;
@@ -213,16 +218,16 @@ __device__ __forceinline__ void bn_apply_slab(const float* __restrict__ x, float
     if (tid < sp.head) py[tid] = (px[tid] - mu) * a + b;
     const f32x4* px4 = reinterpret_cast<const f32x4*>(px + sp.head);
     f32x4* py4 = reinterpret_cast<f32x4*>(py + sp.head);
-    for (int64_t base = 0; base < sp.nvec; base += kBnBlock * kBnUnroll) {
+    for (int64_t base = 0; base < sp.nvec; base += kStep * kBnUnroll) {
       f32x4 v[kBnUnroll];
 #pragma unroll
       for (int u = 0; u < kBnUnroll; ++u) {
-        const int64_t i = base + u * kBnBlock + tid;
+        const int64_t i = base + u * kStep + tid;
         if (i < sp.nvec) v[u] = px4[i];
       }
 #pragma unroll
       for (int u = 0; u < kBnUnroll; ++u) {
-        const int64_t i = base + u * kBnBlock + tid;
+        const int64_t i = base + u * kStep + tid;
         if (i < sp.nvec) {
           f32x4 r;
           r.x = (v[u].x - mu) * a + b;
@@ -278,13 +283,13 @@ __global__ __launch_bounds__(kBnBlock) void bn_apply_train_kernel(const float* _
                                                                   float* ub_invstd) {
   const int64_t c = blockIdx.y;
   const float S = ws_in[c], Q = ws_in[C + c];
-  const float k = x[c * HW];
+  const float k = bn_shift(x, c, HW);  // the statistics launch took its sums about the same value
   const float dm = S / cnt;  // mean - k
   const float mu = k + dm;
   const float istd = 1.f / sqrtf(fmaxf(Q / cnt - dm * dm, 0.f) + eps);
   if (blockIdx.x == 0 && threadIdx.x == 0) {
-    if (sum) sum[c] += S + cnt * k;
-    if (sum_squares) sum_squares[c] += Q + 2.f * k * S + cnt * k * k;
+    if (sum) sum[c] += fmaf(cnt, k, S);
+    if (sum_squares) sum_squares[c] += fmaf(k, fmaf(cnt, k, 2.f * S), Q);
     if (ub_mean) ub_mean[c] = mu;
     if (ub_invstd) ub_invstd[c] = istd;
     ws_clear[c] = 0.f;
@@ -308,7 +313,7 @@ __global__ __launch_bounds__(kBnBlock) void bn_bwd_reduce_kernel(const float* __
   const int64_t n1 = (n0 + slab < N) ? n0 + slab : N;
   const float mu = mean[c], istd = invstd[c];
   float sdy = 0.f, sdyx = 0.f;
-  slab_reduce<true>(x, dy, n0, n1, C, c, HW, sdy, sdyx, [mu, istd](float xv, float g, float& a, float& b) {
+  slab_reduce_waves<true>(x, dy, n0, n1, C, c, HW, sdy, sdyx, [mu, istd](float xv, float g, float& a, float& b) {
     a += g;
     b += g * ((xv - mu) * istd);
   });
@@ -349,9 +354,11 @@ __global__ __launch_bounds__(kBnBlock) void bn_bwd_dx_kernel(const float* __rest
     ws_clear[C + c] = 0.f;
   }
   const float mb = sum_dy * inv_cnt, mg = sum_dyx * inv_cnt;
-  const int tid = threadIdx.x;
+  // a wavefront per plane, as in slab_reduce_waves
+  constexpr int kStep = kWave;
+  const int tid = threadIdx.x % kWave;
   auto one = [=](float xv, float g) { return gi * (g - mb - ((xv - mu) * istd) * mg); };
-  for (int64_t n = n0; n < n1; ++n) {
+  for (int64_t n = n0 + threadIdx.x / kWave; n < n1; n += kBnBlock / kWave) {
     const int64_t off = (n * C + c) * HW;
     const float* px = x + off;
     const float* pg = dy + off;
@@ -360,18 +367,18 @@ __global__ __launch_bounds__(kBnBlock) void bn_bwd_dx_kernel(const float* __rest
     const bool vec = ((((uintptr_t)pg) & 15u) == (((uintptr_t)px) & 15u)) &&
                      ((((uintptr_t)pd) & 15u) == (((uintptr_t)px) & 15u));
     if (!vec) {
-      for (int64_t i = tid; i < HW; i += kBnBlock) pd[i] = one(px[i], pg[i]);
+      for (int64_t i = tid; i < HW; i += kStep) pd[i] = one(px[i], pg[i]);
       continue;
     }
     if (tid < sp.head) pd[tid] = one(px[tid], pg[tid]);
     const f32x4* px4 = reinterpret_cast<const f32x4*>(px + sp.head);
     const f32x4* pg4 = reinterpret_cast<const f32x4*>(pg + sp.head);
     f32x4* pd4 = reinterpret_cast<f32x4*>(pd + sp.head);
-    for (int64_t base = 0; base < sp.nvec; base += kBnBlock * kBnUnroll) {
+    for (int64_t base = 0; base < sp.nvec; base += kStep * kBnUnroll) {
       f32x4 vx[kBnUnroll], vg[kBnUnroll];
 #pragma unroll
       for (int u = 0; u < kBnUnroll; ++u) {
-        const int64_t i = base + u * kBnBlock + tid;
+        const int64_t i = base + u * kStep + tid;
         if (i < sp.nvec) {
           vx[u] = px4[i];
           vg[u] = pg4[i];
@@ -379,7 +386,7 @@ __global__ __launch_bounds__(kBnBlock) void bn_bwd_dx_kernel(const float* __rest
       }
 #pragma unroll
       for (int u = 0; u < kBnUnroll; ++u) {
-        const int64_t i = base + u * kBnBlock + tid;
+        const int64_t i = base + u * kStep + tid;
         if (i < sp.nvec) {
           f32x4 r;
           r.x = one(vx[u].x, vg[u].x);
@@ -400,9 +407,15 @@ __global__ __launch_bounds__(kBnBlock) void bn_bwd_dx_kernel(const float* __rest
 // Samples per workgroup: about `target` elements.  The fused passes use 8192;
 // the stand-alone statistics pass, whose workgroups end with a few dependent
 // atomics, is a little faster with twice that (fewer, longer workgroups).
+#ifndef TS_BN_STATS_TARGET
+#define TS_BN_STATS_TARGET 16384
+#endif
+#ifndef TS_BN_FWD_TARGET
+#define TS_BN_FWD_TARGET 8192
+#endif
 inline int64_t bn_slab(int64_t N, int64_t HW, int64_t target = 8192) {
   int64_t s = (target + HW - 1) / HW;
-  s += s & 1;  // planes are consumed in pairs
+  s = (s + 3) / 4 * 4;  // a wavefront per plane, four to a workgroup
   if (s < 1) s = 1;
   if (s > N) s = N;
   return s;
@@ -429,7 +442,7 @@ int ts_bn_stats(const float* x, int64_t N, int64_t C, int64_t HW, float* ws, flo
   if ((uintptr_t)x & 3u) return TS_ERR_ALIGN;
   hipStream_t st = (hipStream_t)stream;
   const float cnt = (float)((double)N * (double)HW);
-  const int64_t slab = ts::bn_slab(N, HW, 16384);
+  const int64_t slab = ts::bn_slab(N, HW, TS_BN_STATS_TARGET);
   dim3 grid((unsigned)((N + slab - 1) / slab), (unsigned)C);
   hipLaunchKernelGGL(ts::bn_stats_kernel<true>, grid, dim3(ts::kBnBlock), 0, st, x, N, C, HW, slab,
                      cnt, ws, sum, sum_squares, ub_mean, ub_invstd, eps);

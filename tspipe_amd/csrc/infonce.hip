@@ -726,7 +726,10 @@ __device__ __forceinline__ void nce_loss_block(const NceArgs& args, int pairs, i
   }
 }
 
-template <typename T, int C, bool HP>
+// SC: key splits whose partial sums a thread requests in one go (2, 4 or 8,
+// the smallest that covers the launch's split count, more come in further
+// rounds); slots beyond the split count re-read a valid split and are dropped.
+template <typename T, int C, bool HP, int SC>
 __global__ __launch_bounds__(2 * C) void nce_combine_kernel(NceArgs args, int64_t n, int64_t npad, int splits,
                                                             float loss_scale, float* __restrict__ loss_out,
                                                             int xcd_map) {
@@ -780,7 +783,6 @@ __global__ __launch_bounds__(2 * C) void nce_combine_kernel(NceArgs args, int64_
   float l = 0.f;
   const int64_t blk = (tile32 * 2 + a) * FBH + fbl;                // 32-feature blocks in front, within a split
   const int64_t split_blocks = (npad / 32) * 2 * FBH;              // 32-feature blocks per split
-  constexpr int SC = 8;
   for (int s0 = 0; s0 < splits; s0 += SC) {
     float lv[SC];
     f32x4 vf[SC][2];
@@ -865,8 +867,16 @@ int nce_run(const NceArgs& args, int pairs, int64_t n, float tau, const NceLayou
   rc = check_launch();
   if (rc) return rc;
   const int xcd_map = qtile_major && (L.npad / kQTile) % 8 == 0 ? 1 : 0;
-  hipLaunchKernelGGL((nce_combine_kernel<T, C, HP>), dim3((unsigned)(L.npad / 16 + 8), 1, z), dim3(2 * C), 0, stream,
-                     args, n, L.npad, L.splits, 2.f * tau, loss_out, xcd_map);
+  const dim3 cgrid((unsigned)(L.npad / 16 + 8), 1, z);
+  if (L.splits <= 2)
+    hipLaunchKernelGGL((nce_combine_kernel<T, C, HP, 2>), cgrid, dim3(2 * C), 0, stream, args, n, L.npad, L.splits,
+                       2.f * tau, loss_out, xcd_map);
+  else if (L.splits <= 4)
+    hipLaunchKernelGGL((nce_combine_kernel<T, C, HP, 4>), cgrid, dim3(2 * C), 0, stream, args, n, L.npad, L.splits,
+                       2.f * tau, loss_out, xcd_map);
+  else
+    hipLaunchKernelGGL((nce_combine_kernel<T, C, HP, 8>), cgrid, dim3(2 * C), 0, stream, args, n, L.npad, L.splits,
+                       2.f * tau, loss_out, xcd_map);
   return check_launch();
 }
 

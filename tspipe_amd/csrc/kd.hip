@@ -173,6 +173,7 @@ struct KdArgs {
   float kd_gscale;  // kd_scale * inv_T   (gradient factor of the KD term before the 1/B)
   float ce_weight;
   const int* counts;  // device: [0] KD rows, [1] CE rows, [2] rows with any term; null = all n_rows carry KD only
+  int self_count;     // counts is null although a mask selects rows: whoever needs the number of KD rows counts the mask bytes
   float* row_kd;      // per-row KD loss terms (0 for unselected rows)
   float* row_ce;      // per-row CE loss terms
   void* grad;         // may be null
@@ -239,6 +240,29 @@ __device__ __forceinline__ RowJob row_job(const KdArgs& a, int64_t row) {
   return j;
 }
 
+// Number of non-zero mask bytes, counted by the calling workgroup (every
+// thread gets the result; `lds` holds NT / 64 floats).  The mask of a batch is
+// a few kilobytes, so this is an L2-resident read and one block reduction --
+// cheaper than a counting launch in front when only the workgroups of the
+// selected rows need the number.
+template <int NT>
+__device__ __forceinline__ float kd_mask_count(const uint8_t* __restrict__ mask, int64_t n, float* lds) {
+  int c = 0;
+  const int64_t n8 = ((uintptr_t)mask & 7u) == 0 ? n / 8 : 0;
+  const uint64_t* m8 = reinterpret_cast<const uint64_t*>(mask);
+  for (int64_t i = threadIdx.x; i < n8; i += NT) {
+    uint64_t v = m8[i];
+    // a byte counts when any of its bits is set
+    v |= v >> 4;
+    v |= v >> 2;
+    v |= v >> 1;
+    c += __popcll(v & 0x0101010101010101ull);
+  }
+  for (int64_t i = n8 * 8 + threadIdx.x; i < n; i += NT) c += mask[i] != 0;
+  // per-thread counts stay far below 2^24 for any n the launchers accept: the float sum is exact
+  return block_sum<NT / kWave>((float)c, lds);
+}
+
 // Final per-row numbers from the merged states.
 struct RowFinal {
   float lse_t, lse_s, lse1;  // log2 domain
@@ -247,12 +271,12 @@ struct RowFinal {
 
 template <typename T, bool CE>
 __device__ __forceinline__ RowFinal finish_row(const KdArgs& a, const RowJob& j, int64_t row, const TStat& st,
-                                               const SStat& ss, const T* srow, bool writer) {
+                                               const SStat& ss, const T* srow, bool writer, float n_kd_counted = 0.f) {
   RowFinal f;
   f.lse_t = st.m * a.k + log2f(st.z);
   f.lse_s = ss.m * a.k + log2f(ss.z);
   f.lse1 = CE ? ss.m * kLog2e + log2f(ss.z1) : 0.f;
-  const float n_kd = a.counts ? (float)a.counts[0] : (float)a.n_rows;
+  const float n_kd = a.self_count ? n_kd_counted : (a.counts ? (float)a.counts[0] : (float)a.n_rows);
   f.g_kd = j.kd ? a.kd_gscale / n_kd : 0.f;
   f.g_ce = (CE && j.ce) ? a.ce_weight / (float)a.counts[1] : 0.f;
   if (writer) {
@@ -323,25 +347,32 @@ __global__ __launch_bounds__(BLOCK, (KREG * GROUP > 1024 ? 4 : 1)) void kd_rows_
   constexpr int NW = GROUP / kWave;  // wavefronts per group (0 for sub-wavefront groups)
   __shared__ TStat lds_t[BLOCK / kWave];
   __shared__ SStat lds_s[BLOCK / kWave];
+  __shared__ float lds_cnt[BLOCK / kWave];
 
   const int gtid = threadIdx.x % GROUP;
   int64_t row = (int64_t)blockIdx.x * (BLOCK / GROUP) + threadIdx.x / GROUP;
   // With GROUP == BLOCK the whole workgroup shares one row, so the early
   // exits below are uniform; smaller groups never reach a __syncthreads and
   // only shuffle among their own lanes.
-  if (sel_rows) {
+  if (sel_rows || a.self_count) {
     // Masked long rows (one row per workgroup, grid of 2 n_rows): the first
-    // n_rows workgroups walk the compacted list of the rows that carry a loss
-    // term, so that the long-running ones all start first; the next n_rows
-    // zero-fill the rows that carry none.  (Interleaving the two kinds, singly
-    // or in runs of eight, was measured slower than this order.)
+    // n_rows workgroups take the rows that carry a loss term, so that the
+    // long-running ones all start first; the next n_rows zero-fill the rows
+    // that carry none.  (Interleaving the two kinds, singly or in runs of
+    // eight, was measured slower than this order.)  With a compacted row list
+    // (built by the counting launch, which a cross-entropy term needs anyway)
+    // workgroup i of the first half takes the i-th such row; without one it
+    // takes row i if that carries a term and ends at once otherwise.
     if (row >= a.n_rows) {
       row -= a.n_rows;
       const RowJob j0 = row_job(a, row);
       if (j0.kd || j0.ce) return;
-    } else {
+    } else if (sel_rows) {
       if (row >= a.counts[2]) return;
       row = sel_rows[row];
+    } else {
+      const RowJob j0 = row_job(a, row);
+      if (!j0.kd && !j0.ce) return;
     }
   }
   if (row >= a.n_rows) return;
@@ -371,6 +402,12 @@ __global__ __launch_bounds__(BLOCK, (KREG * GROUP > 1024 ? 4 : 1)) void kd_rows_
       rs[j] = load16(srow + g.head + v * VEC);
     }
   }
+  // No counting launch ran in front (mask-only call on long rows): the number
+  // of selected rows, which scales the gradient, is counted here while the
+  // row's loads are in flight.  One row per workgroup in that case, so the
+  // branch is uniform.
+  float n_kd_counted = 0.f;
+  if (GROUP == BLOCK && a.self_count) n_kd_counted = kd_mask_count<BLOCK>(a.mask, a.n_rows, lds_cnt);
 
   // Rows whose operands share one alignment (the usual case): all but a few
   // end elements are 16-byte vectors held in registers, and each of those end
@@ -481,7 +518,7 @@ __global__ __launch_bounds__(BLOCK, (KREG * GROUP > 1024 ? 4 : 1)) void kd_rows_
       }
     }
     const RowFinal f =
-        finish_row<T, CE>(a, job, row, TStat{mt, zt, at}, SStat{ms, zs, z1}, srow, gtid == 0);
+        finish_row<T, CE>(a, job, row, TStat{mt, zt, at}, SStat{ms, zs, z1}, srow, gtid == 0, n_kd_counted);
     if (!grow) return;
     // probabilities first and the weight last, as everywhere in this file
     const float rt_ = 1.f / zt, rs_ = 1.f / zs, r1_ = CE ? 1.f / z1 : 0.f;
@@ -559,7 +596,7 @@ __global__ __launch_bounds__(BLOCK, (KREG * GROUP > 1024 ? 4 : 1)) void kd_rows_
     }
   }
 
-  const RowFinal f = finish_row<T, CE>(a, job, row, st, ss, srow, gtid == 0);
+  const RowFinal f = finish_row<T, CE>(a, job, row, st, ss, srow, gtid == 0, n_kd_counted);
   if (!grow) return;
 
   for (int64_t i = gtid; i < g.head; i += GROUP) grow[i] = grad_one<T, CE>(trow[i], srow[i], i == job.label, a.k, f);
@@ -894,9 +931,11 @@ __global__ __launch_bounds__(1024) void kd_count_kernel(const KdArgs a, int* __r
 __global__ __launch_bounds__(1024) void kd_finalize_kernel(const float* __restrict__ row_kd,
                                                            const float* __restrict__ row_ce, int64_t n,
                                                            float kd_scale, float ce_weight,
-                                                           const int* __restrict__ counts /* null: n KD rows */,
+                                                           const int* __restrict__ counts /* null: n KD rows ... */,
+                                                           const uint8_t* __restrict__ mask /* ... or, if set, the rows it selects */,
                                                            float* __restrict__ out) {
   __shared__ float lds[1024 / kWave];
+  const float n_masked = (!counts && mask) ? kd_mask_count<1024>(mask, n, lds) : 0.f;
   // 16-byte loads, four of them in flight per thread: one block has to get
   // through the whole array, so the loop is bound by memory latency
   const int64_t n4 = n / 4;
@@ -917,7 +956,7 @@ __global__ __launch_bounds__(1024) void kd_finalize_kernel(const float* __restri
   const float sce = block_sum<1024 / kWave>(ace, lds);
   if (threadIdx.x == 0) {
     // 0/0 = NaN for an empty selection, as the reference gives
-    float loss = kd_scale * (skd / (counts ? (float)counts[0] : (float)n));
+    float loss = kd_scale * (skd / (counts ? (float)counts[0] : (mask ? n_masked : (float)n)));
     if (row_ce) loss += ce_weight * (sce / (float)counts[1]);
     *out = loss;
   }
@@ -979,8 +1018,15 @@ int launch_kd_t(KdArgs a, float kd_scale, void* ws, float* loss_out, hipStream_t
   // most are.  The two passes remain for wider or differently aligned rows.
   const bool one_launch = a.n_rows > 0 && parts > 0 && vecs_ <= 1024 * 8 && kd_rows_aligned_alike<T>(a);
   const bool wide = a.n_rows > 0 && parts > 0 && !one_launch;
-  const bool compacted = one_launch && a.mask;  // the row kernel walks the compacted list, then zero-fills
-  if (counted && !wide) {
+  // A mask without labels on such rows needs no launch in front: the only
+  // number the row kernel wants, the count of selected rows, each of its
+  // workgroups takes from the mask itself (a few kilobytes), and so does the
+  // final reduction.
+  const bool self_count = one_launch && a.mask && !a.labels;
+  const bool compacted = one_launch && a.mask && !self_count;  // the row kernel walks the compacted list, then zero-fills
+  a.self_count = self_count ? 1 : 0;
+  if (self_count) a.counts = nullptr;
+  if (counted && !wide && !self_count) {
     hipLaunchKernelGGL(kd_count_kernel, dim3(1), dim3(1024), 0, stream, a, w.counts,
                        (compact || compacted) ? w.sel_rows : (int*)nullptr);
     rc = check_launch();
@@ -988,7 +1034,8 @@ int launch_kd_t(KdArgs a, float kd_scale, void* ws, float* loss_out, hipStream_t
   }
   if (a.n_rows == 0) {
     hipLaunchKernelGGL(kd_finalize_kernel, dim3(1), dim3(1024), 0, stream, w.row_kd,
-                       CE ? w.row_ce : (const float*)nullptr, (int64_t)0, kd_scale, a.ce_weight, a.counts, loss_out);
+                       CE ? w.row_ce : (const float*)nullptr, (int64_t)0, kd_scale, a.ce_weight, a.counts,
+                       (const uint8_t*)nullptr, loss_out);
     return check_launch();
   }
   // 16-byte vectors a row can span, counting a ragged first and last one
@@ -1007,7 +1054,7 @@ int launch_kd_t(KdArgs a, float kd_scale, void* ws, float* loss_out, hipStream_t
     TS_KD_LAUNCH(256, 256, 4);
   } else if (one_launch) {
     if (2 * a.n_rows > 0x7fffffffLL) return TS_ERR_RANGE;
-    const dim3 grid((unsigned)(compacted ? 2 * a.n_rows : a.n_rows));
+    const dim3 grid((unsigned)((compacted || self_count) ? 2 * a.n_rows : a.n_rows));
     const int* sel = compacted ? w.sel_rows : nullptr;
     if (vecs <= 512 * 8)
       hipLaunchKernelGGL((kd_rows_kernel<T, 512, 512, 8, CE>), grid, dim3(512), 0, stream, a, sel);
@@ -1029,7 +1076,7 @@ int launch_kd_t(KdArgs a, float kd_scale, void* ws, float* loss_out, hipStream_t
   rc = check_launch();
   if (rc) return rc;
   hipLaunchKernelGGL(kd_finalize_kernel, dim3(1), dim3(1024), 0, stream, w.row_kd, CE ? w.row_ce : (const float*)nullptr,
-                     a.n_rows, kd_scale, a.ce_weight, a.counts, loss_out);
+                     a.n_rows, kd_scale, a.ce_weight, a.counts, self_count ? a.mask : (const uint8_t*)nullptr, loss_out);
   return check_launch();
 }
 
@@ -1079,6 +1126,7 @@ int ts_kdce_fwd_bwd(const void* s, const void* t, const uint8_t* row_mask, const
   a.kd_gscale = kd_scale * inv_T;
   a.ce_weight = ce_weight;
   a.counts = nullptr;
+  a.self_count = 0;
   a.row_kd = a.row_ce = nullptr;
   a.grad = grad;
   a.n_pieces = 0;
@@ -1137,6 +1185,7 @@ int ts_kdce_pieces_fwd_bwd(const void* const* s_pieces, const void* const* t_pie
   a.kd_gscale = kd_scale * inv_T;
   a.ce_weight = ce_weight;
   a.counts = nullptr;
+  a.self_count = 0;
   a.row_kd = a.row_ce = nullptr;
   hipStream_t st = (hipStream_t)stream;
   switch (dtype) {
