@@ -60,15 +60,13 @@ __device__ __forceinline__ PlaneSplit split_plane(const float* p, int64_t HW) {
 // per lane, against 3.06 per thread of a 256-thread workgroup, whose fourth
 // load has 16 threads in it).  Four loads per lane and operand are in flight at
 // a time; more of them (8, 14: the whole plane) were measured slower.
-#ifndef TS_BN_WAVE_UNROLL
-#define TS_BN_WAVE_UNROLL 4
-#endif
-template <bool TWO, int BLOCK = 256, typename F>
+constexpr int kBnWaveLoads = 4;  // 16-byte loads per lane and operand in flight
+template <bool TWO, int BLOCK = kBnBlock, typename F>
 __device__ __forceinline__ void slab_reduce_waves(const float* __restrict__ x, const float* __restrict__ y, int64_t n0,
                                                   int64_t n1, int64_t C, int64_t c, int64_t HW, float& a, float& b,
                                                   F f) {
   constexpr int NW = BLOCK / kWave;
-  constexpr int U = TS_BN_WAVE_UNROLL;
+  constexpr int U = kBnWaveLoads;
   const int lane = threadIdx.x % kWave, w = threadIdx.x / kWave;
   for (int64_t n = n0 + w; n < n1; n += NW) {
     const int64_t off = (n * C + c) * HW;
@@ -407,15 +405,10 @@ __global__ __launch_bounds__(kBnBlock) void bn_bwd_dx_kernel(const float* __rest
 // Samples per workgroup: about `target` elements.  The fused passes use 8192;
 // the stand-alone statistics pass, whose workgroups end with a few dependent
 // atomics, is a little faster with twice that (fewer, longer workgroups).
-#ifndef TS_BN_STATS_TARGET
-#define TS_BN_STATS_TARGET 16384
-#endif
-#ifndef TS_BN_FWD_TARGET
-#define TS_BN_FWD_TARGET 8192
-#endif
 inline int64_t bn_slab(int64_t N, int64_t HW, int64_t target = 8192) {
   int64_t s = (target + HW - 1) / HW;
-  s = (s + 3) / 4 * 4;  // a wavefront per plane, four to a workgroup
+  constexpr int64_t kw = kBnBlock / kWave;
+  s = (s + kw - 1) / kw * kw;  // a wavefront per plane
   if (s < 1) s = 1;
   if (s > N) s = N;
   return s;
@@ -442,7 +435,7 @@ int ts_bn_stats(const float* x, int64_t N, int64_t C, int64_t HW, float* ws, flo
   if ((uintptr_t)x & 3u) return TS_ERR_ALIGN;
   hipStream_t st = (hipStream_t)stream;
   const float cnt = (float)((double)N * (double)HW);
-  const int64_t slab = ts::bn_slab(N, HW, TS_BN_STATS_TARGET);
+  const int64_t slab = ts::bn_slab(N, HW, 16384);
   dim3 grid((unsigned)((N + slab - 1) / slab), (unsigned)C);
   hipLaunchKernelGGL(ts::bn_stats_kernel<true>, grid, dim3(ts::kBnBlock), 0, st, x, N, C, HW, slab,
                      cnt, ws, sum, sum_squares, ub_mean, ub_invstd, eps);

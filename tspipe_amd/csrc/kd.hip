@@ -936,16 +936,30 @@ __global__ __launch_bounds__(1024) void kd_finalize_kernel(const float* __restri
                                                            float* __restrict__ out) {
   __shared__ float lds[1024 / kWave];
   const float n_masked = (!counts && mask) ? kd_mask_count<1024>(mask, n, lds) : 0.f;
-  // 16-byte loads, four of them in flight per thread: one block has to get
-  // through the whole array, so the loop is bound by memory latency
+  // 16-byte loads, eight of them in flight per thread and array: one block
+  // has to get through the whole array, so the loop is bound by memory latency
+  // (65536 rows are two round trips this way)
   const int64_t n4 = n / 4;
   const f32x4* kd4 = reinterpret_cast<const f32x4*>(row_kd);
   const f32x4* ce4 = reinterpret_cast<const f32x4*>(row_ce);
   f32x4 vkd = {0.f, 0.f, 0.f, 0.f}, vce = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll 4
-  for (int64_t i = threadIdx.x; i < n4; i += 1024) {
-    vkd += kd4[i];
-    if (row_ce) vce += ce4[i];
+  constexpr int kInFlight = 8;
+  for (int64_t i0 = threadIdx.x; i0 < n4; i0 += 1024 * kInFlight) {
+    f32x4 a[kInFlight], c[kInFlight];
+#pragma unroll
+    for (int j = 0; j < kInFlight; ++j) {
+      const int64_t i = i0 + (int64_t)j * 1024;
+      a[j] = c[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+      if (i < n4) {
+        a[j] = kd4[i];
+        if (row_ce) c[j] = ce4[i];
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < kInFlight; ++j) {
+      vkd += a[j];
+      vce += c[j];
+    }
   }
   float akd = (vkd[0] + vkd[1]) + (vkd[2] + vkd[3]), ace = (vce[0] + vce[1]) + (vce[2] + vce[3]);
   for (int64_t i = n4 * 4 + threadIdx.x; i < n; i += 1024) {
