@@ -37,6 +37,7 @@ TIMED_EVERY = 4  # one EMA launch in four carries kernel timing events
 SETUP_STEPS = 12  # untimed calls before the warm-up steps (resource creation, see run_step_benchmark)
 HBM_PEAK_GBS = 8000.0       # MI355X published HBM3E bandwidth
 MFMA_BF16_PEAK_TFLOPS = 2500.0
+MFMA_F32_PEAK_TFLOPS = 157.3
 TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "hbm_traffic_pmc_all_kernels.md")
 
 
@@ -505,8 +506,8 @@ def run_kernel_table(dev, with_cpu=True):
 
     # InfoNCE: cfg4 (single pair), the symmetric two-pair call of MoCo-v3's contrastive_loss, and a
     # batch four times as large, where the fixed costs of the three launches weigh less
-    def nce_entry(name, n, pairs, note=None):
-        mk = lambda: torch.nn.functional.normalize(torch.randn(n, 256, generator=g), dim=1).to(torch.bfloat16).to(dev)
+    def nce_entry(name, n, pairs, note=None, dtype=torch.bfloat16):
+        mk = lambda: torch.nn.functional.normalize(torch.randn(n, 256, generator=g), dim=1).to(dtype).to(dev)
         q1, k1 = mk(), mk()
         q2, k2 = (mk(), mk()) if pairs == 2 else (None, None)
         ws = torch.empty(lib.ts_infonce_workspace_bytes(n, 256, pairs), dtype=torch.uint8, device=dev)
@@ -516,12 +517,14 @@ def run_kernel_table(dev, with_cpu=True):
 
         def f():
             _lib.check(lib.ts_infonce_fwd_bwd(ptr(q1), ptr(k1), ptr(q2), ptr(k2), n, 256, 0.2, ws.data_ptr(),
-                                              loss.data_ptr(), ptr(d1), ptr(d2), _lib.TS_BF16, stream),
+                                              loss.data_ptr(), ptr(d1), ptr(d2), _lib.dtype_code(dtype), stream),
                        "ts_infonce_fwd_bwd")
         ms = _time_stream(f)
         flops = pairs * 2 * 2 * n * n * 256
+        peak_key, peak = (("frac_mfma_bf16_peak", MFMA_BF16_PEAK_TFLOPS) if dtype != torch.float32
+                          else ("frac_mfma_f32_peak", MFMA_F32_PEAK_TFLOPS))
         e = {"ms": round(ms, 4), "TFLOP/s": round(flops / (ms * 1e-3) / 1e12, 1),
-             "frac_mfma_bf16_peak": round(flops / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+             peak_key: round(flops / (ms * 1e-3) / 1e12 / peak, 4),
              "algorithmic_flop": flops, "kernel_launches": 3}
         if note:
             e["note"] = note
@@ -538,6 +541,9 @@ def run_kernel_table(dev, with_cpu=True):
     nce_entry("infonce_2_pairs_4096x256_bf16", 4096, 2, "both directions of the symmetric loss in one call")
     nce_entry("infonce_16384x256_bf16", 16384, 1,
               "not one of the benchmark configurations: the same kernels at 16x the work")
+    nce_entry("infonce_4096x256_f32", 4096, 1,
+              "fp32 embeddings (the reference's TSPipe MoCo run is fp32): fp32-MFMA kernels, every product and sum in "
+              "fp32; not one of the benchmark configurations", dtype=torch.float32)
 
     # BYOL loss (latency only)
     loss = torch.empty((), device=dev)

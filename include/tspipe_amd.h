@@ -384,8 +384,15 @@ int ts_infonce_pieces_fwd_bwd(const void* const* q1_pieces, const void* const* k
  *   - turned into ub_mean = S/cnt and ub_invstd = 1/sqrt(max(Q/cnt - mean^2,0)
  *     + eps), cnt = N*HW, unless those are NULL.
  * One launch: the last workgroup of a channel to finish does the channel's
- * bookkeeping.  ws: 3*C floats that are ZERO on entry (two sums and a ticket
- * counter per channel); the call leaves them zero again. */
+ * bookkeeping.  ws: ts_bn_stats_workspace_bytes(C) bytes (3*C floats: two
+ * sums and a ticket counter per channel) that are ZERO on entry; the call
+ * leaves them zero again.  Calls that share a ws must not overlap on the
+ * device (the last workgroup of a channel reads and clears what the others
+ * added): keep them on one stream, or order the streams with events.  A
+ * buffer of the 2*C floats that an earlier version of this call asked for is
+ * too small. */
+size_t ts_bn_stats_workspace_bytes(int64_t C);
+
 int ts_bn_stats(const float* x, int64_t N, int64_t C, int64_t HW, float* ws, float* sum,
                 float* sum_squares, float* ub_mean, float* ub_invstd, float eps,
                 ts_stream_t stream);

@@ -64,6 +64,7 @@ SIGNATURES = {
                                    c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
     "ts_infonce_pieces_fwd_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                                           c_int64, c_float, c_void_p, c_void_p, c_int, c_void_p]),
+    "ts_bn_stats_workspace_bytes": (c_size_t, [c_int64]),
     "ts_bn_stats": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_void_p,
                             c_void_p, c_float, c_void_p]),
     "ts_bn_commit": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_double,

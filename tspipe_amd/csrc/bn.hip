@@ -425,6 +425,8 @@ inline int bn_check_dims(int64_t N, int64_t C, int64_t HW) {
 
 extern "C" {
 
+size_t ts_bn_stats_workspace_bytes(int64_t C) { return C > 0 ? (size_t)C * 3 * sizeof(float) : 0; }
+
 int ts_bn_stats(const float* x, int64_t N, int64_t C, int64_t HW, float* ws, float* sum,
                 float* sum_squares, float* ub_mean, float* ub_invstd, float eps, ts_stream_t stream) {
   if (!x || !ws) return TS_ERR_ARG;

@@ -29,8 +29,9 @@
 //            reads are free of bank conflicts), two buffers.  A wavefront
 //            accumulates O^T for FBW 32-feature blocks; widths above 256
 //            are covered by several feature groups, each recomputing S.
-//   combine  one wavefront per row: merges the key splits, forms dq; one more
-//            workgroup adds up the loss.
+//   combine  one wavefront per row: merges the key splits, forms dq, leaves the
+//            row's loss term.
+//   sum      one workgroup adds up the loss terms in a fixed order.
 //
 // MFMA 32x32x2 operand layout (lane l, half h = l/32):
 //   A: row l%32, contraction slot h;  B: column l%32, slot h;
@@ -48,6 +49,7 @@ struct NceGenLayout {
   int64_t npad;
   int splits, cp;
   size_t head_bytes, off_rq, off_rk, off_stat, off_opart, pair_bytes;
+  size_t rowloss_bytes;  // behind the pairs' regions: [pairs][npad] per-row loss terms, summed by the last launch
 };
 
 inline int nce_gen_cp(int64_t c) { return c <= 64 ? 64 : (c <= 128 ? 128 : (c <= 256 ? 256 : 512)); }
@@ -76,8 +78,12 @@ inline NceGenLayout nce_gen_layout(int64_t n, int64_t c, int n_pairs) {
   L.off_stat = o;   o += nce_align((size_t)L.splits * L.npad * 16);
   L.off_opart = o;  o += nce_align((size_t)L.splits * L.npad * L.cp * 4);
   L.pair_bytes = o;
+  L.rowloss_bytes = nce_align((size_t)n_pairs * L.npad * 4);
   return L;
 }
+
+// defined in losses.hip
+int launch_sum_scale(const float* v, int64_t n, float scale, float denom, float* out, hipStream_t stream);
 
 // ---------------------------------------------------------------------------
 // norm: one wavefront per row
@@ -323,79 +329,83 @@ __global__ __launch_bounds__(kGenBlock) void nce_gen_main_kernel(NceArgs args, i
 //   l_neg = sum_s w_s l_neg,s   p = sum_s w_s p_s   l = l_neg + p
 //   O'    = sum_s w_s O'_s
 //   dqh   = (2/N) [ O'/l - (l_neg/l) kh_i ]
-// The last workgroup of the grid (pair 0 only) adds up the loss over all pairs,
-//   loss = loss_scale / n * sum_i ln2 (M_i + log2 l_i - s_ii),
-// in a fixed order.
+// Every row also leaves its loss term ln2 (M_i + log2 l_i - s_ii); a last,
+// single-workgroup launch adds them up in a fixed order
+//   loss = loss_scale / n * sum over pairs and rows.
 // ---------------------------------------------------------------------------
 struct NceGenRowStat {
   float M, lneg, p, sdiag;
 };
 
+constexpr int kGenMaxSplits = 16;  // nce_gen_splits never asks for more
+
+// Every split's record of the row is requested before the first is used.
 __device__ __forceinline__ NceGenRowStat nce_gen_merge(const float* stat, int64_t row, int64_t npad, int splits) {
+  f32x4 v[kGenMaxSplits];
+#pragma unroll
+  for (int s = 0; s < kGenMaxSplits; ++s)
+    v[s] = s < splits ? *reinterpret_cast<const f32x4*>(stat + ((int64_t)s * npad + row) * 4)
+                      : f32x4{kGenFloor, 0.f, 0.f, -INFINITY};
   float M = kGenFloor;
-  for (int s = 0; s < splits; ++s) M = fmaxf(M, stat[((int64_t)s * npad + row) * 4]);
+#pragma unroll
+  for (int s = 0; s < kGenMaxSplits; ++s) M = fmaxf(M, v[s][0]);
   NceGenRowStat r{M, 0.f, 0.f, -INFINITY};
-  for (int s = 0; s < splits; ++s) {
-    const f32x4 v = *reinterpret_cast<const f32x4*>(stat + ((int64_t)s * npad + row) * 4);
-    const float wgt = fast_exp2(v[0] - M);
-    r.lneg = fmaf(wgt, v[1], r.lneg);
-    r.p = fmaf(wgt, v[2], r.p);
-    r.sdiag = fmaxf(r.sdiag, v[3]);
+#pragma unroll
+  for (int s = 0; s < kGenMaxSplits; ++s) {
+    const float wgt = fast_exp2(v[s][0] - M);
+    r.lneg = fmaf(wgt, v[s][1], r.lneg);
+    r.p = fmaf(wgt, v[s][2], r.p);
+    r.sdiag = fmaxf(r.sdiag, v[s][3]);
   }
   return r;
 }
 
 template <typename T>
 __global__ __launch_bounds__(kGenBlock) void nce_gen_combine_kernel(NceArgs args, int64_t n, int64_t npad, int c, int cp,
-                                                                    int splits, float loss_scale,
-                                                                    float* __restrict__ loss_out) {
-  __shared__ float red[kGenBlock / kWave];
-  const int tid = threadIdx.x, lane = tid % kWave, w = tid / kWave;
-  const int64_t row_blocks = (n + kGenBlock / kWave - 1) / (kGenBlock / kWave);
-  if ((int64_t)blockIdx.x >= row_blocks) {
-    if (blockIdx.z != 0) return;
-    float acc = 0.f;
-    for (int p = 0; p < (int)gridDim.z; ++p)
-      for (int64_t row = tid; row < n; row += kGenBlock) {
-        const NceGenRowStat r = nce_gen_merge(args.p[p].stat, row, npad, splits);
-        acc += kNceLn2 * (r.M + log2f(r.lneg + r.p) - r.sdiag);
-      }
-    acc = wave_sum(acc);
-    if (lane == 0) red[w] = acc;
-    __syncthreads();
-    if (tid == 0) {
-      float total = 0.f;
-#pragma unroll
-      for (int i = 0; i < kGenBlock / kWave; ++i) total += red[i];
-      *loss_out = total * loss_scale / (float)n;
-    }
-    return;
-  }
+                                                                    int splits, float* __restrict__ rowloss) {
+  const int lane = threadIdx.x % kWave, w = threadIdx.x / kWave;
   const NcePair& pr = args.p[blockIdx.z];
   const int64_t row = (int64_t)blockIdx.x * (kGenBlock / kWave) + w;
-  if (row >= n) return;
+  if (row >= npad) return;
+  float* const my_loss = rowloss + (int64_t)blockIdx.z * npad + row;
+  if (row >= n) {  // padding rows add nothing to the sum
+    if (lane == 0) *my_loss = 0.f;
+    return;
+  }
   const NceRow rp = nce_row<T>(pr, row, c);
-  if (!rp.dq) return;
   const NceGenRowStat r = nce_gen_merge(pr.stat, row, npad, splits);
+  if (lane == 0) *my_loss = kNceLn2 * (r.M + log2f(r.lneg + r.p) - r.sdiag);
+  if (!rp.dq) return;
   const float l = r.lneg + r.p;
   const float inv_l = 1.f / l, w_neg = r.lneg * inv_l;
   const float rq_i = pr.rq[row], rk_i = pr.rk[row];
   const float gn = 2.f / (float)n;
   constexpr int MAXF = 512 / kWave;
+  constexpr int kMaxSplits = kGenMaxSplits;
+  // the splits' weights once, then every partial sum of the row requested before the first is used
+  float wgt[kMaxSplits];
+#pragma unroll
+  for (int s = 0; s < kMaxSplits; ++s)
+    wgt[s] = s < splits ? fast_exp2(pr.stat[((int64_t)s * npad + row) * 4] - r.M) : 0.f;
   float dqh[MAXF], qh[MAXF];
   float dot = 0.f;
 #pragma unroll
   for (int u = 0; u < MAXF; ++u) {
     const int f = u * kWave + lane;
     dqh[u] = qh[u] = 0.f;
-    if (f < c) {
+    if (u * kWave < c) {  // uniform
+      const bool live = f < c;
+      float part[kMaxSplits];
+#pragma unroll
+      for (int s = 0; s < kMaxSplits; ++s)
+        part[s] = (live && s < splits) ? pr.opart[((int64_t)s * npad + row) * cp + f] : 0.f;
+      const float kv = live ? to_f32(((const T*)rp.k)[f]) : 0.f;
+      const float qv = live ? to_f32(((const T*)rp.q)[f]) : 0.f;
       float o = 0.f;
-      for (int s = 0; s < splits; ++s) {
-        const float wgt = fast_exp2(pr.stat[((int64_t)s * npad + row) * 4] - r.M);
-        o = fmaf(wgt, pr.opart[((int64_t)s * npad + row) * cp + f], o);
-      }
-      dqh[u] = gn * (o * inv_l - w_neg * (to_f32(((const T*)rp.k)[f]) * rk_i));
-      qh[u] = to_f32(((const T*)rp.q)[f]) * rq_i;
+#pragma unroll
+      for (int s = 0; s < kMaxSplits; ++s) o = fmaf(wgt[s], part[s], o);
+      dqh[u] = gn * (o * inv_l - w_neg * (kv * rk_i));
+      qh[u] = qv * rq_i;
       dot = fmaf(qh[u], dqh[u], dot);
     }
   }
@@ -410,8 +420,8 @@ __global__ __launch_bounds__(kGenBlock) void nce_gen_combine_kernel(NceArgs args
 }
 
 template <typename T, int CP, int FBW>
-int nce_gen_run(const NceArgs& args, int pairs, int64_t n, int c, float tau, const NceGenLayout& L, float* loss_out,
-                bool vec, hipStream_t stream) {
+int nce_gen_run(const NceArgs& args, int pairs, int64_t n, int c, float tau, const NceGenLayout& L, float* rowloss,
+                float* loss_out, bool vec, hipStream_t stream) {
   constexpr int FG = CP / 32 / FBW;
   const unsigned wave_rows = kGenBlock / kWave;
   hipLaunchKernelGGL((nce_gen_norm_kernel<T>), dim3((unsigned)((L.npad + wave_rows - 1) / wave_rows), 1, (unsigned)pairs),
@@ -423,25 +433,27 @@ int nce_gen_run(const NceArgs& args, int pairs, int64_t n, int c, float tau, con
                      stream, args, n, L.npad, c, L.splits, kNceLog2e / tau, vec ? 1 : 0);
   rc = check_launch();
   if (rc) return rc;
-  hipLaunchKernelGGL((nce_gen_combine_kernel<T>), dim3((unsigned)((n + wave_rows - 1) / wave_rows + 1), 1, (unsigned)pairs),
-                     dim3(kGenBlock), 0, stream, args, n, L.npad, c, CP, L.splits, 2.f * tau, loss_out);
-  return check_launch();
+  hipLaunchKernelGGL((nce_gen_combine_kernel<T>), dim3((unsigned)(L.npad / wave_rows), 1, (unsigned)pairs),
+                     dim3(kGenBlock), 0, stream, args, n, L.npad, c, CP, L.splits, rowloss);
+  rc = check_launch();
+  if (rc) return rc;
+  return launch_sum_scale(rowloss, (int64_t)pairs * L.npad, 2.f * tau, (float)n, loss_out, stream);
 }
 
 template <typename T>
-int nce_gen_dispatch(const NceArgs& args, int pairs, int64_t n, int c, float tau, const NceGenLayout& L, float* loss_out,
-                     bool vec, hipStream_t stream) {
+int nce_gen_dispatch(const NceArgs& args, int pairs, int64_t n, int c, float tau, const NceGenLayout& L, float* rowloss,
+                     float* loss_out, bool vec, hipStream_t stream) {
   switch (L.cp) {
-    case 64: return nce_gen_run<T, 64, 2>(args, pairs, n, c, tau, L, loss_out, vec, stream);
-    case 128: return nce_gen_run<T, 128, 4>(args, pairs, n, c, tau, L, loss_out, vec, stream);
-    case 256: return nce_gen_run<T, 256, 8>(args, pairs, n, c, tau, L, loss_out, vec, stream);
-    default: return nce_gen_run<T, 512, 4>(args, pairs, n, c, tau, L, loss_out, vec, stream);
+    case 64: return nce_gen_run<T, 64, 2>(args, pairs, n, c, tau, L, rowloss, loss_out, vec, stream);
+    case 128: return nce_gen_run<T, 128, 4>(args, pairs, n, c, tau, L, rowloss, loss_out, vec, stream);
+    case 256: return nce_gen_run<T, 256, 8>(args, pairs, n, c, tau, L, rowloss, loss_out, vec, stream);
+    default: return nce_gen_run<T, 512, 4>(args, pairs, n, c, tau, L, rowloss, loss_out, vec, stream);
   }
 }
 
 size_t nce_general_workspace_bytes(int64_t n, int64_t c, int n_pairs) {
   const NceGenLayout L = nce_gen_layout(n, c, n_pairs);
-  return L.head_bytes + L.pair_bytes * (size_t)n_pairs;
+  return L.head_bytes + L.pair_bytes * (size_t)n_pairs + L.rowloss_bytes;
 }
 
 int nce_general_launch(NceArgs& args, int pairs, int64_t n, int64_t c, float tau, void* workspace, float* loss_out,
@@ -468,9 +480,10 @@ int nce_general_launch(NceArgs& args, int pairs, int64_t n, int64_t c, float tau
     if (bits & (4 * esz - 1)) vec = false;
   }
   const int ci = (int)c;
-  if (dtype == TS_F32) return nce_gen_dispatch<float>(args, pairs, n, ci, tau, L, loss_out, vec, stream);
-  if (dtype == TS_F16) return nce_gen_dispatch<f16_t>(args, pairs, n, ci, tau, L, loss_out, vec, stream);
-  return nce_gen_dispatch<bf16_t>(args, pairs, n, ci, tau, L, loss_out, vec, stream);
+  float* rowloss = (float*)(ws + L.head_bytes + (size_t)pairs * L.pair_bytes);
+  if (dtype == TS_F32) return nce_gen_dispatch<float>(args, pairs, n, ci, tau, L, rowloss, loss_out, vec, stream);
+  if (dtype == TS_F16) return nce_gen_dispatch<f16_t>(args, pairs, n, ci, tau, L, rowloss, loss_out, vec, stream);
+  return nce_gen_dispatch<bf16_t>(args, pairs, n, ci, tau, L, rowloss, loss_out, vec, stream);
 }
 
 }  // namespace ts
