@@ -41,18 +41,22 @@ MFMA_F32_PEAK_TFLOPS = 157.3
 TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "hbm_traffic_pmc_all_kernels.md")
 
 
-def _ema_traffic_bytes():
-    """HBM bytes one ViT-B EMA launch moves, read from the committed rocprofv3
-    --pmc summary (FETCH_SIZE and WRITE_SIZE runs scaled by the same counters
-    on a copy of known size); None when the summary is not in the tree.  The
-    value is a record of those profiler runs, not a product of this run."""
+def _ema_traffic():
+    """(bytes, commit): HBM bytes one ViT-B EMA launch moves, read from the
+    committed rocprofv3 --pmc summary (FETCH_SIZE and WRITE_SIZE runs scaled by
+    the same counters on a copy of known size), and the commit those runs were
+    made on; (None, None) when the summary is not in the tree.  The value is a
+    record of those profiler runs, not a product of this run."""
+    nbytes = commit = None
     try:
         for line in open(TRAFFIC_SUMMARY):
             if line.startswith("bench.py roofline.traffic"):
-                return float(line.split("=")[1].split()[0])
+                nbytes = float(line.split("=")[1].split()[0])
+            elif line.startswith("collected on commit"):
+                commit = line.split()[3]
     except OSError:
         pass
-    return None
+    return nbytes, commit
 
 
 def _shapes():
@@ -218,7 +222,7 @@ def run_step_benchmark(steps, warmup, dev):
         "elapsed": elapsed, "n_params": n_params, "loss": float(state["loss"].item()), "host": host_ms,
         "roofline": {"bound": "hbm", "kernel": "ema_multi_kernel", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": _ema_traffic_bytes(),
+                     "traffic": _ema_traffic()[0], "traffic_commit": _ema_traffic()[1],
                      "traffic_source": "profiles/hbm_traffic_pmc_all_kernels.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
                                        "runs of this script, scaled by a copy of known size); not measured by this run",
                      "algorithmic_bytes_per_launch": algo_bytes,
@@ -261,7 +265,7 @@ TIMING_NOTE = ("ms: median over >=50 samples after >=10 warm-up calls; a sample 
                "`calls_per_sample` back-to-back calls, one per rotating buffer set (4 calls on the same buffers "
                "where the entry names no buffer sets)")
 MALL_BYTES = 256 << 20  # Infinity Cache: a working set below this is not an HBM measurement
-KD_MASKED_LAUNCHES = 3   # counting + compaction, row kernel (selected rows, then zero-fill), final reduction
+KD_MASKED_LAUNCHES = 2   # row kernel (selected rows and the zero-fill of the others), final reduction
 
 
 def _cpu_ms(fn, budget_s=1.2, max_iters=20):
@@ -434,7 +438,7 @@ def run_kernel_table(dev, with_cpu=True):
         return fns
     fns = kd_sets(65536, 100, 8)
     one = 3 * 65536 * 100 * 4
-    out["kd_65536x100_f32"] = entry(one, _time_stream(rotate(fns), batch=8), None, 1, working_set=8 * one, sets=8,
+    out["kd_65536x100_f32"] = entry(one, _time_stream(rotate(fns), batch=8), None, 2, working_set=8 * one, sets=8,
                                     resident_ms=_time_stream(fns[0]))
     cpu("kd_65536x100_f32", kd_cpu(*fns[0].operands, 4.0))
     del fns
@@ -442,7 +446,7 @@ def run_kernel_table(dev, with_cpu=True):
     # an ImageNet-sized class count (not one of the benchmark configurations): rows long enough to stream
     fns = kd_sets(32768, 1000, 2)
     one = 3 * 32768 * 1000 * 4
-    out["kd_32768x1000_f32"] = entry(one, _time_stream(rotate(fns), batch=2), "not one of the benchmark configurations", 1,
+    out["kd_32768x1000_f32"] = entry(one, _time_stream(rotate(fns), batch=2), "not one of the benchmark configurations", 2,
                                      working_set=2 * one, sets=2)
     cpu("kd_32768x1000_f32", kd_cpu(*fns[0].operands, 4.0))
     del fns, s, t, f

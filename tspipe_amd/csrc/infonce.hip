@@ -1,4 +1,7 @@
-// MoCo-v3 InfoNCE loss, forward and backward fused, on bf16 MFMA.
+// MoCo-v3 InfoNCE loss, forward and backward fused, on bf16 MFMA: the path
+// for bf16 / fp16 embeddings of 64, 128 or 256 features at tau >= 0.03.  fp32
+// embeddings, other widths and smaller temperatures run on the fp32 MFMA
+// kernels of infonce_general.hip.
 //
 //   qh = q/|q|, kh = k/|k|, logits = qh kh^T / tau,
 //   loss = 2 tau * mean_i( lse_i - logits_ii ),
@@ -14,7 +17,7 @@
 //     different key ranges just add up;
 //   * the keys are normalised in fp32 and rounded to bf16 once, by the prep
 //     kernel; the queries feed the MFMA as they are (bf16 inputs in place,
-//     fp32 / fp16 inputs through a bf16 copy) and their 1/|q| is applied as an
+//     fp16 inputs through a bf16 copy) and their 1/|q| is applied as an
 //     fp32 factor after the contraction (logit_ij = <q_i, kh_j> * rq_i / tau).
 //
 // Kernels:
@@ -111,7 +114,7 @@ inline NceLayout nce_layout(int64_t n, int64_t c, int n_pairs) {
   L.off_pdiag = o;    o += nce_align(L.npad * 8);
   L.off_lpart = o;    o += nce_align((size_t)L.splits * L.npad * 4);
   L.off_khat = o;     o += nce_align((size_t)L.npad * c * 2);
-  L.off_qb = o;       o += nce_align((size_t)L.npad * c * 2);  // used for fp32 / fp16 inputs only
+  L.off_qb = o;       o += nce_align((size_t)L.npad * c * 2);  // used for fp16 inputs only
   L.off_opart = o;    o += nce_align((size_t)L.splits * L.npad * c * 4);
   L.pair_bytes = o;
   return L;
@@ -860,7 +863,7 @@ int nce_run(const NceArgs& args, int pairs, int64_t n, float tau, const NceLayou
   const bool qtile_major = (size_t)L.npad * C * 2 <= ((size_t)4 << 20);
   const dim3 main_grid = qtile_major ? dim3((unsigned)(L.npad / kQTile), (unsigned)L.splits, z)
                                      : dim3((unsigned)L.splits, (unsigned)(L.npad / kQTile), z);
-  // fp32 inputs keep fp32 partial sums; the 2-byte types, whose gradient is rounded to 2^-9 anyway, bf16 ones
+  // the 2-byte types, whose gradient is rounded to 2^-9 anyway, keep bf16 partial sums
   constexpr bool HP = sizeof(T) == 2;
   hipLaunchKernelGGL((nce_main_kernel<C, HP>), main_grid, dim3(kNceMainBlock), 0, stream, args, n, L.npad, L.splits, scale2,
                      qtile_major ? 1 : 0);
@@ -907,11 +910,11 @@ int nce_launch(NceArgs& args, int pairs, int64_t n, int64_t c, float tau, void* 
     P.lpart = (float*)(wsp + L.off_lpart);
     P.opart = (float*)(wsp + L.off_opart);
     P.khat = (uint16_t*)(wsp + L.off_khat);
-    // fp32 and fp16 queries are rounded to a bf16 copy for the MFMA; bf16 ones are read in place
+    // fp16 queries are rounded to a bf16 copy for the MFMA; bf16 ones are read in place
     P.qb = dtype != TS_BF16 ? (uint16_t*)(wsp + L.off_qb) : nullptr;
   }
   // loss = 2 tau / n * sum over all pairs' rows, written by the combine launch
-  if (dtype == TS_F32) return nce_dispatch_c<float>(args, pairs, n, c, tau, L, loss_out, st);
+  if (dtype == TS_F32) return TS_ERR_ARG;  // fp32 embeddings never take this path (nce_bf16_path)
   if (dtype == TS_F16) return nce_dispatch_c<f16_t>(args, pairs, n, c, tau, L, loss_out, st);
   return nce_dispatch_c<bf16_t>(args, pairs, n, c, tau, L, loss_out, st);
 }
