@@ -33,6 +33,7 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
+STEP_NCE_WORKGROUPS = 32   # InfoNCE workgroup target inside the step: one key split, 32 long workgroups
 TIMED_EVERY = 4  # one EMA launch in four carries kernel timing events
 SETUP_STEPS = 12  # untimed calls before the warm-up steps (resource creation, see run_step_benchmark)
 HBM_PEAK_GBS = 8000.0       # MI355X published HBM3E bandwidth
@@ -529,7 +530,7 @@ def run_kernel_table(dev, with_cpu=True):
                           else ("frac_mfma_f32_peak", MFMA_F32_PEAK_TFLOPS))
         e = {"ms": round(ms, 4), "TFLOP/s": round(flops / (ms * 1e-3) / 1e12, 1),
              peak_key: round(flops / (ms * 1e-3) / 1e12 / peak, 4),
-             "algorithmic_flop": flops, "kernel_launches": 3}
+             "algorithmic_flop": flops, "kernel_launches": 3 if dtype != torch.float32 else 4}
         if note:
             e["note"] = note
         out[name] = e
@@ -719,6 +720,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel table")
+    ap.add_argument("--nce-workgroups", type=int, default=STEP_NCE_WORKGROUPS,
+                    help="workgroup target of the InfoNCE kernels inside the step (the kernel table uses the default, 256)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this build measures one GPU only; the kernel path has no cross-GPU exchange "
@@ -732,7 +735,13 @@ def main():
     from tspipe_amd import _lib
     _lib.lib()  # fail loudly if the HIP library is missing
 
+    # Inside the step the loss shares the GPU with the EMA stream: fewer, longer
+    # InfoNCE workgroups (less partial-sum traffic, CUs left to the EMA) make
+    # the step shorter although the loss kernel alone gets slower.
+    from tspipe_amd import set_infonce_workgroup_target
+    set_infonce_workgroup_target(args.nce_workgroups)
     res = run_step_benchmark(args.steps, args.warmup, dev)
+    set_infonce_workgroup_target(0)
     line = {
         "metric": "TS-steps/sec at ViT-B momentum (EMA over 86.6M fp32 params || InfoNCE 4096x256 bf16 fwd+bwd)",
         "value": round(args.steps / res["elapsed"], 2),
@@ -748,7 +757,8 @@ def main():
         "data": "synthetic",
         "config": {"workload": "MoCo-v3 ViT-Base step: fp32 EMA over ViT-B/16 shapes (152 tensors, 86,567,656 params, "
                                "m=0.99) + InfoNCE fwd+bwd on bf16 q,k 4096x256, tau=0.2, two HIP streams",
-                   "ema_tensors": 152, "ema_params": res["n_params"], "infonce_n": 4096, "infonce_c": 256},
+                   "ema_tensors": 152, "ema_params": res["n_params"], "infonce_n": 4096, "infonce_c": 256,
+                   "infonce_workgroup_target": args.nce_workgroups},
         "roofline": res["roofline"],
         "loss": res["loss"],
         "host": res["host"],

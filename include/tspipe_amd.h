@@ -349,6 +349,21 @@ int ts_cosine_pieces_fwd_bwd(const void* const* x_pieces, const void* const* y_p
 
 size_t ts_infonce_workspace_bytes(int64_t n, int64_t c, int n_pairs);
 
+/* No counterpart in the reference: a scheduling knob for callers that run the
+ * loss beside other GPU work, as TSPipe's pipeline does (the loss of one
+ * micro-batch beside the momentum update and the next forward,
+ * tspipe/gpu_task.py:385-410).  The main kernels cut the keys into as many
+ * splits as it takes to put about `workgroups` workgroups on the chip; every
+ * split writes partial sums that the last launch adds up.  The default, 256
+ * (one per CU), makes a call that has the GPU to itself fastest.  A smaller
+ * number means fewer, longer workgroups: fewer partial sums through HBM and
+ * CUs left to whatever runs on the other streams, at the price of a longer
+ * loss kernel.  Results agree to rounding (the partial sums are added in split
+ * order either way).  Process-wide; values outside 1..256 restore the default.
+ * Returns the previous value.  ts_infonce_workspace_bytes does not depend on
+ * it. */
+int ts_infonce_set_workgroup_target(int workgroups);
+
 int ts_infonce_fwd_bwd(const void* q1, const void* k1, const void* q2, const void* k2, int64_t n,
                        int64_t c, float tau, void* workspace, float* loss_out, void* dq1,
                        void* dq2, int dtype, ts_stream_t stream);

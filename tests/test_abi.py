@@ -177,6 +177,14 @@ def test_device_entry_points_validate_before_launching():
     assert lib.ts_infonce_fwd_bwd(p, p, None, None, 16, 64, 0.0, 0x1000, p, None, None, 1, None) == -1   # temperature
     assert lib.ts_infonce_fwd_bwd(p, p, None, None, 16, 64, 0.2, 0x1010, p, None, None, 1, None) == -4   # workspace alignment
     assert lib.ts_infonce_fwd_bwd(p, p, None, None, 16, 64, 0.2, 0x1000, p, None, None, 7, None) == -1   # dtype
+    # the scheduling knob: returns the previous value; out-of-range values restore the default; the workspace
+    # size does not follow it
+    ws_bytes = lib.ts_infonce_workspace_bytes(4096, 256, 1)
+    assert lib.ts_infonce_set_workgroup_target(32) == 256
+    assert lib.ts_infonce_workspace_bytes(4096, 256, 1) == ws_bytes
+    assert lib.ts_infonce_set_workgroup_target(100000) == 32
+    assert lib.ts_infonce_set_workgroup_target(-3) == 256
+    assert lib.ts_infonce_set_workgroup_target(0) == 256
     assert lib.ts_bn_stats(None, 2, 3, 4, p, None, None, None, None, 1e-5, None) == -1
     assert lib.ts_bn_stats(p, 2, 70000, 4, p, None, None, None, None, 1e-5, None) == -5
     assert lib.ts_bn_stats(p, 2, 3, 4, p, p, None, None, None, 1e-5, None) == -1                 # sum without sum_squares

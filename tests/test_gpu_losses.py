@@ -288,6 +288,28 @@ def test_infonce_bf16(device, n, c):
     assert (err <= 1e-3 * peak + gw.abs() * 2.0 ** -8).all() or peak < 1e-9
 
 
+@pytest.mark.parametrize("dtype,n,tol", [(torch.bfloat16, 4096, 1e-3), (torch.bfloat16, 1000, 1e-3),
+                                         (torch.float32, 640, 1e-4)])
+@pytest.mark.parametrize("target", [32, 64, 100])
+def test_infonce_workgroup_target_changes_the_schedule_not_the_result(device, dtype, n, tol, target):
+    # fewer workgroups = fewer key splits (one at 32): same oracle, same bars
+    q, k = _nce_inputs(n, 256, 5, dtype)
+    want, (gw,) = _oracle_grad(lambda a, b: ts_oracle.infonce(a, b, 0.2), q, others=(k,))
+    assert ta.set_infonce_workgroup_target(target) == 256
+    try:
+        qd = q.to(device).requires_grad_()
+        loss = ta.infonce_loss(qd, k.to(device), 0.2)
+        loss.backward()
+        torch.cuda.synchronize()
+    finally:
+        assert ta.set_infonce_workgroup_target(0) == target
+    assert rel_err(loss.item(), want) < (1e-3 if dtype == torch.bfloat16 else 1e-5)
+    peak = gw.abs().max().item()
+    err = (qd.grad.cpu().double() - gw).abs()
+    slack = 2.0 ** -8 if dtype == torch.bfloat16 else 0.0
+    assert (err <= tol * peak + gw.abs() * slack).all()
+
+
 def test_infonce_more_keys_than_an_l2_holds(device):
     # above 8192 rows the launcher makes the key split the fastest grid index; 8330 is not a
     # multiple of the 128-row q tile or the 64-key stage, so padded rows and keys are in play

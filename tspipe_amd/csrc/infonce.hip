@@ -57,6 +57,7 @@
 // MFMA 32x32x16 operand layout used throughout (lane l, half h = l/32):
 //   A: row l%32, contraction slots 8h..8h+7;  B: column l%32, same slots;
 //   D[i]: row (i%4) + 4h + 8(i/4), column l%32.
+#include <atomic>
 #include <type_traits>
 
 #include "infonce_common.h"
@@ -93,20 +94,20 @@ struct NceLayout {
 // Key splits: enough workgroups for one per CU (a workgroup is 4 wavefronts,
 // one per SIMD, each with its own software pipeline; its three stage buffers
 // take most of a CU's LDS).
-inline int nce_splits(int64_t npad, int n_pairs) {
+inline int nce_splits(int64_t npad, int n_pairs, int target) {
   const int64_t qtiles = npad / kQTile * n_pairs;
   const int64_t stages = npad / kStageKeys;
-  int64_t s = (256 + qtiles - 1) / qtiles;
+  int64_t s = (target + qtiles - 1) / qtiles;
   if (s > 16) s = 16;
   if (s > stages) s = stages;
   if (s < 1) s = 1;
   return (int)s;
 }
 
-inline NceLayout nce_layout(int64_t n, int64_t c, int n_pairs) {
+inline NceLayout nce_layout(int64_t n, int64_t c, int n_pairs, int target) {
   NceLayout L;
   L.npad = nce_round_up(n > 0 ? n : 1, kQTile);
-  L.splits = nce_splits(L.npad, n_pairs);
+  L.splits = nce_splits(L.npad, n_pairs, target);
   L.head_bytes = 256;  // scratch for the empty-batch case
   size_t o = 0;
   L.off_rq = o;       o += nce_align(L.npad * 4);
@@ -897,7 +898,7 @@ int nce_dispatch_c(const NceArgs& args, int pairs, int64_t n, int64_t c, float t
 // Fills the per-pair workspace pointers and launches.
 int nce_launch(NceArgs& args, int pairs, int64_t n, int64_t c, float tau, void* workspace, float* loss_out,
                int dtype, hipStream_t st) {
-  const NceLayout L = nce_layout(n, c, pairs);
+  const NceLayout L = nce_layout(n, c, pairs, nce_workgroup_target());
   char* ws = (char*)workspace;
   for (int p = 0; p < 2; ++p) {
     const int src = p < pairs ? p : 0;  // an unused second slot mirrors the first
@@ -940,16 +941,24 @@ inline bool nce_bf16_path(int64_t c, float tau, int dtype) {
   return dtype != TS_F32 && (c == 64 || c == 128 || c == 256) && tau >= 0.03f;
 }
 
+static std::atomic<int> g_nce_workgroup_target{kNceMaxWorkgroupTarget};
+int nce_workgroup_target() { return g_nce_workgroup_target.load(std::memory_order_relaxed); }
+
 }  // namespace ts
 
 extern "C" {
+
+int ts_infonce_set_workgroup_target(int workgroups) {
+  if (workgroups <= 0 || workgroups > ts::kNceMaxWorkgroupTarget) workgroups = ts::kNceMaxWorkgroupTarget;
+  return ts::g_nce_workgroup_target.exchange(workgroups, std::memory_order_relaxed);
+}
 
 size_t ts_infonce_workspace_bytes(int64_t n, int64_t c, int n_pairs) {
   if (n < 0 || c <= 0 || c > 512 || n_pairs < 1 || n_pairs > 2) return 0;
   // dtype and temperature decide the path at call time: room for either
   size_t bytes = ts::nce_general_workspace_bytes(n, c, n_pairs);
   if (c == 64 || c == 128 || c == 256) {
-    const ts::NceLayout L = ts::nce_layout(n, c, n_pairs);
+    const ts::NceLayout L = ts::nce_layout(n, c, n_pairs, ts::kNceMaxWorkgroupTarget);
     const size_t b16 = L.head_bytes + L.pair_bytes * (size_t)n_pairs;
     if (b16 > bytes) bytes = b16;
   }

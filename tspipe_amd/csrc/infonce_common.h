@@ -78,6 +78,12 @@ __device__ __forceinline__ NceRow nce_row(const NcePair& pr, int64_t row, int C)
 // The fp32-MFMA path (infonce_general.hip): any width up to 512, any
 // temperature, products and sums in fp32.  args holds q / k / dq (or their
 // pieces); the workspace pointers are filled in by the launcher.
+// Workgroups the main kernels aim to put on the chip (ts_infonce_set_workgroup_target):
+// the number of key splits follows from it.  kNceMaxWorkgroupTarget, one per
+// CU, is the default and what the workspace is sized for.
+constexpr int kNceMaxWorkgroupTarget = 256;
+int nce_workgroup_target();
+
 size_t nce_general_workspace_bytes(int64_t n, int64_t c, int n_pairs);
 int nce_general_launch(NceArgs& args, int pairs, int64_t n, int64_t c, float tau, void* workspace, float* loss_out,
                        int dtype, hipStream_t stream);

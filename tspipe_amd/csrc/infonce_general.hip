@@ -54,10 +54,10 @@ struct NceGenLayout {
 
 inline int nce_gen_cp(int64_t c) { return c <= 64 ? 64 : (c <= 128 ? 128 : (c <= 256 ? 256 : 512)); }
 
-inline int nce_gen_splits(int64_t npad, int n_pairs, int fgroups) {
+inline int nce_gen_splits(int64_t npad, int n_pairs, int fgroups, int target) {
   const int64_t wgs = npad / kGenQTile * n_pairs * fgroups;
   const int64_t tiles = npad / kGenKeys;
-  int64_t s = (256 + wgs - 1) / wgs;
+  int64_t s = (target + wgs - 1) / wgs;
   if (s > 16) s = 16;
   if (s > tiles) s = tiles;
   if (s < 1) s = 1;
@@ -66,11 +66,11 @@ inline int nce_gen_splits(int64_t npad, int n_pairs, int fgroups) {
 
 inline int nce_gen_fgroups(int cp) { return cp > 256 ? cp / 128 : 1; }
 
-inline NceGenLayout nce_gen_layout(int64_t n, int64_t c, int n_pairs) {
+inline NceGenLayout nce_gen_layout(int64_t n, int64_t c, int n_pairs, int target) {
   NceGenLayout L;
   L.npad = nce_round_up(n > 0 ? n : 1, kGenQTile);
   L.cp = nce_gen_cp(c);
-  L.splits = nce_gen_splits(L.npad, n_pairs, nce_gen_fgroups(L.cp));
+  L.splits = nce_gen_splits(L.npad, n_pairs, nce_gen_fgroups(L.cp), target);
   L.head_bytes = 256;
   size_t o = 0;
   L.off_rq = o;     o += nce_align(L.npad * 4);
@@ -452,14 +452,14 @@ int nce_gen_dispatch(const NceArgs& args, int pairs, int64_t n, int c, float tau
 }
 
 size_t nce_general_workspace_bytes(int64_t n, int64_t c, int n_pairs) {
-  const NceGenLayout L = nce_gen_layout(n, c, n_pairs);
+  const NceGenLayout L = nce_gen_layout(n, c, n_pairs, kNceMaxWorkgroupTarget);
   return L.head_bytes + L.pair_bytes * (size_t)n_pairs + L.rowloss_bytes;
 }
 
 int nce_general_launch(NceArgs& args, int pairs, int64_t n, int64_t c, float tau, void* workspace, float* loss_out,
                        int dtype, hipStream_t stream) {
   if (c < 1 || c > 512) return TS_ERR_RANGE;
-  const NceGenLayout L = nce_gen_layout(n, c, pairs);
+  const NceGenLayout L = nce_gen_layout(n, c, pairs, nce_workgroup_target());
   char* ws = (char*)workspace;
   const size_t esz = dtype == TS_F32 ? 4 : 2;
   // four elements per load when every row starts on a multiple of that load's size

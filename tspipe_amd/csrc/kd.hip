@@ -417,10 +417,9 @@ __global__ __launch_bounds__(BLOCK, (KREG * GROUP > 1024 ? 4 : 1)) void kd_rows_
   const int64_t ntail = V - g.tail0;
   if (kAlignedOnly || (g.head < VEC && ntail < VEC)) {
     // The packed row pair stays in registers and is walked three times
-    // (maxima, sums, gradient), the exponentials being retaken in the third
-    // walk.  Keeping them instead (two per logit pair fewer) was measured no
-    // faster for short rows and slower for long ones: it doubles the
-    // registers, and occupancy is what hides the load latency here.
+    // (maxima, sums, gradient).  (Keeping the exponentials BESIDE the logits
+    // doubles the registers and was measured slower: occupancy is what hides
+    // the load latency here.)
     const bool has_h = gtid < g.head, has_t = gtid < ntail;
     float eh_t = kNegBig, eh_s = kNegBig, el_t = kNegBig, el_s = kNegBig;  // end elements: head, last
     if (has_h) {
@@ -473,22 +472,42 @@ __global__ __launch_bounds__(BLOCK, (KREG * GROUP > 1024 ? 4 : 1)) void kd_rows_
       }
     }
     const float mtk = mt * a.k, msk = ms * a.k, ms1 = ms * kLog2e;
+    // fp32 rows: the second walk leaves its exponentials where the logits
+    // were (the student's logit stays when the CE term needs it at temperature
+    // 1), so the gradient walk takes none again.  16-bit rows retake them: a
+    // 16-bit slot would round them, and p_s - p_t cancels.
+    constexpr bool kKeep = sizeof(T) == 4;
     float zt = 0.f, at = 0.f, zs = 0.f, z1 = 0.f;
-    auto add = [&](float tv, float sv) {
-      const float et = fast_exp2(fmaf(tv, a.k, -mtk));
-      zt += et;
-      zs += fast_exp2(fmaf(sv, a.k, -msk));
-      at = acc_weighted_diff(et, tv, sv, at);
-      if (CE) z1 += fast_exp2(fmaf(sv, kLog2e, -ms1));
-    };
-    add(eh_t, eh_s);  // a missing end element contributes 2^(-huge) = 0
-    add(el_t, el_s);
+    // a missing end element contributes 2^(-huge) = 0; most wavefronts have none at all
+    if (__any(has_h || has_t)) {
+      auto add = [&](float tv, float sv) {
+        const float et = fast_exp2(fmaf(tv, a.k, -mtk));
+        zt += et;
+        zs += fast_exp2(fmaf(sv, a.k, -msk));
+        at = acc_weighted_diff(et, tv, sv, at);
+        if (CE) z1 += fast_exp2(fmaf(sv, kLog2e, -ms1));
+      };
+      add(eh_t, eh_s);
+      add(el_t, el_s);
+    }
 #pragma unroll
     for (int j = 0; j < KREG; ++j) {
       if (gtid + j * GROUP < (int)g.nvec) {
         fresh(j);
 #pragma unroll
-        for (int i = 0; i < VEC; ++i) add(to_f32(rt[j].v[i]), to_f32(rs[j].v[i]));
+        for (int i = 0; i < VEC; ++i) {
+          const float tv = to_f32(rt[j].v[i]), sv = to_f32(rs[j].v[i]);
+          const float et = fast_exp2(fmaf(tv, a.k, -mtk));
+          const float es = fast_exp2(fmaf(sv, a.k, -msk));
+          zt += et;
+          zs += es;
+          at = acc_weighted_diff(et, tv, sv, at);
+          if (CE) z1 += fast_exp2(fmaf(sv, kLog2e, -ms1));
+          if constexpr (kKeep) {
+            rt[j].v[i] = et;
+            if (!CE) rs[j].v[i] = es;
+          }
+        }
       }
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -542,7 +561,22 @@ __global__ __launch_bounds__(BLOCK, (KREG * GROUP > 1024 ? 4 : 1)) void kd_rows_
         Vec16<T> o;
         const int e0 = (int)g.head + (gtid + j * GROUP) * VEC;
 #pragma unroll
-        for (int i = 0; i < VEC; ++i) o.v[i] = grad_of(to_f32(rt[j].v[i]), to_f32(rs[j].v[i]), e0 + i);
+        for (int i = 0; i < VEC; ++i) {
+          if constexpr (kKeep) {
+            const float pt = rt[j].v[i] * rt_;
+            if (CE) {
+              const float sv = rs[j].v[i];
+              const float es = fast_exp2(fmaf(sv, a.k, -msk));
+              const float e1 = fast_exp2(fmaf(sv, kLog2e, -ms1));
+              const float gv = f.g_kd * fmaf(es, rs_, -pt);
+              o.v[i] = fmaf(f.g_ce, fmaf(e1, r1_, e0 + i == label ? -1.f : 0.f), gv);
+            } else {
+              o.v[i] = f.g_kd * fmaf(rs[j].v[i], rs_, -pt);
+            }
+          } else {
+            o.v[i] = grad_of(to_f32(rt[j].v[i]), to_f32(rs[j].v[i]), e0 + i);
+          }
+        }
         store16(grow + e0, o);
       }
       __builtin_amdgcn_sched_barrier(0);

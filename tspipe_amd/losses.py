@@ -577,6 +577,17 @@ def _infonce(q1: Tensor, k1: Tensor, q2: Optional[Tensor], k2: Optional[Tensor],
     return _InfoNCEFn.apply(q1, k1, q2, k2, tau)
 
 
+def set_infonce_workgroup_target(workgroups: int = 0) -> int:
+    """Scheduling knob of the InfoNCE kernels (``ts_infonce_set_workgroup_target``):
+    about how many workgroups the main kernel puts on the 256 CUs.  The default
+    (0 or 256) suits a loss that has the GPU to itself; a pipeline that runs the
+    loss beside bandwidth-bound work on another stream, as TSPipe runs it beside
+    the momentum update (tspipe/gpu_task.py:385-410), gets a shorter step from
+    64: fewer partial sums through HBM, CUs left to the other stream.
+    Process-wide; returns the previous value."""
+    return int(_lib.lib().ts_infonce_set_workgroup_target(int(workgroups)))
+
+
 def infonce_loss(q: Tensor, k: Tensor, tau: float) -> Tensor:
     """One direction of MoCo-v3's loss: ``CE(q^ k^T / tau, arange(N)) * 2 tau``
     (benchmarks/moco-v3/main.py:149-160)."""
