@@ -11,7 +11,10 @@ import threading
 from ctypes import c_char_p, c_double, c_float, c_int, c_int64, c_size_t, c_void_p
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libtspipe_amd.so")
+# TSPIPE_AMD_LIBRARY names another build of the same C ABI (a measurement
+# variant from `python -m tspipe_amd.build --variant NAME`); unset, the
+# library next to this file is the one.
+LIB_PATH = os.environ.get("TSPIPE_AMD_LIBRARY") or os.path.join(_HERE, "libtspipe_amd.so")
 
 TS_F32, TS_BF16, TS_F16 = 0, 1, 2
 

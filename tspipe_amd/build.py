@@ -21,9 +21,9 @@ DEVICE_FLAGS = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang"
 COMMON_FLAGS = ["-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function", "-x", "hip"]
 
 
-def _compile(src: str) -> str:
-    obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")
-    cmd = [HIPCC, *COMMON_FLAGS, *DEVICE_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+def _compile(src: str, defines=(), obj_dir: str = OBJ_DIR) -> str:
+    obj = os.path.join(obj_dir, os.path.splitext(src)[0] + ".o")
+    cmd = [HIPCC, *COMMON_FLAGS, *DEVICE_FLAGS, *["-D" + d for d in defines], "-c", os.path.join(CSRC, src), "-o", obj]
     res = subprocess.run(cmd, capture_output=True, text=True)
     noise = "is not a recognized feature for this target"
     err = "\n".join(l for l in res.stderr.splitlines() if noise not in l)
@@ -47,6 +47,35 @@ def build(verbose: bool = True) -> str:
     if verbose:
         print(f"built {LIB_PATH}")
     return LIB_PATH
+
+
+# Measurement variants: the library with one source rebuilt under a macro, for
+# A/B runs against the default build (TSPIPE_AMD_LIBRARY selects the file that
+# tspipe_amd loads).  None of them is loaded unless asked for.
+VARIANTS = {
+    # long 16-bit KD rows parked in LDS instead of registers between the walks
+    "kd-rows-in-lds": ("kd.hip", ["TS_KD_ROWS_IN_LDS"]),
+}
+
+
+def build_variant(name: str, verbose: bool = True) -> str:
+    """Builds libtspipe_amd.<name>.so: the objects of the default build (built
+    first if missing) with the variant's source recompiled under its macros."""
+    src, defines = VARIANTS[name]
+    if not all(os.path.exists(os.path.join(OBJ_DIR, os.path.splitext(s)[0] + ".o")) for s in SOURCES):
+        build(verbose=False)
+    var_dir = os.path.join(OBJ_DIR, name)
+    os.makedirs(var_dir, exist_ok=True)
+    var_obj = _compile(src, defines, var_dir)
+    objs = [var_obj if s == src else os.path.join(OBJ_DIR, os.path.splitext(s)[0] + ".o") for s in SOURCES]
+    out = os.path.join(HERE, f"libtspipe_amd.{name}.so")
+    res = subprocess.run([HIPCC, "-shared", "-fPIC", "--offload-arch=gfx950", *objs, "-o", out],
+                         capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"link failed:\n{res.stderr}")
+    if verbose:
+        print(f"built {out}")
+    return out
 
 
 HOST_DIR = os.path.join(HERE, "csrc_host")
@@ -88,6 +117,9 @@ def build_consumer(verbose: bool = False) -> str:
 
 
 if __name__ == "__main__":
-    build()
-    build_host()
-    build_consumer()
+    if len(sys.argv) > 2 and sys.argv[1] == "--variant":
+        build_variant(sys.argv[2])
+    else:
+        build()
+        build_host()
+        build_consumer()

@@ -394,12 +394,30 @@ __global__ __launch_bounds__(BLOCK, (KREG * GROUP > 1024 ? 4 : 1)) void kd_rows_
 
   const RowGeom g = row_geom<T>(srow, trow, grow, V);
   Vec16<T> rt[KREG], rs[KREG];
+#ifdef TS_KD_ROWS_IN_LDS
+  // Measurement variant, not part of the default build: the 512-thread
+  // long-row instantiation for 16-bit logits parks the row pair in LDS (2 x 64
+  // KB, one workgroup per CU) instead of in registers, every lane reading back
+  // the vectors it wrote, one pair at a time in each of the three walks.
+  constexpr bool kStage = BLOCK == 512 && KREG * GROUP > 1024 && sizeof(T) == 2;
+  __shared__ u32x4 stage_t[kStage ? KREG * GROUP : 1], stage_s[kStage ? KREG * GROUP : 1];
+#else
+  constexpr bool kStage = false;
+  u32x4* const stage_t = nullptr;
+  u32x4* const stage_s = nullptr;
+#endif
 #pragma unroll
   for (int j = 0; j < KREG; ++j) {
     const int64_t v = gtid + (int64_t)j * GROUP;
     if (v < g.nvec) {
-      rt[j] = load16(trow + g.head + v * VEC);
-      rs[j] = load16(srow + g.head + v * VEC);
+      if constexpr (kStage) {
+        const Vec16<T> lt = load16(trow + g.head + v * VEC), ls = load16(srow + g.head + v * VEC);
+        __builtin_memcpy(&stage_t[v], &lt, 16);
+        __builtin_memcpy(&stage_s[v], &ls, 16);
+      } else {
+        rt[j] = load16(trow + g.head + v * VEC);
+        rs[j] = load16(srow + g.head + v * VEC);
+      }
     }
   }
   // No counting launch ran in front (mask-only call on long rows): the number
@@ -433,6 +451,11 @@ __global__ __launch_bounds__(BLOCK, (KREG * GROUP > 1024 ? 4 : 1)) void kd_rows_
     // Each walk starts from registers the compiler can assume nothing about;
     // otherwise it would unpack the row once and keep all the fp32 values.
     auto fresh = [&](int j) {
+      if constexpr (kStage) {
+        __builtin_memcpy(&rt[j], &stage_t[gtid + j * GROUP], 16);
+        __builtin_memcpy(&rs[j], &stage_s[gtid + j * GROUP], 16);
+        return;
+      }
       u32x4 bt, bs;
       __builtin_memcpy(&bt, &rt[j], 16);
       __builtin_memcpy(&bs, &rs[j], 16);
@@ -444,6 +467,7 @@ __global__ __launch_bounds__(BLOCK, (KREG * GROUP > 1024 ? 4 : 1)) void kd_rows_
 #pragma unroll
     for (int j = 0; j < KREG; ++j) {
       if (gtid + j * GROUP < (int)g.nvec) {
+        if constexpr (kStage) fresh(j);
 #pragma unroll
         for (int i = 0; i < VEC; ++i) {
           mt = fmaxf(mt, to_f32(rt[j].v[i]));
