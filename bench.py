@@ -266,6 +266,8 @@ TIMING_NOTE = ("ms: median over >=50 samples after >=10 warm-up calls; a sample 
                "`calls_per_sample` back-to-back calls, one per rotating buffer set (4 calls on the same buffers "
                "where the entry names no buffer sets)")
 MALL_BYTES = 256 << 20  # Infinity Cache: a working set below this is not an HBM measurement
+ONE_SET_NOTE = ("the same call looping on one set: the logits of its selected rows (75 MB) can stay in the Infinity "
+                "Cache between calls")
 KD_MASKED_LAUNCHES = 2   # row kernel (selected rows and the zero-fill of the others), final reduction
 
 
@@ -327,7 +329,7 @@ def run_kernel_table(dev, with_cpu=True):
                 ts_oracle.distil_ce(s_c, t_c, m_c, T).backward()
         return f
 
-    def entry(nbytes, ms, note=None, launches=None, working_set=None, sets=1, resident_ms=None):
+    def entry(nbytes, ms, note=None, launches=None, working_set=None, sets=1, resident_ms=None, resident_note=None):
         """working_set: bytes the timed calls touch between two visits of the
         same address (all rotating sets together); sets: buffer sets rotated
         through; resident_ms: the same call looping on ONE set, when that set
@@ -345,7 +347,8 @@ def run_kernel_table(dev, with_cpu=True):
         if resident_ms is not None:
             e["infinity_cache_resident"] = {"ms": round(resident_ms, 4),
                                             "GB/s": round(nbytes / (resident_ms * 1e-3) / 1e9, 1),
-                                            "note": "the same call looping on one buffer set that fits the Infinity Cache"}
+                                            "note": resident_note or "the same call looping on one buffer set that fits "
+                                                                     "the Infinity Cache"}
         if note:
             e["note"] = note
         return e
@@ -452,11 +455,19 @@ def run_kernel_table(dev, with_cpu=True):
     cpu("kd_32768x1000_f32", kd_cpu(*fns[0].operands, 4.0))
     del fns, s, t, f
 
-    # DistilBERT-shaped masked KD (cfg3) after a gather of 4 micro-batches
-    pieces_s = [(torch.randn(8, 128, 30522, generator=g) * 2).to(torch.bfloat16).to(dev) for _ in range(4)]
-    pieces_t = [(torch.randn(8, 128, 30522, generator=g) * 2).to(torch.bfloat16).to(dev) for _ in range(4)]
-    mask = (torch.rand(32, 128, generator=g) < 0.15).to(dev)
+    # DistilBERT-shaped masked KD (cfg3) after a gather of 4 micro-batches.  The selected rows of one
+    # set of logits (75 MB) would survive in the Infinity Cache from call to call, so the loss entries
+    # take two sets (their own logits, mask and gradient buffers) in turn.
+    import ctypes
+    row_b = 30522 * 2
+    sets = []
+    for _ in range(2):
+        ps = [(torch.randn(8, 128, 30522, generator=g) * 2).to(torch.bfloat16).to(dev) for _ in range(4)]
+        pt = [(torch.randn(8, 128, 30522, generator=g) * 2).to(torch.bfloat16).to(dev) for _ in range(4)]
+        sets.append({"s": ps, "t": pt, "mask": (torch.rand(32, 128, generator=g) < 0.15).to(dev)})
+    pieces_s, pieces_t, mask = sets[0]["s"], sets[0]["t"], sets[0]["mask"]
     n_sel = int(mask.sum().item())
+    n_sel_avg = sum(int(d["mask"].sum().item()) for d in sets) / len(sets)
     s_full = torch.empty(32, 128, 30522, dtype=torch.bfloat16, device=dev)
     dsts = list(s_full.chunk(4))
     for i in range(25):
@@ -470,35 +481,48 @@ def run_kernel_table(dev, with_cpu=True):
     out["gather_4x62.5MB_bf16"] = entry(2 * 250036224, statistics.median(ms), "kernel-only events", 1)
     pieces_c = [p_.cpu() for p_ in pieces_s]
     cpu("gather_4x62.5MB_bf16", lambda: ts_oracle.gather(pieces_c))
-    del pieces_c
-    t_full = ta.gather([ta.Batch(p) for p in pieces_t])
-    row_b = 30522 * 2
-    # the same loss straight from the four micro-batch outputs (no gather of s or t)
-    import ctypes
-    flat_s = [p.view(-1, 30522) for p in pieces_s]
-    flat_t = [p.view(-1, 30522) for p in pieces_t]
-    grads = [torch.empty_like(p) for p in flat_s]
-    ws_p = torch.empty(lib.ts_kd_workspace_bytes(4096, 30522, _lib.TS_BF16), dtype=torch.uint8, device=dev)
-    loss_p = torch.empty((), device=dev)
-    arr = lambda ts: (ctypes.c_void_p * 4)(*[t.data_ptr() for t in ts])
-    a_s, a_t, a_g, a_r = arr(flat_s), arr(flat_t), arr(grads), (ctypes.c_int64 * 4)(1024, 1024, 1024, 1024)
-    mptr = mask.view(torch.uint8).data_ptr()
+    del pieces_c, s_full, dsts
+    kd_bytes = int(3 * n_sel_avg * row_b + (4096 - n_sel_avg) * row_b)
 
-    def f_pieces():
-        _lib.check(lib.ts_kdce_pieces_fwd_bwd(a_s, a_t, a_g, a_r, 4, mptr, None, 0, 30522, 0.5, 4.0, 0.0, ws_p.data_ptr(),
-                                              loss_p.data_ptr(), _lib.TS_BF16, stream), "ts_kdce_pieces_fwd_bwd")
+    # the loss straight from the four micro-batch outputs (no gather of s or t)
+    def pieces_call(d):
+        flat_s = [p.view(-1, 30522) for p in d["s"]]
+        flat_t = [p.view(-1, 30522) for p in d["t"]]
+        grads = [torch.empty_like(p) for p in flat_s]
+        ws_p = torch.empty(lib.ts_kd_workspace_bytes(4096, 30522, _lib.TS_BF16), dtype=torch.uint8, device=dev)
+        loss_p = torch.empty((), device=dev)
+        arr = lambda ts: (ctypes.c_void_p * 4)(*[t.data_ptr() for t in ts])
+        a_s, a_t, a_g, a_r = arr(flat_s), arr(flat_t), arr(grads), (ctypes.c_int64 * 4)(1024, 1024, 1024, 1024)
+        mptr = d["mask"].view(torch.uint8).data_ptr()
+
+        def f():
+            _lib.check(lib.ts_kdce_pieces_fwd_bwd(a_s, a_t, a_g, a_r, 4, mptr, None, 0, 30522, 0.5, 4.0, 0.0,
+                                                  ws_p.data_ptr(), loss_p.data_ptr(), _lib.TS_BF16, stream),
+                       "ts_kdce_pieces_fwd_bwd")
+        f.keep = (flat_s, flat_t, grads, ws_p, loss_p, a_s, a_t, a_g, a_r)
+        return f
+    fns = [pieces_call(d) for d in sets]
     out["kd_masked_4_pieces_8x128x30522_bf16"] = entry(
-        3 * n_sel * row_b + (4096 - n_sel) * row_b, _time_stream(f_pieces),
-        "same loss read from the 4 micro-batch outputs in place: replaces 2 gathers (2 x ~77 us) + the call below",
-        KD_MASKED_LAUNCHES, working_set=3 * 4096 * row_b)
-    del pieces_s, pieces_t, flat_s, flat_t, grads, ws_p
-    f = kd_call(s_full, t_full, mask, 2.0, torch.empty_like(s_full))
-    out["kd_masked_32x128x30522_bf16"] = entry(3 * n_sel * row_b + (4096 - n_sel) * row_b, _time_stream(f),
-                                               f"n_sel={n_sel}; bytes = read s,t + write grad for selected rows, "
-                                               f"zero-fill of the other rows", KD_MASKED_LAUNCHES,
-                                               working_set=3 * 4096 * row_b)
+        kd_bytes, _time_stream(rotate(fns), batch=2),
+        "same loss read from the 4 micro-batch outputs in place: replaces 2 gathers (2 x ~78 us) + the call below",
+        KD_MASKED_LAUNCHES, working_set=2 * 3 * 4096 * row_b, sets=2, resident_ms=_time_stream(fns[0]),
+        resident_note=ONE_SET_NOTE)
+    del fns
+    # the gathered form: s, t of each set concatenated first (untimed), the pieces released
+    for d in sets:
+        d["s_full"] = ta.gather([ta.Batch(p) for p in d["s"]])
+        d["t_full"] = ta.gather([ta.Batch(p) for p in d["t"]])
+        d["s"] = d["t"] = None
+    del pieces_s, pieces_t
+    fns = [kd_call(d["s_full"], d["t_full"], d["mask"], 2.0, torch.empty_like(d["s_full"])) for d in sets]
+    out["kd_masked_32x128x30522_bf16"] = entry(
+        kd_bytes, _time_stream(rotate(fns), batch=2),
+        f"n_sel={n_sel_avg:.0f} on average; bytes = read s,t + write grad for selected rows, zero-fill of the other rows",
+        KD_MASKED_LAUNCHES, working_set=2 * 3 * 4096 * row_b, sets=2, resident_ms=_time_stream(fns[0]),
+        resident_note=ONE_SET_NOTE)
     if with_cpu:
-        s_c, t_c, m_c = s_full.cpu(), t_full.cpu(), mask.cpu()
+        d = sets[0]
+        s_c, t_c, m_c = d["s_full"].cpu(), d["t_full"].cpu(), d["mask"].cpu()
         sp_c, tp_c = list(s_c.chunk(4)), list(t_c.chunk(4))
         cpu("kd_masked_32x128x30522_bf16", kd_cpu(s_c, t_c, 2.0, m_c))
 
@@ -507,7 +531,7 @@ def run_kernel_table(dev, with_cpu=True):
             ts_oracle.distil_ce(s_all, ts_oracle.gather(tp_c), m_c, 2.0).backward()
         cpu("kd_masked_4_pieces_8x128x30522_bf16", pieces_cpu)
         del s_c, t_c, m_c, sp_c, tp_c
-    del s_full, t_full, f
+    del fns, sets
 
     # InfoNCE: cfg4 (single pair), the symmetric two-pair call of MoCo-v3's contrastive_loss, and a
     # batch four times as large, where the fixed costs of the three launches weigh less
