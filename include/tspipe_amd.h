@@ -405,7 +405,10 @@ int ts_infonce_pieces_fwd_bwd(const void* const* q1_pieces, const void* const* k
  * device (the last workgroup of a channel reads and clears what the others
  * added): keep them on one stream, or order the streams with events.  A
  * buffer of the 2*C floats that an earlier version of this call asked for is
- * too small. */
+ * too small.  x is fetched with non-temporal loads (it is not read again by
+ * this call): a caller that goes on to normalise the same x should use
+ * ts_bn_forward_train, whose statistics half leaves x to its second half in
+ * the caches. */
 size_t ts_bn_stats_workspace_bytes(int64_t C);
 
 int ts_bn_stats(const float* x, int64_t N, int64_t C, int64_t HW, float* ws, float* sum,
