@@ -668,10 +668,10 @@ def run_kernel_table(dev, with_cpu=True):
         commit()
     out["bn_cfg5_track_x8_commit"] = entry(MB * one_x, _time_stream(cfg5_track, batch=1), "8 x _track over 8 different "
                                            "micro-batches + _commit (momentum 0.1): one mini-batch of the configuration",
-                                           MB + 2, working_set=MB * one_x, sets=1)
+                                           MB + 1, working_set=MB * one_x, sets=1)
     out["bn_cfg5_forward_x8_commit"] = entry(3 * MB * one_x, _time_stream(cfg5_forward, batch=1), "8 x training forward "
                                              "(statistics + normalise with gamma, beta) + _commit: what DeferredBatchNorm "
-                                             "runs for one mini-batch of the configuration", 2 * MB + 2,
+                                             "runs for one mini-batch of the configuration", 2 * MB + 1,
                                              working_set=2 * MB * one_x, sets=1)
     del ys, y
     dys = [torch.randn(32, 256, 56, 56, generator=dgen, device=dev) for _ in range(4)]

@@ -175,18 +175,22 @@ __global__ __launch_bounds__(kBnBlock) void bn_stats_kernel(const float* __restr
 // The reference's rounding order, one fp32 operation at a time:
 //   mean = sum / counter;  var = sum_squares / counter - mean**2
 //   running *= (1 - f);  running += stat * f
-__global__ __launch_bounds__(256) void bn_commit_kernel(float* __restrict__ sum, float* __restrict__ sum_squares,
-                                                        float* __restrict__ running_mean,
-                                                        float* __restrict__ running_var,
-                                                        int64_t* __restrict__ nbt, int64_t C, float counter,
-                                                        double momentum) {
-  const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  // every thread reads the counter before thread 0 of block 0 bumps it: the
-  // value used is "after the increment", computed locally
+// One workgroup walks all channels (a few thousand at most), so that the
+// counter can be read by every thread, then bumped, inside one launch.
+constexpr int kBnCommitBlock = 1024;
+__global__ __launch_bounds__(kBnCommitBlock) void bn_commit_kernel(float* __restrict__ sum,
+                                                                   float* __restrict__ sum_squares,
+                                                                   float* __restrict__ running_mean,
+                                                                   float* __restrict__ running_var,
+                                                                   int64_t* __restrict__ nbt, int64_t C, float counter,
+                                                                   double momentum) {
+  // the value used is "after the increment"; thread 0 stores it once every thread has read the old one
   const int64_t tracked = nbt ? *nbt + 1 : 1;
+  __syncthreads();
+  if (nbt && threadIdx.x == 0) *nbt = tracked;
   const double f = (momentum < 0.0) ? 1.0 / (double)tracked : momentum;
   const float f32 = (float)f, omf32 = (float)(1.0 - f);
-  if (c < C) {
+  for (int64_t c = threadIdx.x; c < C; c += kBnCommitBlock) {
 #pragma clang fp contract(off)
     const float mean = sum[c] / counter;
     const float msq = mean * mean;
@@ -199,8 +203,6 @@ __global__ __launch_bounds__(256) void bn_commit_kernel(float* __restrict__ sum,
     sum_squares[c] = 0.f;
   }
 }
-
-__global__ void bn_bump_counter_kernel(int64_t* nbt) { *nbt += 1; }
 
 // y = (x - mu) * a + b over this workgroup's slab of channel c
 __device__ __forceinline__ void bn_apply_slab(const float* __restrict__ x, float* __restrict__ y, int64_t N,
@@ -456,18 +458,9 @@ int ts_bn_commit(float* sum, float* sum_squares, float* running_mean, float* run
   if (C <= 0) return TS_ERR_ARG;
   if (momentum < 0.0 && !num_batches_tracked) return TS_ERR_ARG;
   hipStream_t st = (hipStream_t)stream;
-  hipLaunchKernelGGL(ts::bn_commit_kernel, dim3((unsigned)((C + 255) / 256)), dim3(256), 0, st, sum,
-                     sum_squares, running_mean, running_var, num_batches_tracked, C, (float)counter,
-                     momentum);
-  int rc = ts::check_launch();
-  if (rc) return rc;
-  if (num_batches_tracked) {
-    // after the commit kernel on the same stream, so every workgroup of it
-    // saw the old value
-    hipLaunchKernelGGL(ts::bn_bump_counter_kernel, dim3(1), dim3(1), 0, st, num_batches_tracked);
-    rc = ts::check_launch();
-  }
-  return rc;
+  hipLaunchKernelGGL(ts::bn_commit_kernel, dim3(1), dim3(ts::kBnCommitBlock), 0, st, sum, sum_squares, running_mean,
+                     running_var, num_batches_tracked, C, (float)counter, momentum);
+  return ts::check_launch();
 }
 
 int ts_bn_apply(const float* x, float* y, const float* mean, const float* invstd_or_var,
