@@ -80,6 +80,48 @@ __device__ __forceinline__ f16_t from_f32<f16_t>(float x) {
 // rescaling them.
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// ---- 16-byte vectors of a storage type -------------------------------------
+
+template <typename T>
+struct Vec16 {
+  static constexpr int N = 16 / sizeof(T);
+  T v[N];
+};
+
+template <typename T>
+__device__ __forceinline__ Vec16<T> load16(const T* p) {
+  const u32x4 raw = *reinterpret_cast<const u32x4*>(p);
+  Vec16<T> r;
+  __builtin_memcpy(&r, &raw, 16);
+  return r;
+}
+
+template <typename T>
+__device__ __forceinline__ Vec16<T> load16_stream(const T* p) {
+  const u32x4 raw = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+  Vec16<T> r;
+  __builtin_memcpy(&r, &raw, 16);
+  return r;
+}
+
+template <typename T>
+__device__ __forceinline__ void store16(T* p, const Vec16<T>& v) {
+  u32x4 raw;
+  __builtin_memcpy(&raw, &v, 16);
+  *reinterpret_cast<u32x4*>(p) = raw;
+}
+
+// Non-temporal store, for data that is written once and read only by a later
+// kernel.  Whether it pays is measured per kernel: the KD gradient rows and
+// the BatchNorm outputs gain from it; a pure zero-fill loses (the same bytes
+// take 1.6x as long as with plain stores).
+template <typename T>
+__device__ __forceinline__ void store16_stream(T* p, const Vec16<T>& v) {
+  u32x4 raw;
+  __builtin_memcpy(&raw, &v, 16);
+  __builtin_nontemporal_store(raw, reinterpret_cast<u32x4*>(p));
+}
+
 // ---- wavefront / block reductions -----------------------------------------
 
 __device__ __forceinline__ float wave_sum(float v) {

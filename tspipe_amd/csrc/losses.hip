@@ -260,42 +260,99 @@ __global__ __launch_bounds__(256) void cosine_rows_kernel(const RowPieces tab, c
 constexpr int kMseBlock = 256;
 constexpr int kMseSpan = 2048;
 
+// One element: its squared difference into acc, its gradient (or a zero) out.
+template <typename T>
+__device__ __forceinline__ T mse_grad_one(T sv, T tv, T gold, float k, int accumulate, float& acc) {
+  const float d = to_f32(sv) - to_f32(tv);
+  acc += d * d;
+  return from_f32<T>(accumulate ? to_f32(gold) + k * d : k * d);
+}
+
+// A workgroup owns kMseSpan elements of one row.  Where s, t and the gradient
+// row sit at the same offset from a 16-byte boundary (the usual case) these
+// are the span's 16-byte vectors of the row's aligned middle, and the first
+// workgroup of the row also takes the few elements in front of and behind
+// that middle; otherwise the span is walked element by element.
 template <typename T>
 __global__ __launch_bounds__(kMseBlock) void mse_rows_kernel(const RowPieces tab, const uint8_t* __restrict__ mask,
                                                               const int* __restrict__ n_sel_dev, int64_t n_rows,
                                                               int64_t V, float weight, int per_element, int accumulate,
                                                               float* __restrict__ partial) {
+  constexpr int VEC = 16 / sizeof(T);
+  constexpr int kVecSpan = kMseSpan / VEC;          // vectors per workgroup
+  constexpr int kPerThread = kVecSpan / kMseBlock;  // vectors per thread (1 for 16-bit types, 2 for fp32)
+  static_assert(kPerThread >= 1 && kVecSpan % kMseBlock == 0, "span and block do not fit the vector width");
   __shared__ float lds[kMseBlock / kWave];
   const int64_t parts = gridDim.x;
   const float rows_sel = n_sel_dev ? (float)(*n_sel_dev) : (float)n_rows;
   const float denom = per_element ? rows_sel * (float)V : rows_sel;
   const float k = 2.f * weight / denom;
+  const int tid = threadIdx.x;
   for (int64_t row = blockIdx.y; row < n_rows; row += gridDim.y) {
     const bool sel = !mask || mask[row] != 0;
-    const int64_t i0 = (int64_t)blockIdx.x * kMseSpan + threadIdx.x;  // consecutive lanes, consecutive elements
     float acc = 0.f;
     const RowPtrs<T> rp = row_ptrs<T>(tab, row);
-    if (sel) {
-      const T* sr = rp.a;
-      const T* tr = rp.b;
-      T* gr = rp.g;
+    const T* sr = rp.a;
+    const T* tr = rp.b;
+    T* gr = rp.g;
+    if (sel || (gr && !accumulate)) {
+      const uint32_t mis = (uint32_t)((uintptr_t)sr & 15u);
+      const bool alike = mis == (uint32_t)((uintptr_t)tr & 15u) && (!gr || mis == (uint32_t)((uintptr_t)gr & 15u)) &&
+                         mis % sizeof(T) == 0;
+      int64_t head = alike ? (int64_t)(((16u - mis) & 15u) / sizeof(T)) : V;
+      if (head > V) head = V;
+      const int64_t nvec = (V - head) / VEC, tail0 = head + nvec * VEC;
+      const T zero = from_f32<T>(0.f);
+      auto one = [&](int64_t i) {
+        if (sel) {
+          const T gv = mse_grad_one<T>(sr[i], tr[i], (gr && accumulate) ? gr[i] : zero, k, accumulate, acc);
+          if (gr) gr[i] = gv;
+        } else {
+          gr[i] = zero;
+        }
+      };
+      if (!alike) {
+        // consecutive lanes, consecutive elements
+        const int64_t i0 = (int64_t)blockIdx.x * kMseSpan + tid;
 #pragma unroll
-      for (int j = 0; j < kMseSpan / kMseBlock; ++j) {
-        const int64_t i = i0 + j * kMseBlock;
-        if (i < V) {
-          const float d = to_f32(sr[i]) - to_f32(tr[i]);
-          acc += d * d;
-          if (gr) gr[i] = from_f32<T>(accumulate ? to_f32(gr[i]) + k * d : k * d);
+        for (int j = 0; j < kMseSpan / kMseBlock; ++j)
+          if (i0 + j * kMseBlock < V) one(i0 + j * kMseBlock);
+      } else {
+        if (blockIdx.x == 0) {
+          if (tid < head) one(tid);
+          if (tail0 + tid < V) one(tail0 + tid);
+        }
+        const T* s4 = sr + head;
+        const T* t4 = tr + head;
+        T* g4 = gr + head;
+        const int64_t v0 = (int64_t)blockIdx.x * kVecSpan + tid;
+        Vec16<T> vs[kPerThread], vt[kPerThread], vg[kPerThread];
+#pragma unroll
+        for (int j = 0; j < kPerThread; ++j) {
+          const int64_t v = v0 + j * kMseBlock;
+          if (v < nvec && sel) {
+            vs[j] = load16(s4 + v * VEC);
+            vt[j] = load16(t4 + v * VEC);
+            if (gr && accumulate) vg[j] = load16(g4 + v * VEC);
+          }
+        }
+#pragma unroll
+        for (int j = 0; j < kPerThread; ++j) {
+          const int64_t v = v0 + j * kMseBlock;
+          if (v < nvec) {
+            Vec16<T> o;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e)
+              o.v[e] = sel ? mse_grad_one<T>(vs[j].v[e], vt[j].v[e], (gr && accumulate) ? vg[j].v[e] : zero, k,
+                                             accumulate, acc)
+                           : zero;
+            if (gr) store16(g4 + v * VEC, o);
+          }
         }
       }
-    } else if (rp.g && !accumulate) {
-      T* gr = rp.g;
-#pragma unroll
-      for (int j = 0; j < kMseSpan / kMseBlock; ++j)
-        if (i0 + j * kMseBlock < V) gr[i0 + j * kMseBlock] = from_f32<T>(0.f);
     }
     const float tot = block_sum<kMseBlock / kWave>(acc, lds);
-    if (threadIdx.x == 0) partial[row * parts + blockIdx.x] = tot;
+    if (tid == 0) partial[row * parts + blockIdx.x] = tot;
     __syncthreads();  // lds is reused by the next row
   }
 }
