@@ -152,4 +152,27 @@ __device__ __forceinline__ float block_sum(float v, float* lds) {
   return r;
 }
 
+// Number of non-zero mask bytes, counted by the calling workgroup (every
+// thread gets the result; `lds` holds NT / 64 floats).  The mask of a batch is
+// a few kilobytes, so this is an L2-resident read and one block reduction --
+// cheaper than a counting launch in front when only the workgroups of the
+// selected rows need the number.
+template <int NT>
+__device__ __forceinline__ float mask_count_block(const uint8_t* __restrict__ mask, int64_t n, float* lds) {
+  int c = 0;
+  const int64_t n8 = ((uintptr_t)mask & 7u) == 0 ? n / 8 : 0;
+  const uint64_t* m8 = reinterpret_cast<const uint64_t*>(mask);
+  for (int64_t i = threadIdx.x; i < n8; i += NT) {
+    uint64_t v = m8[i];
+    // a byte counts when any of its bits is set
+    v |= v >> 4;
+    v |= v >> 2;
+    v |= v >> 1;
+    c += __popcll(v & 0x0101010101010101ull);
+  }
+  for (int64_t i = n8 * 8 + threadIdx.x; i < n; i += NT) c += mask[i] != 0;
+  // per-thread counts stay far below 2^24 for any n the launchers accept: the float sum is exact
+  return block_sum<NT / kWave>((float)c, lds);
+}
+
 }  // namespace ts

@@ -219,29 +219,6 @@ __device__ __forceinline__ RowJob row_job(const KdArgs& a, int64_t row) {
   return j;
 }
 
-// Number of non-zero mask bytes, counted by the calling workgroup (every
-// thread gets the result; `lds` holds NT / 64 floats).  The mask of a batch is
-// a few kilobytes, so this is an L2-resident read and one block reduction --
-// cheaper than a counting launch in front when only the workgroups of the
-// selected rows need the number.
-template <int NT>
-__device__ __forceinline__ float kd_mask_count(const uint8_t* __restrict__ mask, int64_t n, float* lds) {
-  int c = 0;
-  const int64_t n8 = ((uintptr_t)mask & 7u) == 0 ? n / 8 : 0;
-  const uint64_t* m8 = reinterpret_cast<const uint64_t*>(mask);
-  for (int64_t i = threadIdx.x; i < n8; i += NT) {
-    uint64_t v = m8[i];
-    // a byte counts when any of its bits is set
-    v |= v >> 4;
-    v |= v >> 2;
-    v |= v >> 1;
-    c += __popcll(v & 0x0101010101010101ull);
-  }
-  for (int64_t i = n8 * 8 + threadIdx.x; i < n; i += NT) c += mask[i] != 0;
-  // per-thread counts stay far below 2^24 for any n the launchers accept: the float sum is exact
-  return block_sum<NT / kWave>((float)c, lds);
-}
-
 // Final per-row numbers from the merged states.
 struct RowFinal {
   float lse_t, lse_s, lse1;  // log2 domain
@@ -405,7 +382,7 @@ __global__ __launch_bounds__(BLOCK, (KREG * GROUP > 1024 ? 4 : 1)) void kd_rows_
   // row's loads are in flight.  One row per workgroup in that case, so the
   // branch is uniform.
   float n_kd_counted = 0.f;
-  if (GROUP == BLOCK && a.self_count) n_kd_counted = kd_mask_count<BLOCK>(a.mask, a.n_rows, lds_cnt);
+  if (GROUP == BLOCK && a.self_count) n_kd_counted = mask_count_block<BLOCK>(a.mask, a.n_rows, lds_cnt);
 
   // Rows whose operands share one alignment (the usual case): all but a few
   // end elements are 16-byte vectors held in registers, and each of those end
@@ -974,7 +951,7 @@ __global__ __launch_bounds__(1024) void kd_finalize_kernel(const float* __restri
                                                            const uint8_t* __restrict__ mask /* ... or, if set, the rows it selects */,
                                                            float* __restrict__ out) {
   __shared__ float lds[1024 / kWave];
-  const float n_masked = (!counts && mask) ? kd_mask_count<1024>(mask, n, lds) : 0.f;
+  const float n_masked = (!counts && mask) ? mask_count_block<1024>(mask, n, lds) : 0.f;
   // 16-byte loads, eight of them in flight per thread and array: one block
   // has to get through the whole array, so the loop is bound by memory latency
   // (65536 rows are two round trips this way)

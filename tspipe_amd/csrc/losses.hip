@@ -213,9 +213,13 @@ inline int row_pieces(const void* const* a, const void* const* b, void* const* g
 //   loss  = weight * mean over selected rows of (1 - cos_i);  gradient to x only.
 template <typename T>
 __global__ __launch_bounds__(256) void cosine_rows_kernel(const RowPieces tab, const uint8_t* __restrict__ mask,
-                                                          const int* __restrict__ n_sel_dev, int64_t n, int64_t c,
-                                                          float weight, float* __restrict__ row_loss) {
+                                                          int64_t n, int64_t c, float weight,
+                                                          float* __restrict__ row_loss) {
   constexpr float kEps = 1e-12f;
+  __shared__ float lds_cnt[256 / kWave];
+  // the number of selected rows scales the gradient: every workgroup counts the
+  // mask's few kilobytes itself (no counting launch in front)
+  const float n_sel = mask ? mask_count_block<256>(mask, n, lds_cnt) : (float)n;
   const int lane = threadIdx.x % kWave;
   const int64_t row = (int64_t)blockIdx.x * (256 / kWave) + threadIdx.x / kWave;
   if (row >= n) return;
@@ -243,13 +247,26 @@ __global__ __launch_bounds__(256) void cosine_rows_kernel(const RowPieces tab, c
   const float cosv = sxy * inv_den;
   if (lane == 0) row_loss[row] = 1.f - cosv;
   if (!gr) return;
-  const float B = n_sel_dev ? (float)(*n_sel_dev) : (float)n;
-  const float k = -weight / B;
+  const float k = -weight / n_sel;
   const float proj = cosv / sxx;
   for (int64_t i = lane; i < c; i += kWave) {
     const float a = to_f32(xr[i]), b = to_f32(yr[i]);
     gr[i] = from_f32<T>(k * (b * inv_den - proj * a));
   }
+}
+
+// loss = weight * sum(row_loss) / selected rows, fixed summation order; the
+// workgroup counts the mask itself.  0/0 = NaN for an empty selection, as the
+// reference gives.
+__global__ __launch_bounds__(1024) void cosine_finalize_kernel(const float* __restrict__ row_loss, int64_t n,
+                                                               float weight, const uint8_t* __restrict__ mask,
+                                                               float* __restrict__ out) {
+  __shared__ float lds[1024 / kWave];
+  const float n_sel = mask ? mask_count_block<1024>(mask, n, lds) : (float)n;
+  float acc = 0.f;
+  for (int64_t i = threadIdx.x; i < n; i += 1024) acc += row_loss[i];
+  const float tot = block_sum<1024 / kWave>(acc, lds);
+  if (threadIdx.x == 0) *out = weight * (tot / n_sel);
 }
 
 // ---- squared error between logits (fused backward) -----------------------
@@ -400,19 +417,12 @@ int launch_mse(const RowPieces& tab, const uint8_t* mask, int64_t n_rows, int64_
 template <typename T>
 int launch_cosine(const RowPieces& tab, const uint8_t* mask, int64_t n, int64_t c, float weight, void* ws,
                   float* loss_out, hipStream_t stream) {
-  int* n_sel = reinterpret_cast<int*>(ws);
   float* row_loss = reinterpret_cast<float*>(reinterpret_cast<char*>(ws) + 16);
-  if (mask) {
-    hipLaunchKernelGGL(mask_count_kernel, dim3(1), dim3(1024), 0, stream, mask, n, n_sel);
-    int rc = check_launch();
-    if (rc) return rc;
-  }
-  hipLaunchKernelGGL((cosine_rows_kernel<T>), dim3((unsigned)((n + 3) / 4)), dim3(256), 0, stream, tab, mask,
-                     mask ? n_sel : (const int*)nullptr, n, c, weight, row_loss);
+  hipLaunchKernelGGL((cosine_rows_kernel<T>), dim3((unsigned)((n + 3) / 4)), dim3(256), 0, stream, tab, mask, n, c,
+                     weight, row_loss);
   int rc = check_launch();
   if (rc) return rc;
-  hipLaunchKernelGGL(sum_scale_kernel, dim3(1), dim3(1024), 0, stream, row_loss, n, weight,
-                     mask ? n_sel : (const int*)nullptr, (float)n, loss_out);
+  hipLaunchKernelGGL(cosine_finalize_kernel, dim3(1), dim3(1024), 0, stream, row_loss, n, weight, mask, loss_out);
   return check_launch();
 }
 
