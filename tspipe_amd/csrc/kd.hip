@@ -152,7 +152,7 @@ struct KdArgs {
   float kd_gscale;  // kd_scale * inv_T   (gradient factor of the KD term before the 1/B)
   float ce_weight;
   const int* counts;  // device: [0] KD rows, [1] CE rows, [2] rows with any term; null = all n_rows carry KD only
-  int self_count;     // counts is null although a mask selects rows: whoever needs the number of KD rows counts the mask bytes
+  int self_count;     // counts is null although a mask or labels select rows: whoever needs the numbers of KD / CE rows counts them
   float* row_kd;      // per-row KD loss terms (0 for unselected rows)
   float* row_ce;      // per-row CE loss terms
   void* grad;         // may be null
@@ -225,16 +225,30 @@ struct RowFinal {
   float g_kd, g_ce;          // gradient factors (0 when the term is off for this row)
 };
 
+// Number of rows whose label selects a class (not the ignore index, inside
+// [0, V)), counted by the calling workgroup like mask_count_block.
+template <int NT>
+__device__ __forceinline__ float label_count_block(const int64_t* __restrict__ labels, int64_t n, int64_t ignore_index,
+                                                   int64_t V, float* lds) {
+  int c = 0;
+  for (int64_t i = threadIdx.x; i < n; i += NT) {
+    const int64_t l = labels[i];
+    c += (l != ignore_index && l >= 0 && l < V) ? 1 : 0;
+  }
+  return block_sum<NT / kWave>((float)c, lds);
+}
+
 template <typename T, bool CE>
 __device__ __forceinline__ RowFinal finish_row(const KdArgs& a, const RowJob& j, int64_t row, const TStat& st,
-                                               const SStat& ss, const T* srow, bool writer, float n_kd_counted = 0.f) {
+                                               const SStat& ss, const T* srow, bool writer, float n_kd_counted = 0.f,
+                                               float n_ce_counted = 0.f) {
   RowFinal f;
   f.lse_t = st.m * a.k + log2f(st.z);
   f.lse_s = ss.m * a.k + log2f(ss.z);
   f.lse1 = CE ? ss.m * kLog2e + log2f(ss.z1) : 0.f;
   const float n_kd = a.self_count ? n_kd_counted : (a.counts ? (float)a.counts[0] : (float)a.n_rows);
   f.g_kd = j.kd ? a.kd_gscale / n_kd : 0.f;
-  f.g_ce = (CE && j.ce) ? a.ce_weight / (float)a.counts[1] : 0.f;
+  f.g_ce = (CE && j.ce) ? a.ce_weight / (a.self_count ? n_ce_counted : (float)a.counts[1]) : 0.f;
   if (writer) {
     a.row_kd[row] = j.kd ? kLn2 * (a.k * st.a / st.z - f.lse_t + f.lse_s) : 0.f;
     if (CE) a.row_ce[row] = j.ce ? kLn2 * (f.lse1 - to_f32(srow[j.label]) * kLog2e) : 0.f;
@@ -377,12 +391,15 @@ __global__ __launch_bounds__(BLOCK, (KREG * GROUP > 1024 ? 4 : 1)) void kd_rows_
       }
     }
   }
-  // No counting launch ran in front (mask-only call on long rows): the number
-  // of selected rows, which scales the gradient, is counted here while the
-  // row's loads are in flight.  One row per workgroup in that case, so the
+  // No counting launch ran in front (long rows under a mask and / or with
+  // labels): the numbers of rows with a KD and with a CE term, which scale the
+  // gradient, are counted here while the row's loads are in flight.  One row per workgroup in that case, so the
   // branch is uniform.
-  float n_kd_counted = 0.f;
-  if (GROUP == BLOCK && a.self_count) n_kd_counted = mask_count_block<BLOCK>(a.mask, a.n_rows, lds_cnt);
+  float n_kd_counted = 0.f, n_ce_counted = 0.f;
+  if (GROUP == BLOCK && a.self_count) {
+    n_kd_counted = a.mask ? mask_count_block<BLOCK>(a.mask, a.n_rows, lds_cnt) : (float)a.n_rows;
+    if (CE && a.labels) n_ce_counted = label_count_block<BLOCK>(a.labels, a.n_rows, a.ignore_index, a.V, lds_cnt);
+  }
 
   // Rows whose operands share one alignment (the usual case): all but a few
   // end elements are 16-byte vectors held in registers, and each of those end
@@ -518,7 +535,7 @@ __global__ __launch_bounds__(BLOCK, (KREG * GROUP > 1024 ? 4 : 1)) void kd_rows_
       }
     }
     const RowFinal f =
-        finish_row<T, CE>(a, job, row, TStat{mt, zt, at}, SStat{ms, zs, z1}, srow, gtid == 0, n_kd_counted);
+        finish_row<T, CE>(a, job, row, TStat{mt, zt, at}, SStat{ms, zs, z1}, srow, gtid == 0, n_kd_counted, n_ce_counted);
     if (!grow) return;
     // probabilities first and the weight last, as everywhere in this file
     const float rt_ = 1.f / zt, rs_ = 1.f / zs, r1_ = CE ? 1.f / z1 : 0.f;
@@ -611,7 +628,7 @@ __global__ __launch_bounds__(BLOCK, (KREG * GROUP > 1024 ? 4 : 1)) void kd_rows_
     }
   }
 
-  const RowFinal f = finish_row<T, CE>(a, job, row, st, ss, srow, gtid == 0, n_kd_counted);
+  const RowFinal f = finish_row<T, CE>(a, job, row, st, ss, srow, gtid == 0, n_kd_counted, n_ce_counted);
   if (!grow) return;
 
   for (int64_t i = gtid; i < g.head; i += GROUP) grow[i] = grad_one<T, CE>(trow[i], srow[i], i == job.label, a.k, f);
@@ -944,14 +961,18 @@ __global__ __launch_bounds__(1024) void kd_count_kernel(const KdArgs a, int* __r
 }
 
 // loss = kd_scale * sum(row_kd) / counts[0] + ce_weight * sum(row_ce) / counts[1], fixed summation order.
+// Without counts the workgroup takes the two numbers from the mask (null: all
+// n rows carry the KD term) and the labels themselves.
 __global__ __launch_bounds__(1024) void kd_finalize_kernel(const float* __restrict__ row_kd,
                                                            const float* __restrict__ row_ce, int64_t n,
                                                            float kd_scale, float ce_weight,
-                                                           const int* __restrict__ counts /* null: n KD rows ... */,
-                                                           const uint8_t* __restrict__ mask /* ... or, if set, the rows it selects */,
-                                                           float* __restrict__ out) {
+                                                           const int* __restrict__ counts,
+                                                           const uint8_t* __restrict__ mask,
+                                                           const int64_t* __restrict__ labels, int64_t ignore_index,
+                                                           int64_t V, float* __restrict__ out) {
   __shared__ float lds[1024 / kWave];
   const float n_masked = (!counts && mask) ? mask_count_block<1024>(mask, n, lds) : 0.f;
+  const float n_labelled = (!counts && row_ce && labels) ? label_count_block<1024>(labels, n, ignore_index, V, lds) : 0.f;
   // 16-byte loads, eight of them in flight per thread and array: one block
   // has to get through the whole array, so the loop is bound by memory latency
   // (65536 rows are two round trips this way)
@@ -987,7 +1008,7 @@ __global__ __launch_bounds__(1024) void kd_finalize_kernel(const float* __restri
   if (threadIdx.x == 0) {
     // 0/0 = NaN for an empty selection, as the reference gives
     float loss = kd_scale * (skd / (counts ? (float)counts[0] : (mask ? n_masked : (float)n)));
-    if (row_ce) loss += ce_weight * (sce / (float)counts[1]);
+    if (row_ce) loss += ce_weight * (sce / (counts ? (float)counts[1] : n_labelled));
     *out = loss;
   }
 }
@@ -1048,12 +1069,12 @@ int launch_kd_t(KdArgs a, float kd_scale, void* ws, float* loss_out, hipStream_t
   // most are.  The two passes remain for wider or differently aligned rows.
   const bool one_launch = a.n_rows > 0 && parts > 0 && vecs_ <= 1024 * 8 && kd_rows_aligned_alike<T>(a);
   const bool wide = a.n_rows > 0 && parts > 0 && !one_launch;
-  // A mask without labels on such rows needs no launch in front: the only
-  // number the row kernel wants, the count of selected rows, each of its
-  // workgroups takes from the mask itself (a few kilobytes), and so does the
-  // final reduction.
-  const bool self_count = one_launch && a.mask && !a.labels;
-  const bool compacted = one_launch && a.mask && !self_count;  // the row kernel walks the compacted list, then zero-fills
+  // Such rows need no counting launch in front: the numbers the row kernel
+  // wants, the counts of rows with a KD and with a CE term, each of its
+  // workgroups takes from the mask and the labels themselves (a few
+  // kilobytes each), and so does the final reduction.
+  const bool self_count = one_launch && counted;
+  const bool compacted = false;  // (the row kernel can also walk a compacted list of rows with a term)
   a.self_count = self_count ? 1 : 0;
   if (self_count) a.counts = nullptr;
   if (counted && !wide && !self_count) {
@@ -1065,7 +1086,7 @@ int launch_kd_t(KdArgs a, float kd_scale, void* ws, float* loss_out, hipStream_t
   if (a.n_rows == 0) {
     hipLaunchKernelGGL(kd_finalize_kernel, dim3(1), dim3(1024), 0, stream, w.row_kd,
                        CE ? w.row_ce : (const float*)nullptr, (int64_t)0, kd_scale, a.ce_weight, a.counts,
-                       (const uint8_t*)nullptr, loss_out);
+                       (const uint8_t*)nullptr, (const int64_t*)nullptr, a.ignore_index, a.V, loss_out);
     return check_launch();
   }
   // 16-byte vectors a row can span, counting a ragged first and last one
@@ -1084,7 +1105,8 @@ int launch_kd_t(KdArgs a, float kd_scale, void* ws, float* loss_out, hipStream_t
     TS_KD_LAUNCH(256, 256, 4);
   } else if (one_launch) {
     if (2 * a.n_rows > 0x7fffffffLL) return TS_ERR_RANGE;
-    const dim3 grid((unsigned)((compacted || self_count) ? 2 * a.n_rows : a.n_rows));
+    // a second half of zero-filling workgroups only where rows without a term can exist
+    const dim3 grid((unsigned)((compacted || (self_count && a.mask)) ? 2 * a.n_rows : a.n_rows));
     const int* sel = compacted ? w.sel_rows : nullptr;
     if (vecs <= 512 * 8)
       hipLaunchKernelGGL((kd_rows_kernel<T, 512, 512, 8, CE>), grid, dim3(512), 0, stream, a, sel);
@@ -1106,7 +1128,8 @@ int launch_kd_t(KdArgs a, float kd_scale, void* ws, float* loss_out, hipStream_t
   rc = check_launch();
   if (rc) return rc;
   hipLaunchKernelGGL(kd_finalize_kernel, dim3(1), dim3(1024), 0, stream, w.row_kd, CE ? w.row_ce : (const float*)nullptr,
-                     a.n_rows, kd_scale, a.ce_weight, a.counts, self_count ? a.mask : (const uint8_t*)nullptr, loss_out);
+                     a.n_rows, kd_scale, a.ce_weight, a.counts, self_count ? a.mask : (const uint8_t*)nullptr,
+                     self_count ? a.labels : (const int64_t*)nullptr, a.ignore_index, a.V, loss_out);
   return check_launch();
 }
 
