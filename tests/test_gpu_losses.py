@@ -577,8 +577,32 @@ def test_distil_loss_fn_clm_and_mse_terms(device, mode):
     assert ((sd.grad.cpu().double() - gs).abs() <= 1e-3 * peak + gs.abs() * 2.0 ** -6).all()
 
 
+def test_logits_mse_operands_aligned_differently(device):
+    # s and t at different offsets from a 16-byte boundary (views into larger buffers): the kernel
+    # walks such rows element by element; rows of 2051 elements also exercise a second span
+    g = seeded(77)
+    rows, V = 9, 2051
+    for dtype, tol in ((torch.float32, 1e-5), (torch.bfloat16, 1e-3)):
+        s = (torch.randn(rows, V, generator=g) * 3).to(dtype)
+        t = (torch.randn(rows, V, generator=g) * 3).to(dtype)
+        want, (gw,) = _oracle_grad(lambda a, b: ts_oracle.logits_mse(a, b), s, others=(t,))
+        buf_s = torch.zeros(rows * V + 8, dtype=dtype, device=device)
+        buf_t = torch.zeros(rows * V + 8, dtype=dtype, device=device)
+        sd = buf_s[1:1 + rows * V].view(rows, V)
+        td = buf_t[3:3 + rows * V].view(rows, V)
+        sd.copy_(s)
+        td.copy_(t)
+        sd = sd.detach().requires_grad_()
+        loss = ta.logits_mse_loss(sd, td)
+        loss.backward()
+        assert rel_err(loss.item(), want) < tol
+        slack = gw.abs() * (2.0 ** -8 if dtype != torch.float32 else 0.0)
+        assert ((sd.grad.cpu().double() - gw).abs() <= tol * gw.abs().max().item() + slack).all()
+
+
 @pytest.mark.parametrize("rows,V,dtype", [(256, 100, torch.float32), (33, 5000, torch.float32),
-                                          (40, 30522, torch.bfloat16)])
+                                          (40, 30522, torch.bfloat16), (37, 101, torch.float32),
+                                          (19, 1001, torch.bfloat16)])
 def test_logits_mse_and_kd_mode_logits(device, rows, V, dtype):
     from argparse import Namespace
     g = seeded(240 + V)
