@@ -201,3 +201,14 @@ def test_device_entry_points_validate_before_launching():
     assert lib.ts_cosine_workspace_bytes(5) == 48
     assert lib.ts_infonce_workspace_bytes(4096, 256, 1) > 4096 * 256 * 4
     assert lib.ts_infonce_workspace_bytes(4096, 256, 3) == 0
+
+
+def test_measurement_variants_name_macros_their_sources_use():
+    # `python -m tspipe_amd.build --variant NAME` rebuilds one source under macros: each macro must
+    # exist in that source, or the variant would silently equal the default build
+    from tspipe_amd import build
+    for name, (src, defines) in build.VARIANTS.items():
+        text = open(os.path.join(build.CSRC, src)).read()
+        assert src in build.SOURCES, name
+        for d in defines:
+            assert f"#ifdef {d}" in text, (name, d)
