@@ -684,38 +684,55 @@ __global__ __launch_bounds__(kNceMainBlock) void nce_main_kernel(NceArgs args, i
 //   l_i = (l~_i - P~_ii) + P_ii  (the positive term unrounded).
 // Re-deriving l_i here instead of reading the other workgroups' results keeps
 // the reduction inside this launch; the order of every addition is fixed.
-// Four rows per thread and trip, all loads of a trip issued before the first use.
-template <int NT>
+// QN x 4 rows per thread and trip, all loads of a trip issued before the first
+// use: the workgroup walks the whole batch alone, so its time is the number
+// of trips times the memory latency.  SC: splits requested in one go, as in the
+// combine kernel (QN shrinks as SC grows; the registers are what bounds both).
+template <int NT, int SC>
 __device__ __forceinline__ void nce_loss_block(const NceArgs& args, int pairs, int64_t n, int64_t npad, int splits,
                                                float loss_scale, float* __restrict__ loss_out) {
   __shared__ float red[NT / kWave];
   const int tid = threadIdx.x;
-  constexpr int SC = 8;  // splits per batch of loads
+  constexpr int QN = SC == 2 ? 4 : (SC == 4 ? 2 : 1);
   float acc = 0.f;
   for (int p = 0; p < pairs; ++p) {
     const float* __restrict__ lpart = args.p[p].lpart;
     const float* __restrict__ pdiag = args.p[p].pdiag;
-    for (int64_t quad = tid; quad < npad / 4; quad += NT) {
-      const f32x4 d0 = *reinterpret_cast<const f32x4*>(pdiag + 8 * quad);      // rows 4q, 4q+1: exact, rounded
-      const f32x4 d1 = *reinterpret_cast<const f32x4*>(pdiag + 8 * quad + 4);  // rows 4q+2, 4q+3
-      f32x4 l = {0.f, 0.f, 0.f, 0.f};
-      for (int s0 = 0; s0 < splits; s0 += SC) {
-        f32x4 v[SC];
-        float keep[SC];
+    const int64_t nquad = npad / 4;
+    for (int64_t q0 = tid; q0 < nquad; q0 += (int64_t)NT * QN) {
+      f32x4 d0[QN], d1[QN], l[QN];
 #pragma unroll
-        for (int c = 0; c < SC; ++c) {
-          keep[c] = s0 + c < splits ? 1.f : 0.f;
-          const int sp = s0 + c < splits ? s0 + c : s0;
-          v[c] = *reinterpret_cast<const f32x4*>(lpart + (int64_t)sp * npad + 4 * quad);
+      for (int u = 0; u < QN; ++u) {
+        const int64_t quad = q0 + (int64_t)u * NT < nquad ? q0 + (int64_t)u * NT : q0;  // beyond the end: re-read, dropped below
+        d0[u] = *reinterpret_cast<const f32x4*>(pdiag + 8 * quad);      // rows 4q, 4q+1: exact, rounded
+        d1[u] = *reinterpret_cast<const f32x4*>(pdiag + 8 * quad + 4);  // rows 4q+2, 4q+3
+        l[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+      }
+      for (int s0 = 0; s0 < splits; s0 += SC) {
+        f32x4 v[QN][SC];
+#pragma unroll
+        for (int u = 0; u < QN; ++u) {
+          const int64_t quad = q0 + (int64_t)u * NT < nquad ? q0 + (int64_t)u * NT : q0;
+#pragma unroll
+          for (int c = 0; c < SC; ++c) {
+            const int sp = s0 + c < splits ? s0 + c : s0;
+            v[u][c] = *reinterpret_cast<const f32x4*>(lpart + (int64_t)sp * npad + 4 * quad);
+          }
         }
 #pragma unroll
-        for (int c = 0; c < SC; ++c) l += v[c] * keep[c];
-      }
-      const float pe[4] = {d0[0], d0[2], d1[0], d1[2]}, pr[4] = {d0[1], d0[3], d1[1], d1[3]};
+        for (int u = 0; u < QN; ++u)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const float t = kNceLn2 * (log2f((l[j] - pr[j]) + pe[j]) - log2f(pe[j]));
-        acc += (4 * quad + j < n) ? t : 0.f;
+          for (int c = 0; c < SC; ++c) l[u] += v[u][c] * (s0 + c < splits ? 1.f : 0.f);
+      }
+#pragma unroll
+      for (int u = 0; u < QN; ++u) {
+        const int64_t quad = q0 + (int64_t)u * NT;
+        const float pe[4] = {d0[u][0], d0[u][2], d1[u][0], d1[u][2]}, pr[4] = {d0[u][1], d0[u][3], d1[u][1], d1[u][3]};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float t = kNceLn2 * (log2f((l[u][j] - pr[j]) + pe[j]) - log2f(pe[j]));
+          acc += (quad < nquad && 4 * quad + j < n) ? t : 0.f;
+        }
       }
     }
   }
@@ -744,7 +761,7 @@ __global__ __launch_bounds__(2 * C) void nce_combine_kernel(NceArgs args, int64_
   const int64_t units = npad / 16;
   if (blockIdx.x >= units) {
     if (blockIdx.x == units && blockIdx.z == 0)
-      nce_loss_block<2 * C>(args, (int)gridDim.z, n, npad, splits, loss_scale, loss_out);
+      nce_loss_block<2 * C, SC>(args, (int)gridDim.z, n, npad, splits, loss_scale, loss_out);
     return;
   }
   // Workgroup ids are dealt round-robin to the 8 XCDs and the grid's width is
