@@ -520,6 +520,62 @@ def run_kernel_table(dev, with_cpu=True):
         f"n_sel={n_sel_avg:.0f} on average; bytes = read s,t + write grad for selected rows, zero-fill of the other rows",
         KD_MASKED_LAUNCHES, working_set=2 * 3 * 4096 * row_b, sets=2, resident_ms=_time_stream(fns[0]),
         resident_note=ONE_SET_NOTE)
+    # the rest of TSPipeDistiller.loss_fn on the same two sets (not benchmark configurations of their own):
+    # KD + masked-LM cross-entropy in one pass (alpha_mlm > 0, restrict_ce_to_mask), the squared-error term on
+    # the logits, the cosine term on [32, 128, 768] hidden states
+    def kdce_call(d, grad):
+        labels = torch.full((4096,), -100, dtype=torch.long)
+        m_host = d["mask"].reshape(-1).cpu()
+        labels[m_host] = torch.randint(0, 30522, (int(m_host.sum()),), generator=g)
+        labels = labels.to(dev)
+        ws = torch.empty(lib.ts_kd_workspace_bytes(4096, 30522, _lib.TS_BF16), dtype=torch.uint8, device=dev)
+        loss = torch.empty((), device=dev)
+        mptr = d["mask"].view(torch.uint8).data_ptr()
+
+        def f():
+            _lib.check(lib.ts_kdce_fwd_bwd(d["s_full"].data_ptr(), d["t_full"].data_ptr(), mptr, labels.data_ptr(), -100,
+                                           4096, 30522, 30522, 30522, 0.5, 4.0 * 0.5, 2.0, ws.data_ptr(), loss.data_ptr(),
+                                           grad.data_ptr(), 30522, _lib.TS_BF16, stream), "ts_kdce_fwd_bwd")
+        f.keep = (labels, ws, loss, grad)
+        return f
+
+    def mse_call(d, grad):
+        ws = torch.empty(lib.ts_mse_workspace_bytes(4096, 30522), dtype=torch.uint8, device=dev)
+        loss = torch.empty((), device=dev)
+        mptr = d["mask"].view(torch.uint8).data_ptr()
+
+        def f():
+            _lib.check(lib.ts_mse_fwd_bwd(d["s_full"].data_ptr(), d["t_full"].data_ptr(), mptr, 4096, 30522, 30522, 30522,
+                                          0.1, 0, 0, ws.data_ptr(), loss.data_ptr(), grad.data_ptr(), 30522, _lib.TS_BF16,
+                                          stream), "ts_mse_fwd_bwd")
+        f.keep = (ws, loss, grad)
+        return f
+    grads = [torch.empty_like(d["s_full"]) for d in sets]
+    fns2 = [kdce_call(d, gr) for d, gr in zip(sets, grads)]
+    out["kdce_masked_32x128x30522_bf16"] = entry(
+        kd_bytes, _time_stream(rotate(fns2), batch=2),
+        "KD + cross-entropy on the masked tokens in one pass (distiller.py:719-744), two sets of logits in turn", 2,
+        working_set=2 * 3 * 4096 * row_b, sets=2)
+    fns2 = [mse_call(d, gr) for d, gr in zip(sets, grads)]
+    out["mse_masked_32x128x30522_bf16"] = entry(
+        kd_bytes, _time_stream(rotate(fns2), batch=2),
+        "squared-error term on the masked tokens (distiller.py:751-755): counting launch, rows, final sum", 3,
+        working_set=2 * 3 * 4096 * row_b, sets=2)
+    del fns2, grads
+    hid = [torch.randn(4096, 768, generator=g).to(dev) for _ in range(2)]
+    ghid = torch.empty_like(hid[0])
+    ws_c = torch.empty(lib.ts_cosine_workspace_bytes(4096), dtype=torch.uint8, device=dev)
+    loss_c = torch.empty((), device=dev)
+
+    def f_cos():
+        _lib.check(lib.ts_cosine_fwd_bwd(hid[0].data_ptr(), hid[1].data_ptr(), sets[0]["mask"].view(torch.uint8).data_ptr(),
+                                         4096, 768, 1.0, ws_c.data_ptr(), loss_c.data_ptr(), ghid.data_ptr(), _lib.TS_F32,
+                                         stream), "ts_cosine_fwd_bwd")
+    n0 = int(sets[0]["mask"].sum().item())
+    out["cosine_masked_4096x768_f32"] = entry(
+        (3 * n0 + (4096 - n0)) * 768 * 4, _time_stream(f_cos),
+        "cosine term on the hidden states (distiller.py:756-770); latency-bound", 2, working_set=3 * 4096 * 768 * 4)
+    del hid, ghid
     if with_cpu:
         d = sets[0]
         s_c, t_c, m_c = d["s_full"].cpu(), d["t_full"].cpu(), d["mask"].cpu()
