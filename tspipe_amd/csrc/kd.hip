@@ -151,6 +151,7 @@ struct KdArgs {
   float k;          // inv_T * log2(e)
   float kd_gscale;  // kd_scale * inv_T   (gradient factor of the KD term before the 1/B)
   float ce_weight;
+  int t_pow;        // the temperature when it is exactly 1, 2 or 4 (then 2^x at temperature 1 is a power of 2^x at T), else 0
   const int* counts;  // device: [0] KD rows, [1] CE rows, [2] rows with any term; null = all n_rows carry KD only
   int self_count;     // counts is null although a mask or labels select rows: whoever needs the numbers of KD / CE rows counts them
   float* row_kd;      // per-row KD loss terms (0 for unselected rows)
@@ -470,6 +471,18 @@ __global__ __launch_bounds__(BLOCK, (KREG * GROUP > 1024 ? 4 : 1)) void kd_rows_
       }
     }
     const float mtk = mt * a.k, msk = ms * a.k, ms1 = ms * kLog2e;
+    // The CE term wants 2^((s - m) log2e), the KD term has 2^((s - m) log2e / T):
+    // for T = 1, 2, 4 the first is a power of the second, two multiplies at
+    // most instead of a v_exp_f32 (a quarter-rate instruction in a kernel
+    // that is bound by its vector arithmetic).  t_pow is uniform.
+    const int t_pow = CE ? a.t_pow : 0;
+    auto e1_of = [&](float sv, float es) {
+      if (t_pow == 0) return fast_exp2(fmaf(sv, kLog2e, -ms1));
+      float e = es;
+      if (t_pow >= 2) e *= e;
+      if (t_pow == 4) e *= e;
+      return e;
+    };
     // fp32 rows: the second walk leaves its exponentials where the logits
     // were (the student's logit stays when the CE term needs it at temperature
     // 1), so the gradient walk takes none again.  16-bit rows retake them: a
@@ -480,10 +493,11 @@ __global__ __launch_bounds__(BLOCK, (KREG * GROUP > 1024 ? 4 : 1)) void kd_rows_
     if (__any(has_h || has_t)) {
       auto add = [&](float tv, float sv) {
         const float et = fast_exp2(fmaf(tv, a.k, -mtk));
+        const float es = fast_exp2(fmaf(sv, a.k, -msk));
         zt += et;
-        zs += fast_exp2(fmaf(sv, a.k, -msk));
+        zs += es;
         at = acc_weighted_diff(et, tv, sv, at);
-        if (CE) z1 += fast_exp2(fmaf(sv, kLog2e, -ms1));
+        if (CE) z1 += e1_of(sv, es);
       };
       add(eh_t, eh_s);
       add(el_t, el_s);
@@ -500,7 +514,7 @@ __global__ __launch_bounds__(BLOCK, (KREG * GROUP > 1024 ? 4 : 1)) void kd_rows_
           zt += et;
           zs += es;
           at = acc_weighted_diff(et, tv, sv, at);
-          if (CE) z1 += fast_exp2(fmaf(sv, kLog2e, -ms1));
+          if (CE) z1 += e1_of(sv, es);
           if constexpr (kKeep) {
             rt[j].v[i] = et;
             if (!CE) rs[j].v[i] = es;
@@ -544,10 +558,7 @@ __global__ __launch_bounds__(BLOCK, (KREG * GROUP > 1024 ? 4 : 1)) void kd_rows_
       const float et = fast_exp2(fmaf(tv, a.k, -mtk));
       const float es = fast_exp2(fmaf(sv, a.k, -msk));
       float gv = f.g_kd * fmaf(es, rs_, -(et * rt_));
-      if (CE) {
-        const float e1 = fast_exp2(fmaf(sv, kLog2e, -ms1));
-        gv = fmaf(f.g_ce, fmaf(e1, r1_, col == label ? -1.f : 0.f), gv);
-      }
+      if (CE) gv = fmaf(f.g_ce, fmaf(e1_of(sv, es), r1_, col == label ? -1.f : 0.f), gv);
       return from_f32<T>(gv);
     };
     if (has_h) grow[gtid] = grad_of(eh_t, eh_s, gtid);
@@ -565,9 +576,8 @@ __global__ __launch_bounds__(BLOCK, (KREG * GROUP > 1024 ? 4 : 1)) void kd_rows_
             if (CE) {
               const float sv = rs[j].v[i];
               const float es = fast_exp2(fmaf(sv, a.k, -msk));
-              const float e1 = fast_exp2(fmaf(sv, kLog2e, -ms1));
               const float gv = f.g_kd * fmaf(es, rs_, -pt);
-              o.v[i] = fmaf(f.g_ce, fmaf(e1, r1_, e0 + i == label ? -1.f : 0.f), gv);
+              o.v[i] = fmaf(f.g_ce, fmaf(e1_of(sv, es), r1_, e0 + i == label ? -1.f : 0.f), gv);
             } else {
               o.v[i] = f.g_kd * fmaf(rs[j].v[i], rs_, -pt);
             }
@@ -1013,6 +1023,9 @@ __global__ __launch_bounds__(1024) void kd_finalize_kernel(const float* __restri
   }
 }
 
+// 1, 2 or 4 when the temperature is exactly that, else 0 (KdArgs::t_pow).
+inline int kd_t_pow(float inv_T) { return inv_T == 1.f ? 1 : (inv_T == 0.5f ? 2 : (inv_T == 0.25f ? 4 : 0)); }
+
 struct KdWorkspace {
   int* counts;
   float* row_kd;
@@ -1178,6 +1191,7 @@ int ts_kdce_fwd_bwd(const void* s, const void* t, const uint8_t* row_mask, const
   a.k = inv_T * ts::kLog2e;
   a.kd_gscale = kd_scale * inv_T;
   a.ce_weight = ce_weight;
+  a.t_pow = ts::kd_t_pow(inv_T);
   a.counts = nullptr;
   a.self_count = 0;
   a.row_kd = a.row_ce = nullptr;
@@ -1237,6 +1251,7 @@ int ts_kdce_pieces_fwd_bwd(const void* const* s_pieces, const void* const* t_pie
   a.k = inv_T * ts::kLog2e;
   a.kd_gscale = kd_scale * inv_T;
   a.ce_weight = ce_weight;
+  a.t_pow = ts::kd_t_pow(inv_T);
   a.counts = nullptr;
   a.self_count = 0;
   a.row_kd = a.row_ce = nullptr;
