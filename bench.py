@@ -429,7 +429,8 @@ def run_kernel_table(dev, with_cpu=True):
     s = (torch.randn(256, 100, generator=g) * 3).to(dev)
     t = (torch.randn(256, 100, generator=g) * 3).to(dev)
     f = kd_call(s, t, None, 4.0, torch.empty_like(s))
-    out["kd_256x100_f32"] = entry(3 * 256 * 100 * 4, _time_stream(f), "latency-bound: one launch of a few us", 1)
+    out["kd_256x100_f32"] = entry(3 * 256 * 100 * 4, _time_stream(f), "cfg2 itself; latency-bound: two launches (rows, final sum)", 2,
+                                  working_set=3 * 256 * 100 * 4)
     cpu("kd_256x100_f32", kd_cpu(s, t, 4.0))
 
     def kd_sets(rows, V, n_sets):
