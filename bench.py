@@ -33,7 +33,7 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-STEP_NCE_WORKGROUPS = 32   # InfoNCE workgroup target inside the step: one key split, 32 long workgroups
+STEP_NCE_WORKGROUPS = 64   # InfoNCE workgroup target inside the step: two key splits, 64 long workgroups
 TIMED_EVERY = 4  # one EMA launch in four carries kernel timing events
 SETUP_STEPS = 12  # untimed calls before the warm-up steps (resource creation, see run_step_benchmark)
 HBM_PEAK_GBS = 8000.0       # MI355X published HBM3E bandwidth

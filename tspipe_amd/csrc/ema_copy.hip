@@ -13,6 +13,17 @@
 
 namespace ts {
 
+// The table hands out plain 64-bit addresses, which the compiler can only
+// treat as generic: it would use flat_load / flat_store, instructions that are
+// booked on the LDS counter as well.  All of them are device memory, so the
+// vector paths say so and get global_load / global_store.
+#define TS_GLOBAL __attribute__((address_space(1)))
+typedef TS_GLOBAL const f32x4* gc_f32x4_ptr;
+typedef TS_GLOBAL f32x4* g_f32x4_ptr;
+typedef TS_GLOBAL const u32x4* gc_u32x4_ptr;
+typedef TS_GLOBAL u32x4* g_u32x4_ptr;
+
+
 constexpr int kEmaBlock = 256;
 constexpr int kSubElems = kEmaBlock * 4;  // one 16-byte vector per thread and operand
 
@@ -49,15 +60,15 @@ __global__ __launch_bounds__(kEmaBlock) void ema_multi_kernel(const ts_ema_chunk
   if ((ch.flags & 1u) && (!CLONE || (clone_offset & 15) == 0)) {
     const uint32_t n4 = n >> 2;
     if (tid < n4) {
-      const f32x4 a = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(tp) + tid);
-      const f32x4 b = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(sp) + tid);
+      const f32x4 a = __builtin_nontemporal_load((gc_f32x4_ptr)tp + tid);
+      const f32x4 b = __builtin_nontemporal_load((gc_f32x4_ptr)sp + tid);
       f32x4 r;
       r.x = ema1(a.x, b.x, m, c);
       r.y = ema1(a.y, b.y, m, c);
       r.z = ema1(a.z, b.z, m, c);
       r.w = ema1(a.w, b.w, m, c);
-      __builtin_nontemporal_store(r, reinterpret_cast<f32x4*>(op) + tid);
-      if (CLONE) __builtin_nontemporal_store(b, reinterpret_cast<f32x4*>(cp) + tid);
+      __builtin_nontemporal_store(r, (g_f32x4_ptr)op + tid);
+      if (CLONE) __builtin_nontemporal_store(b, (g_f32x4_ptr)cp + tid);
     }
     const uint32_t rem = n & 3u;
     if (tid < rem) {
@@ -121,8 +132,8 @@ __global__ __launch_bounds__(kEmaBlock) void ema_multi_kernel_2byte(const ts_ema
   if (ch.flags & 1u) {
     const uint32_t n8 = n >> 3;
     if (tid < n8) {
-      const u32x4 ra = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(tp) + tid);
-      const u32x4 rb = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(sp) + tid);
+      const u32x4 ra = __builtin_nontemporal_load((gc_u32x4_ptr)tp + tid);
+      const u32x4 rb = __builtin_nontemporal_load((gc_u32x4_ptr)sp + tid);
       T a[8], b[8], r[8];
       __builtin_memcpy(a, &ra, 16);
       __builtin_memcpy(b, &rb, 16);
@@ -130,7 +141,7 @@ __global__ __launch_bounds__(kEmaBlock) void ema_multi_kernel_2byte(const ts_ema
       for (int e = 0; e < 8; ++e) r[e] = ema1_t<T>(a[e], b[e], m, c);
       u32x4 rr;
       __builtin_memcpy(&rr, r, 16);
-      __builtin_nontemporal_store(rr, reinterpret_cast<u32x4*>(op) + tid);
+      __builtin_nontemporal_store(rr, (g_u32x4_ptr)op + tid);
     }
     const uint32_t rem = n & 7u;
     if (tid < rem) {
@@ -165,8 +176,8 @@ __global__ __launch_bounds__(kCopyBlock) void copy_segments_kernel(const ts_copy
   if (ch.flags & 1u) {
     const uint32_t n16 = bytes >> 4;
     if (tid < n16) {
-      const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(s) + tid);
-      __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(d) + tid);
+      const u32x4 v = __builtin_nontemporal_load((gc_u32x4_ptr)s + tid);
+      __builtin_nontemporal_store(v, (g_u32x4_ptr)d + tid);
     }
     const uint32_t rem = bytes & 15u;
     if (tid < rem) d[(n16 << 4) + tid] = s[(n16 << 4) + tid];
