@@ -364,3 +364,26 @@ def test_arena_reuse_waits_for_announced_readers_and_can_be_switched_off(device)
     finally:
         ema_mod.set_recycling(True)
         ema_mod.release_pool()
+
+
+def test_ema_more_chunks_than_a_grid_dimension_holds(device):
+    # a caller-chosen chunk of 1024 elements over 70 M parameters: 68,360 chunks, more than the
+    # 65,535 that fit the grid's second dimension, so the launch falls back to a flat grid with
+    # the chunk index derived by division; same arithmetic, bit for bit
+    import numpy as np
+    from tspipe_amd import _lib, _tables
+    g = torch.Generator(device=device).manual_seed(5)
+    n = 70_000_001
+    t = torch.randn(n, generator=g, device=device) * 0.02
+    s = torch.randn(n, generator=g, device=device) * 0.02
+    out = torch.empty_like(t)
+    ptr = lambda x: np.array([x.data_ptr()], dtype=np.uint64)
+    with torch.cuda.device(device):
+        table = _tables.stage_ema(ptr(t), ptr(s), ptr(out), np.array([n], dtype=np.int64), device, chunk_elems=1024)
+        assert table.n_chunks > 65535
+        _lib.check(_lib.lib().ts_ema_multi(table.dev_ptr, table.n_chunks, table.chunk, 0.99, 1.0 - 0.99,
+                                           _lib.current_stream_ptr(device)), "ts_ema_multi")
+        table.done()
+    torch.cuda.synchronize()
+    want = t * torch.tensor(0.99, dtype=torch.float32) + s * torch.tensor(1.0 - 0.99, dtype=torch.float32)
+    assert torch.equal(out, want)

@@ -17,6 +17,33 @@ namespace ts {
 // treat as generic: it would use flat_load / flat_store, instructions that are
 // booked on the LDS counter as well.  All of them are device memory, so the
 // vector paths say so and get global_load / global_store.
+// Keeps every field of a table entry in one round of scalar loads: left to
+// itself the compiler fetches the length first and the pointers only behind
+// the early exit, a second dependent round in front of the vector loads.
+#if defined(__HIP_DEVICE_COMPILE__)
+#define TS_PIN_SCALARS(...) asm volatile("" : : __VA_ARGS__)
+#else
+#define TS_PIN_SCALARS(...) (void)0
+#endif
+
+// Which (chunk, sub-block) a workgroup is.  The launchers use a two-dimensional
+// grid (x = sub-block, y = chunk: the same dispatch order as chunk * subs + sub)
+// whenever the chunk count fits gridDim.y, which spares every workgroup an
+// integer division in front of its first load.
+__device__ __forceinline__ void chunk_and_sub(uint32_t subs, uint32_t& chunk, uint32_t& sub) {
+  if (gridDim.x == subs) {  // two-dimensional launch (also right for a single chunk)
+    chunk = blockIdx.y;
+    sub = blockIdx.x;
+  } else {
+    chunk = blockIdx.x / subs;
+    sub = blockIdx.x % subs;
+  }
+}
+
+inline dim3 chunk_grid(int64_t n_chunks, int64_t subs) {
+  return n_chunks <= 65535 ? dim3((unsigned)subs, (unsigned)n_chunks) : dim3((unsigned)(n_chunks * subs));
+}
+
 #define TS_GLOBAL __attribute__((address_space(1)))
 typedef TS_GLOBAL const f32x4* gc_f32x4_ptr;
 typedef TS_GLOBAL f32x4* g_f32x4_ptr;
@@ -45,8 +72,10 @@ __global__ __launch_bounds__(kEmaBlock) void ema_multi_kernel(const ts_ema_chunk
                                                               uint32_t subs, float m, float c,
                                                               int64_t clone_offset) {
   // Uniform per workgroup: the compiler turns these into scalar loads.
-  const uint32_t chunk = blockIdx.x / subs, sub = blockIdx.x % subs;
+  uint32_t chunk, sub;
+  chunk_and_sub(subs, chunk, sub);
   const ts_ema_chunk ch = table[chunk];
+  TS_PIN_SCALARS("s"(ch.t), "s"(ch.s), "s"(ch.out), "s"(ch.n), "s"(ch.flags));
   const uint32_t begin = sub * kSubElems;
   if (begin >= ch.n) return;  // short chunk (tensor tail or small tensor)
   const uint32_t n = (ch.n - begin < (uint32_t)kSubElems) ? ch.n - begin : (uint32_t)kSubElems;
@@ -120,8 +149,10 @@ __device__ __forceinline__ T ema1_t(T t, T s, float m, float c) {
 template <typename T>
 __global__ __launch_bounds__(kEmaBlock) void ema_multi_kernel_2byte(const ts_ema_chunk* __restrict__ table,
                                                                     uint32_t subs, float m, float c) {
-  const uint32_t chunk = blockIdx.x / subs, sub = blockIdx.x % subs;
+  uint32_t chunk, sub;
+  chunk_and_sub(subs, chunk, sub);
   const ts_ema_chunk ch = table[chunk];
+  TS_PIN_SCALARS("s"(ch.t), "s"(ch.s), "s"(ch.out), "s"(ch.n), "s"(ch.flags));
   const uint32_t begin = sub * kSubElems2;
   if (begin >= ch.n) return;
   const uint32_t n = (ch.n - begin < (uint32_t)kSubElems2) ? ch.n - begin : (uint32_t)kSubElems2;
@@ -163,8 +194,10 @@ constexpr int kSubBytes = kCopyBlock * 16;
 
 __global__ __launch_bounds__(kCopyBlock) void copy_segments_kernel(const ts_copy_chunk* __restrict__ table,
                                                                    uint32_t subs) {
-  const uint32_t chunk = blockIdx.x / subs, sub = blockIdx.x % subs;
+  uint32_t chunk, sub;
+  chunk_and_sub(subs, chunk, sub);
   const ts_copy_chunk ch = table[chunk];
+  TS_PIN_SCALARS("s"(ch.src), "s"(ch.dst), "s"(ch.bytes), "s"(ch.flags));
   const uint64_t begin = (uint64_t)sub * kSubBytes;
   if (begin >= ch.bytes) return;
   const uint32_t bytes =
@@ -219,7 +252,7 @@ int ts_ema_multi(const ts_ema_chunk* table_dev, int64_t n_chunks, int64_t chunk_
   if (!table_dev) return TS_ERR_ARG;
   const int64_t subs = chunk_elems / ts::kSubElems;
   if (subs > 0x7fffffffLL || n_chunks * subs > 0x7fffffffLL) return TS_ERR_RANGE;
-  TS_LAUNCH_TIMED(ts::ema_multi_kernel<false>, dim3((unsigned)(n_chunks * subs)), dim3(ts::kEmaBlock),
+  TS_LAUNCH_TIMED(ts::ema_multi_kernel<false>, ts::chunk_grid(n_chunks, subs), dim3(ts::kEmaBlock),
                   (hipStream_t)stream, table_dev, (uint32_t)subs, m32, c32, (int64_t)0);
   return ts::check_launch();
 }
@@ -233,7 +266,7 @@ int ts_ema_multi_dtype(const ts_ema_chunk* table_dev, int64_t n_chunks, int64_t 
   if (!table_dev) return TS_ERR_ARG;
   const int64_t subs = chunk_elems / ts::kSubElems2;
   if (subs > 0x7fffffffLL || n_chunks * subs > 0x7fffffffLL) return TS_ERR_RANGE;
-  const dim3 grid((unsigned)(n_chunks * subs));
+  const dim3 grid = ts::chunk_grid(n_chunks, subs);
   if (dtype == TS_BF16)
     TS_LAUNCH_TIMED(ts::ema_multi_kernel_2byte<ts::bf16_t>, grid, dim3(ts::kEmaBlock), (hipStream_t)stream,
                     table_dev, (uint32_t)subs, m32, c32);
@@ -252,7 +285,7 @@ int ts_ema_clone_multi(const ts_ema_chunk* table_dev, int64_t n_chunks, int64_t 
   if (!table_dev) return TS_ERR_ARG;
   const int64_t subs = chunk_elems / ts::kSubElems;
   if (subs > 0x7fffffffLL || n_chunks * subs > 0x7fffffffLL) return TS_ERR_RANGE;
-  TS_LAUNCH_TIMED(ts::ema_multi_kernel<true>, dim3((unsigned)(n_chunks * subs)), dim3(ts::kEmaBlock),
+  TS_LAUNCH_TIMED(ts::ema_multi_kernel<true>, ts::chunk_grid(n_chunks, subs), dim3(ts::kEmaBlock),
                   (hipStream_t)stream, table_dev, (uint32_t)subs, m32, c32, clone_offset_bytes);
   return ts::check_launch();
 }
@@ -264,7 +297,7 @@ int ts_copy_segments(const ts_copy_chunk* table_dev, int64_t n_chunks, int64_t c
   if (!table_dev) return TS_ERR_ARG;
   const int64_t subs = chunk_bytes / ts::kSubBytes;
   if (subs > 0x7fffffffLL || n_chunks * subs > 0x7fffffffLL) return TS_ERR_RANGE;
-  TS_LAUNCH_TIMED(ts::copy_segments_kernel, dim3((unsigned)(n_chunks * subs)), dim3(ts::kCopyBlock),
+  TS_LAUNCH_TIMED(ts::copy_segments_kernel, ts::chunk_grid(n_chunks, subs), dim3(ts::kCopyBlock),
                      (hipStream_t)stream, table_dev, (uint32_t)subs);
   return ts::check_launch();
 }
