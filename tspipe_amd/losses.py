@@ -583,7 +583,7 @@ def set_infonce_workgroup_target(workgroups: int = 0) -> int:
     (0 or 256) suits a loss that has the GPU to itself; a pipeline that runs the
     loss beside bandwidth-bound work on another stream, as TSPipe runs it beside
     the momentum update (tspipe/gpu_task.py:385-410), gets a shorter step from
-    64: fewer partial sums through HBM, CUs left to the other stream.
+    32 to 64: fewer partial sums through HBM, CUs left to the other stream.
     Process-wide; returns the previous value."""
     return int(_lib.lib().ts_infonce_set_workgroup_target(int(workgroups)))
 
