@@ -60,7 +60,8 @@ __device__ __forceinline__ PlaneSplit split_plane(const float* p, int64_t HW) {
 // per lane, against 3.06 per thread of a 256-thread workgroup, whose fourth
 // load has 16 threads in it).  Four loads per lane and operand are in flight at
 // a time; more of them (8, 14: the whole plane) were measured slower.
-constexpr int kBnWaveLoads = 4;  // 16-byte loads per lane and operand in flight
+constexpr int kBnWaveLoads = 4;   // 16-byte loads per lane in flight, one operand (2 and 3: 1-2 % slower)
+constexpr int kBnWaveLoads2 = 2;  // per operand when there are two (backward 80.3 us against 83.2 with 4; 1: 80.1, 6: 82.6)
 // STREAM: the operands are not read again by a kernel of the same call, so
 // they are fetched with non-temporal loads (the stand-alone statistics pass:
 // 20.4 against 22.2 us on 103 MB; the statistics half of the fused forward
@@ -71,7 +72,7 @@ __device__ __forceinline__ void slab_reduce_waves(const float* __restrict__ x, c
                                                   int64_t n1, int64_t C, int64_t c, int64_t HW, float& a, float& b,
                                                   F f) {
   constexpr int NW = BLOCK / kWave;
-  constexpr int U = kBnWaveLoads;
+  constexpr int U = TWO ? kBnWaveLoads2 : kBnWaveLoads;
   const int lane = threadIdx.x % kWave, w = threadIdx.x / kWave;
   for (int64_t n = n0 + w; n < n1; n += NW) {
     const int64_t off = (n * C + c) * HW;
