@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the teacher-student step kernels on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-kernels]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-eager] [--no-kernels]
 
 One "step" is the MoCo-v3 ViT-Base teacher-student step of the kernel path:
 the momentum EMA over the ViT-B/16 parameter list (152 fp32 tensors,
@@ -18,8 +18,10 @@ per launch (12 B per parameter) over its average duration, measured with HIP
 events that the launch itself stamps with the kernel's begin and end, on the
 kernel's own stream, inside the timed region;
 `cpu_baseline` is the oracle's eager PyTorch restatement of the same step on
-the host cores (bounded sample); `kernels` holds stand-alone timings of every
-kernel at the other configurations (informational).
+the host cores (bounded sample); `eager_gpu_baseline` is the same eager op
+chain -- what the reference's plug-ins execute -- on this GPU through
+PyTorch-ROCm; `kernels` holds stand-alone timings of every kernel at the other
+configurations (informational), each with `cpu_ms` and `eager_gpu_ms` beside it.
 """
 import argparse
 import gc
@@ -288,7 +290,25 @@ def _cpu_ms(fn, budget_s=1.2, max_iters=20):
     return statistics.median(times) * 1e3, len(times)
 
 
-def run_kernel_table(dev, with_cpu=True):
+def _eager_gpu_ms(fn, budget_s=1.0, max_iters=30):
+    """Wall milliseconds per call of fn(), an eager PyTorch op chain on the GPU:
+    two untimed calls, then back-to-back calls until the budget is spent (at
+    least three), closed by a device synchronize.  Wall time, because that is
+    what such a chain costs its caller: many of them are bound by the host's
+    launches rather than by the kernels.  Returns (ms, calls)."""
+    import torch
+    fn()
+    fn()
+    torch.cuda.synchronize()
+    n, t0 = 0, time.perf_counter()
+    while n < 3 or (n < max_iters and time.perf_counter() - t0 < budget_s):
+        fn()
+        n += 1
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / n * 1e3, n
+
+
+def run_kernel_table(dev, with_cpu=True, with_eager=True):
     """Stand-alone device timings of each kernel at the other configurations,
     called through the C ABI with preallocated outputs and workspaces; beside
     each, `cpu_ms`: the oracle's eager PyTorch chain for the same operation on
@@ -316,10 +336,21 @@ def run_kernel_table(dev, with_cpu=True):
         out[name]["cpu_calls"] = calls
         out[name]["gpu_over_cpu"] = round(ms / out[name]["ms"], 1)
 
-    def kd_cpu(s, t, T, mask=None):
-        s_c = s.detach().cpu().requires_grad_()
-        t_c = t.detach().cpu()
-        m_c = None if mask is None else mask.cpu()
+    def eager(name, fn):
+        """Adds the timing of the same operation as the reference's eager op
+        chain on this GPU to out[name]."""
+        if not with_eager:
+            return
+        ms, calls = _eager_gpu_ms(fn)
+        out[name]["eager_gpu_ms"] = round(ms, 4)
+        out[name]["eager_gpu_calls"] = calls
+        out[name]["eager_gpu_over_this"] = round(ms / out[name]["ms"], 1)
+        torch.cuda.empty_cache()  # the chain's temporaries go back before the next entry sizes its buffers
+
+    def kd_cpu(s, t, T, mask=None, device="cpu"):
+        s_c = s.detach().to(device).requires_grad_()
+        t_c = t.detach().to(device)
+        m_c = None if mask is None else mask.to(device)
 
         def f():
             s_c.grad = None
@@ -385,6 +416,7 @@ def run_kernel_table(dev, with_cpu=True):
         out[name] = entry(nbytes, statistics.median(ms), note, 1)
         t_c, s_c = [t.cpu() for t in teacher], [s_.cpu() for s_ in student]
         cpu(name, lambda: ts_oracle.ema_update(m, s_c, t_c))
+        eager(name, lambda: ts_oracle.ema_update(m, student, teacher))
         del teacher, student, st, t_c, s_c
     ema_mod.release_pool()
 
@@ -408,6 +440,8 @@ def run_kernel_table(dev, with_cpu=True):
                                             "kernel-only events", 1)
     t_c, s_c = [t.cpu() for t in teacher], [s_.cpu() for s_ in student]
     cpu("ema_clone_fused_vit_base", lambda: ([p_.detach().clone() for p_ in s_c], ts_oracle.ema_update(0.99, s_c, t_c)))
+    eager("ema_clone_fused_vit_base",
+          lambda: ([p_.detach().clone() for p_ in student], ts_oracle.ema_update(0.99, student, teacher)))
     del teacher, student, keep, t_c, s_c
     ema_mod.release_pool()
 
@@ -432,6 +466,7 @@ def run_kernel_table(dev, with_cpu=True):
     out["kd_256x100_f32"] = entry(3 * 256 * 100 * 4, _time_stream(f), "cfg2 itself; latency-bound: two launches (rows, final sum)", 2,
                                   working_set=3 * 256 * 100 * 4)
     cpu("kd_256x100_f32", kd_cpu(s, t, 4.0))
+    eager("kd_256x100_f32", kd_cpu(s, t, 4.0, device=dev))
 
     def kd_sets(rows, V, n_sets):
         fns = []
@@ -446,6 +481,7 @@ def run_kernel_table(dev, with_cpu=True):
     out["kd_65536x100_f32"] = entry(one, _time_stream(rotate(fns), batch=8), None, 2, working_set=8 * one, sets=8,
                                     resident_ms=_time_stream(fns[0]))
     cpu("kd_65536x100_f32", kd_cpu(*fns[0].operands, 4.0))
+    eager("kd_65536x100_f32", kd_cpu(*fns[0].operands, 4.0, device=dev))
     del fns
 
     # an ImageNet-sized class count (not one of the benchmark configurations): rows long enough to stream
@@ -454,6 +490,7 @@ def run_kernel_table(dev, with_cpu=True):
     out["kd_32768x1000_f32"] = entry(one, _time_stream(rotate(fns), batch=2), "not one of the benchmark configurations", 2,
                                      working_set=2 * one, sets=2)
     cpu("kd_32768x1000_f32", kd_cpu(*fns[0].operands, 4.0))
+    eager("kd_32768x1000_f32", kd_cpu(*fns[0].operands, 4.0, device=dev))
     del fns, s, t, f
 
     # DistilBERT-shaped masked KD (cfg3) after a gather of 4 micro-batches.  The selected rows of one
@@ -482,6 +519,7 @@ def run_kernel_table(dev, with_cpu=True):
     out["gather_4x62.5MB_bf16"] = entry(2 * 250036224, statistics.median(ms), "kernel-only events", 1)
     pieces_c = [p_.cpu() for p_ in pieces_s]
     cpu("gather_4x62.5MB_bf16", lambda: ts_oracle.gather(pieces_c))
+    eager("gather_4x62.5MB_bf16", lambda: ts_oracle.gather(pieces_s))
     del pieces_c, s_full, dsts
     kd_bytes = int(3 * n_sel_avg * row_b + (4096 - n_sel_avg) * row_b)
 
@@ -557,6 +595,15 @@ def run_kernel_table(dev, with_cpu=True):
         kd_bytes, _time_stream(rotate(fns2), batch=2),
         "KD + cross-entropy on the masked tokens in one pass (distiller.py:719-744), two sets of logits in turn", 2,
         working_set=2 * 3 * 4096 * row_b, sets=2)
+    sg = sets[0]["s_full"].detach().requires_grad_()
+    lab2d = fns2[0].keep[0].view(32, 128)
+
+    def kdce_eager():  # distiller.py:719-744 with alpha_ce 0.5, alpha_mlm 2, temperature 2, CE restricted to the mask
+        sg.grad = None
+        ts_oracle.distil_loss(sg, sets[0]["t_full"], None, None, lab2d, sets[0]["mask"], 0.5, 2.0, 0.0, 2.0, True).backward()
+    eager("kdce_masked_32x128x30522_bf16", kdce_eager)
+    sg.grad = None
+    del sg, lab2d
     fns2 = [mse_call(d, gr) for d, gr in zip(sets, grads)]
     out["mse_masked_32x128x30522_bf16"] = entry(
         kd_bytes, _time_stream(rotate(fns2), batch=2),
@@ -577,8 +624,16 @@ def run_kernel_table(dev, with_cpu=True):
         (3 * n0 + (4096 - n0)) * 768 * 4, _time_stream(f_cos),
         "cosine term on the hidden states (distiller.py:756-770); latency-bound", 2, working_set=3 * 4096 * 768 * 4)
     del hid, ghid
+    d = sets[0]
+    eager("kd_masked_32x128x30522_bf16", kd_cpu(d["s_full"], d["t_full"], 2.0, d["mask"], device=dev))
+    sp_g, tp_g = list(d["s_full"].chunk(4)), list(d["t_full"].chunk(4))
+
+    def pieces_eager():  # the reference's order: gather both outputs, then the loss
+        s_all = ts_oracle.gather(sp_g).requires_grad_()
+        ts_oracle.distil_ce(s_all, ts_oracle.gather(tp_g), d["mask"], 2.0).backward()
+    eager("kd_masked_4_pieces_8x128x30522_bf16", pieces_eager)
+    del sp_g, tp_g
     if with_cpu:
-        d = sets[0]
         s_c, t_c, m_c = d["s_full"].cpu(), d["t_full"].cpu(), d["mask"].cpu()
         sp_c, tp_c = list(s_c.chunk(4)), list(t_c.chunk(4))
         cpu("kd_masked_32x128x30522_bf16", kd_cpu(s_c, t_c, 2.0, m_c))
@@ -623,6 +678,14 @@ def run_kernel_table(dev, with_cpu=True):
                 t.grad = None
             sum(ts_oracle.infonce(a, b, 0.2) for a, b in zip(qc, kc)).backward()
         cpu(name, f_cpu)
+        qg = [t.detach().clone().requires_grad_() for t in ((q1, q2) if pairs == 2 else (q1,))]
+        kg = (k1, k2) if pairs == 2 else (k1,)
+
+        def f_eager():
+            for t in qg:
+                t.grad = None
+            sum(ts_oracle.infonce(a, b, 0.2) for a, b in zip(qg, kg)).backward()
+        eager(name, f_eager)
     nce_entry("infonce_4096x256_bf16", 4096, 1)
     nce_entry("infonce_2_pairs_4096x256_bf16", 4096, 2, "both directions of the symmetric loss in one call")
     nce_entry("infonce_16384x256_bf16", 16384, 1,
@@ -650,6 +713,14 @@ def run_kernel_table(dev, with_cpu=True):
         oc[0].grad = oc[1].grad = None
         ts_oracle.byol_contrastive_loss(*oc).backward()
     cpu("byol_256x128_f32", byol_cpu)
+    og = [t.detach().clone() for t in o]
+    og[0].requires_grad_()
+    og[1].requires_grad_()
+
+    def byol_eager():
+        og[0].grad = og[1].grad = None
+        ts_oracle.byol_contrastive_loss(*og).backward()
+    eager("byol_256x128_f32", byol_eager)
 
     # DeferredBatchNorm (cfg5): 8 different micro-batches of [32, 256, 56, 56] (822 MB of inputs, and as much
     # again of outputs) taken in turn, as the configuration has them: no call finds its micro-batch in the
@@ -747,6 +818,42 @@ def run_kernel_table(dev, with_cpu=True):
         5 * one_x, _time_stream(rotate([bwd_of(xi, dyi, dxi) for xi, dyi, dxi in zip(xs, dys, dxs)]), batch=4),
         "bytes = read x,dy twice + write dx", 2, working_set=3 * 4 * one_x, sets=4)
     del dxs
+    # the reference's module arithmetic on this GPU: its buffers moved to the device
+    ora_g = ts_oracle.DeferredBNOracle(256, chunks=1 << 30, weight=gamma, bias=beta)
+    for attr in ("running_mean", "running_var", "num_batches_tracked", "sum", "sum_squares"):
+        setattr(ora_g, attr, getattr(ora_g, attr).to(dev))
+    it = {"i": 0}
+
+    def next_x():
+        it["i"] += 1
+        return xs[it["i"] % MB]
+    eager("bn_stats_32x256x56x56_f32", lambda: ora_g.track(next_x()))
+    eager("bn_stats_normalise_32x256x56x56_f32", lambda: ora_g.forward(next_x()))
+    eager("bn_forward_train_32x256x56x56_f32", lambda: ora_g.forward(next_x()))
+
+    def cfg5_track_eager():
+        for xi in xs:
+            ora_g.track(xi)
+        ora_g.commit()
+
+    def cfg5_forward_eager():
+        for xi in xs:
+            ora_g.forward(xi)
+        ora_g.commit()
+    eager("bn_cfg5_track_x8_commit", cfg5_track_eager)
+    eager("bn_cfg5_forward_x8_commit", cfg5_forward_eager)
+    if with_eager:  # four graphs over four micro-batches in turn, like the entry above
+        we, be = gamma.clone().requires_grad_(), beta.clone().requires_grad_()
+        xes = [xi.clone().requires_grad_() for xi in xs[:4]]
+        yes = [torch.nn.functional.batch_norm(xe, None, None, we, be, True, 0.0, 1e-5) for xe in xes]
+
+        def bn_bwd_eager():
+            it["i"] += 1
+            i = it["i"] % 4
+            xes[i].grad = we.grad = be.grad = None
+            yes[i].backward(dys[i], retain_graph=True)
+        eager("bn_backward_32x256x56x56_f32", bn_bwd_eager)
+        del xes, yes, we, be
     if with_cpu:
         x_c, dy_c, gamma_c, beta_c = x.cpu(), dy.cpu(), gamma.cpu(), beta.cpu()
         ora = ts_oracle.DeferredBNOracle(256, chunks=1 << 30, weight=gamma_c, bias=beta_c)
@@ -796,6 +903,40 @@ def run_cpu_baseline(budget_s=12.0):
                       f"fwd+bwd, eager PyTorch on CPU) in {el:.1f} s"}
 
 
+def run_eager_gpu_baseline(dev, budget_s=4.0):
+    """The oracle's eager-PyTorch step on this GPU: the op chain the reference's
+    plug-ins execute (per-tensor EMA loop, normalize / einsum / cross-entropy
+    and its backward), issued from one host thread in the order TSPipe's compute
+    thread runs them, through PyTorch-ROCm."""
+    import torch
+    from oracle import ts_oracle
+    _, _, vit = _shapes()
+    g = torch.Generator().manual_seed(3)
+    teacher = [(torch.randn(s, generator=g) * 0.02).to(dev) for s in vit]
+    student = [(torch.randn(s, generator=g) * 0.02).to(dev) for s in vit]
+    q = torch.nn.functional.normalize(torch.randn(4096, 256, generator=g), dim=1).to(torch.bfloat16).to(dev).requires_grad_()
+    k = torch.nn.functional.normalize(torch.randn(4096, 256, generator=g), dim=1).to(torch.bfloat16).to(dev)
+
+    def step(t):
+        t = ts_oracle.ema_update(0.99, student, t, skip_none=True)
+        q.grad = None
+        ts_oracle.infonce(q, k, 0.2).backward()
+        return t
+
+    for _ in range(5):
+        teacher = step(teacher)
+    torch.cuda.synchronize()
+    n, t0 = 0, time.perf_counter()
+    while n < 20 or (n < 2000 and time.perf_counter() - t0 < budget_s):
+        teacher = step(teacher)
+        n += 1
+    torch.cuda.synchronize()
+    el = time.perf_counter() - t0
+    return {"value": round(n / el, 2), "unit": "steps/s", "kind": "port", "device": torch.cuda.get_device_name(dev),
+            "sample": f"{n} full steps (the same eager PyTorch op chain as cpu_baseline, on the GPU through PyTorch-ROCm, "
+                      f"one host thread, one stream) in {el:.1f} s"}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -803,6 +944,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel table")
+    ap.add_argument("--no-eager", action="store_true",
+                    help="skip the eager-PyTorch-on-GPU legs (thousands of small launches: leave them out under a profiler)")
     ap.add_argument("--nce-workgroups", type=int, default=STEP_NCE_WORKGROUPS,
                     help="workgroup target of the InfoNCE kernels inside the step (the kernel table uses the default, 256)")
     args = ap.parse_args()
@@ -847,11 +990,19 @@ def main():
         "host": res["host"],
     }
     if not args.no_kernels:
-        line["kernels"] = run_kernel_table(dev, with_cpu=not args.no_cpu)
+        line["kernels"] = run_kernel_table(dev, with_cpu=not args.no_cpu, with_eager=not args.no_eager)
         line["kernels_timing_note"] = TIMING_NOTE
         line["kernels_cpu_note"] = ("cpu_ms: the oracle's eager PyTorch chain for the same operation and shape on "
                                     f"{min(os.cpu_count() or 1, int(os.environ.get('OMP_NUM_THREADS', os.cpu_count() or 1)))} "
                                     "host threads, median of up to 20 calls within ~1.2 s (a single call when one takes longer)")
+        line["kernels_eager_gpu_note"] = ("eager_gpu_ms: the same eager PyTorch chain (the reference's arithmetic) on this GPU, "
+                                          "wall time per call over up to 30 back-to-back calls within ~1 s, temporaries and "
+                                          "launch overhead included as the reference's caller pays them")
+    if not args.no_eager:
+        line["eager_gpu_baseline"] = run_eager_gpu_baseline(dev)
+        line["eager_gpu_baseline"]["this_over_eager_gpu"] = round(line["value"] / line["eager_gpu_baseline"]["value"], 1)
+    else:
+        line["eager_gpu_baseline"] = None
     if not args.no_cpu:
         line["cpu_baseline"] = run_cpu_baseline()
     else:

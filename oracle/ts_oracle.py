@@ -130,7 +130,7 @@ def infonce(q: Tensor, k: Tensor, tau: float) -> Tensor:
     q = F.normalize(q, dim=1)
     k = F.normalize(k, dim=1)
     logits = torch.einsum("nc,mc->nm", [q, k]) / tau
-    labels = torch.arange(logits.shape[0], dtype=torch.long)
+    labels = torch.arange(logits.shape[0], dtype=torch.long).to(logits.device)  # main.py:155-157: built on the host, then moved
     return nn.CrossEntropyLoss()(logits, labels) * (2 * tau)
 
 

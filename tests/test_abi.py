@@ -165,6 +165,11 @@ def test_device_entry_points_validate_before_launching():
     assert lib.ts_ema_multi(p, -1, 4096, 0.9, 0.1, None) == -1
     assert lib.ts_ema_multi(p, 5, 1000, 0.9, 0.1, None) == -1
     assert lib.ts_ema_multi(p, 0, 4096, 0.9, 0.1, None) == 0           # nothing to do
+    # a grid dimension times the workgroup size (256) must stay below 2^32 threads: the chunk count above
+    # 65535 runs as a flat grid of chunks x sub-blocks
+    assert lib.ts_ema_multi(p, 70000, 1024 * 300, 0.9, 0.1, None) == -5
+    assert lib.ts_ema_multi(p, 1, 1024 * (1 << 24), 0.9, 0.1, None) == -5
+    assert lib.ts_copy_segments(p, 1 << 25, 4096, None) == -5
     assert lib.ts_copy_segments(None, 3, 16384, None) == -1
     assert lib.ts_copy_segments(p, 0, 16384, None) == 0
     assert lib.ts_kd_fwd_bwd(None, p, None, 4, 10, 10, 10, 1.0, 1.0, p, p, None, 10, 0, None) == -1

@@ -13,10 +13,6 @@
 
 namespace ts {
 
-// The table hands out plain 64-bit addresses, which the compiler can only
-// treat as generic: it would use flat_load / flat_store, instructions that are
-// booked on the LDS counter as well.  All of them are device memory, so the
-// vector paths say so and get global_load / global_store.
 // Keeps every field of a table entry in one round of scalar loads: left to
 // itself the compiler fetches the length first and the pointers only behind
 // the early exit, a second dependent round in front of the vector loads.
@@ -44,12 +40,21 @@ inline dim3 chunk_grid(int64_t n_chunks, int64_t subs) {
   return n_chunks <= 65535 ? dim3((unsigned)subs, (unsigned)n_chunks) : dim3((unsigned)(n_chunks * subs));
 }
 
+// A grid dimension times the workgroup size has to stay below 2^32 threads.
+inline bool chunk_grid_fits(int64_t n_chunks, int64_t subs, int block) {
+  const int64_t limit = 0xffffffffLL / block;
+  return subs <= limit && (n_chunks <= 65535 || n_chunks <= limit / subs);
+}
+
+// The table hands out plain 64-bit addresses, which the compiler can only
+// treat as generic: it would use flat_load / flat_store, instructions that are
+// booked on the LDS counter as well.  All of them are device memory, so the
+// vector paths say so and get global_load / global_store.
 #define TS_GLOBAL __attribute__((address_space(1)))
 typedef TS_GLOBAL const f32x4* gc_f32x4_ptr;
 typedef TS_GLOBAL f32x4* g_f32x4_ptr;
 typedef TS_GLOBAL const u32x4* gc_u32x4_ptr;
 typedef TS_GLOBAL u32x4* g_u32x4_ptr;
-
 
 constexpr int kEmaBlock = 256;
 constexpr int kSubElems = kEmaBlock * 4;  // one 16-byte vector per thread and operand
@@ -251,7 +256,7 @@ int ts_ema_multi(const ts_ema_chunk* table_dev, int64_t n_chunks, int64_t chunk_
   if (n_chunks == 0) return TS_OK;
   if (!table_dev) return TS_ERR_ARG;
   const int64_t subs = chunk_elems / ts::kSubElems;
-  if (subs > 0x7fffffffLL || n_chunks * subs > 0x7fffffffLL) return TS_ERR_RANGE;
+  if (!ts::chunk_grid_fits(n_chunks, subs, ts::kEmaBlock)) return TS_ERR_RANGE;
   TS_LAUNCH_TIMED(ts::ema_multi_kernel<false>, ts::chunk_grid(n_chunks, subs), dim3(ts::kEmaBlock),
                   (hipStream_t)stream, table_dev, (uint32_t)subs, m32, c32, (int64_t)0);
   return ts::check_launch();
@@ -265,7 +270,7 @@ int ts_ema_multi_dtype(const ts_ema_chunk* table_dev, int64_t n_chunks, int64_t 
   if (n_chunks == 0) return TS_OK;
   if (!table_dev) return TS_ERR_ARG;
   const int64_t subs = chunk_elems / ts::kSubElems2;
-  if (subs > 0x7fffffffLL || n_chunks * subs > 0x7fffffffLL) return TS_ERR_RANGE;
+  if (!ts::chunk_grid_fits(n_chunks, subs, ts::kEmaBlock)) return TS_ERR_RANGE;
   const dim3 grid = ts::chunk_grid(n_chunks, subs);
   if (dtype == TS_BF16)
     TS_LAUNCH_TIMED(ts::ema_multi_kernel_2byte<ts::bf16_t>, grid, dim3(ts::kEmaBlock), (hipStream_t)stream,
@@ -284,7 +289,7 @@ int ts_ema_clone_multi(const ts_ema_chunk* table_dev, int64_t n_chunks, int64_t 
   if (n_chunks == 0) return TS_OK;
   if (!table_dev) return TS_ERR_ARG;
   const int64_t subs = chunk_elems / ts::kSubElems;
-  if (subs > 0x7fffffffLL || n_chunks * subs > 0x7fffffffLL) return TS_ERR_RANGE;
+  if (!ts::chunk_grid_fits(n_chunks, subs, ts::kEmaBlock)) return TS_ERR_RANGE;
   TS_LAUNCH_TIMED(ts::ema_multi_kernel<true>, ts::chunk_grid(n_chunks, subs), dim3(ts::kEmaBlock),
                   (hipStream_t)stream, table_dev, (uint32_t)subs, m32, c32, clone_offset_bytes);
   return ts::check_launch();
@@ -296,7 +301,7 @@ int ts_copy_segments(const ts_copy_chunk* table_dev, int64_t n_chunks, int64_t c
   if (n_chunks == 0) return TS_OK;
   if (!table_dev) return TS_ERR_ARG;
   const int64_t subs = chunk_bytes / ts::kSubBytes;
-  if (subs > 0x7fffffffLL || n_chunks * subs > 0x7fffffffLL) return TS_ERR_RANGE;
+  if (!ts::chunk_grid_fits(n_chunks, subs, ts::kCopyBlock)) return TS_ERR_RANGE;
   TS_LAUNCH_TIMED(ts::copy_segments_kernel, ts::chunk_grid(n_chunks, subs), dim3(ts::kCopyBlock),
                      (hipStream_t)stream, table_dev, (uint32_t)subs);
   return ts::check_launch();
