@@ -607,7 +607,7 @@ def run_kernel_table(dev, with_cpu=True, with_eager=True):
     fns2 = [mse_call(d, gr) for d, gr in zip(sets, grads)]
     out["mse_masked_32x128x30522_bf16"] = entry(
         kd_bytes, _time_stream(rotate(fns2), batch=2),
-        "squared-error term on the masked tokens (distiller.py:751-755): counting launch, rows, final sum", 3,
+        "squared-error term on the masked tokens (distiller.py:751-755): a workgroup per row, final sum", 2,
         working_set=2 * 3 * 4096 * row_b, sets=2)
     del fns2, grads
     hid = [torch.randn(4096, 768, generator=g).to(dev) for _ in range(2)]

@@ -579,10 +579,11 @@ def test_distil_loss_fn_clm_and_mse_terms(device, mode):
 
 def test_logits_mse_operands_aligned_differently(device):
     # s and t at different offsets from a 16-byte boundary (views into larger buffers): the kernel
-    # walks such rows element by element; rows of 2051 elements also exercise a second span
+    # walks such rows element by element; rows of 2051 elements also exercise a second span, rows of 8200
+    # the kernel that gives a row a workgroup of its own
     g = seeded(77)
-    rows, V = 9, 2051
-    for dtype, tol in ((torch.float32, 1e-5), (torch.bfloat16, 1e-3)):
+    for rows, V, dtype, tol in ((9, 2051, torch.float32, 1e-5), (9, 2051, torch.bfloat16, 1e-3),
+                                (3, 8200, torch.float32, 1e-5), (3, 8200, torch.bfloat16, 1e-3)):  # a workgroup per row
         s = (torch.randn(rows, V, generator=g) * 3).to(dtype)
         t = (torch.randn(rows, V, generator=g) * 3).to(dtype)
         want, (gw,) = _oracle_grad(lambda a, b: ts_oracle.logits_mse(a, b), s, others=(t,))
@@ -602,7 +603,12 @@ def test_logits_mse_operands_aligned_differently(device):
 
 @pytest.mark.parametrize("rows,V,dtype", [(256, 100, torch.float32), (33, 5000, torch.float32),
                                           (40, 30522, torch.bfloat16), (37, 101, torch.float32),
-                                          (19, 1001, torch.bfloat16)])
+                                          (19, 1001, torch.bfloat16),
+                                          # rows of 8192 elements and more take a workgroup each: the threshold itself,
+                                          # rows that start at every offset from a 16-byte boundary, more vectors than
+                                          # one round of loads holds
+                                          (5, 8192, torch.float32), (7, 9001, torch.float32),
+                                          (3, 40003, torch.bfloat16), (2, 20000, torch.float16)])
 def test_logits_mse_and_kd_mode_logits(device, rows, V, dtype):
     from argparse import Namespace
     g = seeded(240 + V)
