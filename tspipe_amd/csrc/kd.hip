@@ -386,6 +386,12 @@ __global__ __launch_bounds__(BLOCK, (KREG * GROUP > 1024 ? 4 : 1)) void kd_rows_
         const Vec16<T> lt = load16(trow + g.head + v * VEC), ls = load16(srow + g.head + v * VEC);
         __builtin_memcpy(&stage_t[v], &lt, 16);
         __builtin_memcpy(&stage_s[v], &ls, 16);
+      } else if constexpr (GROUP <= kWave) {
+        // rows that a wavefront or less holds: short-lived workgroups streaming through, where
+        // non-temporal loads pay (32768 x 1000 fp32: 75.0 -> 71.0 us; 65536 x 100: 22.7 -> 22.4); on the
+        // workgroup-wide rows they cost (4096 x 30522 bf16 under a 15 % mask: 83 against 77)
+        rt[j] = load16_stream(trow + g.head + v * VEC);
+        rs[j] = load16_stream(srow + g.head + v * VEC);
       } else {
         rt[j] = load16(trow + g.head + v * VEC);
         rs[j] = load16(srow + g.head + v * VEC);
