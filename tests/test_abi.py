@@ -190,6 +190,11 @@ def test_device_entry_points_validate_before_launching():
     assert lib.ts_infonce_set_workgroup_target(100000) == 32
     assert lib.ts_infonce_set_workgroup_target(-3) == 256
     assert lib.ts_infonce_set_workgroup_target(0) == 256
+    # the accuracy switch: returns the previous setting, leaves the workspace size alone
+    assert lib.ts_infonce_set_fp32_arithmetic(1) == 0
+    assert lib.ts_infonce_workspace_bytes(4096, 256, 1) == ws_bytes
+    assert lib.ts_infonce_set_fp32_arithmetic(0) == 1
+    assert lib.ts_infonce_set_fp32_arithmetic(0) == 0
     assert lib.ts_bn_stats(None, 2, 3, 4, p, None, None, None, None, 1e-5, None) == -1
     assert lib.ts_bn_stats(p, 2, 70000, 4, p, None, None, None, None, 1e-5, None) == -5
     assert lib.ts_bn_stats(p, 2, 3, 4, p, p, None, None, None, 1e-5, None) == -1                 # sum without sum_squares

@@ -810,6 +810,45 @@ def test_infonce_nearly_aligned_pairs(device, dtype, tau, noise, tol):
     assert max_rel_to_peak(qd.grad, gw) < tol
 
 
+@pytest.mark.parametrize("dtype,tau,noise", [(torch.bfloat16, 0.2, 0.01), (torch.bfloat16, 0.2, 1.0),
+                                             (torch.bfloat16, 0.07, 0.1), (torch.float16, 0.2, 0.01)])
+def test_infonce_fp32_arithmetic_switch_on_16_bit_pairs(device, dtype, tau, noise):
+    # the same nearly aligned pairs with the accuracy switch on: 16-bit embeddings on the fp32-MFMA
+    # kernels.  What is left is the storage rounding of dq itself (2^-9 of each element for bf16)
+    # on top of the fp32 path's 1e-4 of the peak (1e-3 at tau = 0.07), instead of 4e-3 .. 1.5e-2 of
+    # the peak on the bf16-MFMA kernels.
+    n, c = 512, 256
+    g = seeded(77)
+    q = torch.nn.functional.normalize(torch.randn(n, c, generator=g), dim=1)
+    k = torch.nn.functional.normalize(q + noise * torch.randn(n, c, generator=g) / 16, dim=1)
+    q, k = q.to(dtype), k.to(dtype)
+    want, (gw,) = _oracle_grad(lambda a, b: ts_oracle.infonce(a, b, tau), q, others=(k,))
+    assert ta.set_infonce_fp32_arithmetic(True) is False
+    try:
+        qd = q.to(device).requires_grad_()
+        loss = ta.infonce_loss(qd, k.to(device), tau)
+        loss.backward()
+        # and the un-gathered form takes the same route
+        qp = [p.contiguous().requires_grad_() for p in q.to(device).split([200, 312])]
+        kp = [p.contiguous() for p in k.to(device).split([200, 312])]
+        from argparse import Namespace
+        lp = ta.moco_contrastive_loss_pieces(qp, qp, kp, kp, None, Namespace(moco_t=tau))
+        lp.backward()
+    finally:
+        assert ta.set_infonce_fp32_arithmetic(False) is True
+    assert abs(loss.item() - want) < 1e-5 * abs(want) + 1e-7
+    assert abs(lp.item() - 2 * want) < 1e-5 * abs(2 * want) + 1e-7  # both directions were the same pair
+    peak = gw.abs().max().item()
+    slack = 1e-4 if tau >= 0.2 else 1e-3
+    # (an fp16 gradient this small is stored in subnormals: their spacing, 2^-24, joins the bound)
+    floor = 2.0 ** -24 if dtype == torch.float16 else 0.0
+    assert ((qd.grad.cpu().double() - gw).abs() <= slack * peak + gw.abs() * 2.0 ** -8 + floor).all()
+    # the switch is off again: the same call is back on the bf16-MFMA kernels (a different rounding)
+    qd2 = q.to(device).requires_grad_()
+    ta.infonce_loss(qd2, k.to(device), tau).backward()
+    assert not torch.equal(qd2.grad, qd.grad)
+
+
 @pytest.mark.parametrize("dtype,c,rows", [(torch.bfloat16, 256, [96, 32, 100, 28]), (torch.float32, 128, [40, 40, 17]),
                                          (torch.bfloat16, 64, [64])])
 def test_moco_loss_on_pieces_equals_the_gathered_loss(device, dtype, c, rows):

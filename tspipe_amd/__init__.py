@@ -11,7 +11,7 @@ from .ema import (bind_params_, calculate_target_network_parameters, calculate_u
 from .losses import (Logits, SoftTarget, byol_contrastive_loss, byol_contrastive_loss_pieces, byol_loss, cosine_embedding_loss, cosine_embedding_loss_pieces, distil_ce_loss,
                      distil_loss_fn, distil_loss_fn_pieces, infonce_loss, kd_ce_loss, kd_ce_loss_pieces,
                      kd_soft_target_loss, logits_mse_loss, moco_contrastive_loss, moco_contrastive_loss_pair,
-                     moco_contrastive_loss_pieces, set_infonce_workgroup_target,
+                     moco_contrastive_loss_pieces, set_infonce_fp32_arithmetic, set_infonce_workgroup_target,
                      soft_target_tspipe_loss)
 from .model_wrapper import TSPipeModelOutput, TSPipeModelWrapper
 from .utils import generic_object_gather, generic_object_scatter, traverse_tensor_map

@@ -954,7 +954,10 @@ inline void nce_clear_pieces(NcePair& P) {
 // temperatures its fixed soft-max reference point can represent
 // (2^(-2 log2(e)/tau) must stay a normal fp32); everything else -- fp32 inputs,
 // other widths, smaller temperatures -- goes to the fp32-MFMA path.
+static std::atomic<int> g_nce_fp32_arithmetic{0};
+
 inline bool nce_bf16_path(int64_t c, float tau, int dtype) {
+  if (g_nce_fp32_arithmetic.load(std::memory_order_relaxed)) return false;
   return dtype != TS_F32 && (c == 64 || c == 128 || c == 256) && tau >= 0.03f;
 }
 
@@ -968,6 +971,10 @@ extern "C" {
 int ts_infonce_set_workgroup_target(int workgroups) {
   if (workgroups <= 0 || workgroups > ts::kNceMaxWorkgroupTarget) workgroups = ts::kNceMaxWorkgroupTarget;
   return ts::g_nce_workgroup_target.exchange(workgroups, std::memory_order_relaxed);
+}
+
+int ts_infonce_set_fp32_arithmetic(int on) {
+  return ts::g_nce_fp32_arithmetic.exchange(on ? 1 : 0, std::memory_order_relaxed);
 }
 
 size_t ts_infonce_workspace_bytes(int64_t n, int64_t c, int n_pairs) {

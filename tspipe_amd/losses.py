@@ -588,6 +588,17 @@ def set_infonce_workgroup_target(workgroups: int = 0) -> int:
     return int(_lib.lib().ts_infonce_set_workgroup_target(int(workgroups)))
 
 
+def set_infonce_fp32_arithmetic(on: bool = True) -> bool:
+    """Accuracy switch of the InfoNCE kernels (``ts_infonce_set_fp32_arithmetic``):
+    when on, bf16 / fp16 embeddings also run on the fp32-MFMA kernels (every
+    product and sum in fp32, as the reference's fp32 run,
+    benchmarks/moco-v3/main.py:149-160), about seven times slower than the
+    bf16-MFMA kernels.  Meant for nearly aligned (q, k) pairs, where the bf16
+    kernels' rounding of the negatives' weights shows in the gradient.
+    Process-wide; returns the previous setting."""
+    return bool(_lib.lib().ts_infonce_set_fp32_arithmetic(1 if on else 0))
+
+
 def infonce_loss(q: Tensor, k: Tensor, tau: float) -> Tensor:
     """One direction of MoCo-v3's loss: ``CE(q^ k^T / tau, arange(N)) * 2 tau``
     (benchmarks/moco-v3/main.py:149-160)."""
