@@ -486,6 +486,50 @@ def test_kd_ce_row_sets_and_ignore_index(device):
     assert torch.isnan(l).item() and torch.isnan(torch.nn.CrossEntropyLoss(ignore_index=-100)(s, none)).item()
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_kd_ce_mse_at_every_row_width_boundary(device, dtype):
+    # The launcher picks a kernel by the number of 16-byte vectors a row can span: 16-, 32- and 64-lane
+    # groups, a 256-thread workgroup, 512 and 1024 threads with the row in registers, two passes beyond.
+    # Every boundary from both sides, with all three terms at once (KD under a mask, cross entropy with
+    # ignored labels, squared error), rows that start off a 16-byte boundary because the width is odd,
+    # and once more with the student one element off the teacher's alignment.
+    vec = 16 // torch.empty((), dtype=dtype).element_size()
+    widths = []
+    for vecs in (32, 64, 256, 1024, 4096, 8192):   # largest ceil(V / vec) + 1 each kernel takes
+        widths += [(vecs - 1) * vec, (vecs - 1) * vec + 1]
+    widths += [8191, 8192, 8193]                   # the squared-error term's own threshold (elements)
+    tol = 1e-5 if dtype == torch.float32 else 1e-3
+    rows = 5
+    for V in widths:
+        for shift in (0, 1):
+            g = seeded(9000 + V + shift)
+            s = (torch.randn(rows, V, generator=g) * 2).to(dtype)
+            t = (torch.randn(rows, V, generator=g) * 2).to(dtype)
+            mask = torch.tensor([True, False, True, True, False])
+            y = torch.tensor([V - 1, 0, -100, V // 2, -100])
+
+            def ref(a, b):
+                kd = ts_oracle.distil_ce(a.view(1, rows, V), b.view(1, rows, V), mask.view(1, rows), 2.0, 0.5)
+                ce = torch.nn.CrossEntropyLoss(ignore_index=-100)(a, y)
+                d = (a[mask] - b[mask])
+                return kd + 2.0 * ce + 0.05 * (d * d).sum() / int(mask.sum())
+            want, (gw,) = _oracle_grad(ref, s, others=(t,))
+            buf = torch.zeros(rows * V + 8, dtype=dtype, device=device)
+            sd = buf[shift:shift + rows * V].view(rows, V)
+            sd.copy_(s)
+            sd = sd.detach().requires_grad_()
+            loss = ta.kd_ce_loss(sd, t.to(device), y.to(device), 2.0, kd_weight=0.5, ce_weight=2.0,
+                                 row_mask=mask.to(device), mse_weight=0.05)
+            loss.backward()
+            case = f"V={V} shift={shift}"
+            assert rel_err(loss.item(), want) < tol, case
+            peak = gw.abs().max().item()
+            # 16-bit gradients: the squared-error term is added to a KD + CE gradient already stored
+            slack = gw.abs() * (2.0 ** -7 if dtype != torch.float32 else 0.0)
+            assert ((sd.grad.cpu().double() - gw).abs() <= tol * peak + slack).all(), case
+            assert (sd.grad.cpu()[4] == 0).all(), case   # neither masked in nor labelled
+
+
 def test_cosine_embedding_loss(device):
     g = seeded(220)
     x = torch.randn(3, 7, 48, generator=g)
