@@ -137,6 +137,50 @@ def test_deferred_bn_backward(device):
     _check_workspace(bn)
 
 
+@pytest.mark.parametrize("shape", [(2, 3, 1), (2, 5, 1, 1), (1, 2, 130, 130), (3, 4, 64, 64), (5, 3, 257),
+                                   (33, 2, 7, 7), (2, 70, 3, 3), (9, 1, 4, 5), (17, 6, 2)])
+def test_deferred_bn_forward_and_backward_over_plane_and_batch_sizes(device, shape):
+    # planes of one element, planes longer than one round of a wavefront's loads, planes that start off a
+    # 16-byte boundary (odd sizes), more samples than a workgroup's slab, a single channel, many channels:
+    # statistics, output and all three gradients against an fp64 evaluation
+    C = shape[1]
+    g = seeded(440 + len(shape) + shape[0])
+    x = _make(shape, 441 + shape[-1])
+    dy = torch.randn(shape, generator=g)
+    bn = ta.DeferredBatchNorm(C, chunks=1).to(device)
+    with torch.no_grad():
+        bn.weight.copy_(torch.rand(C, generator=g) + 0.5)
+        bn.bias.copy_(torch.randn(C, generator=g) * 0.1)
+    xd = x.to(device).requires_grad_()
+    y = bn(xd)
+    y.backward(dy.to(device))
+    x64 = x.double().requires_grad_()
+    w64 = bn.weight.detach().cpu().double().requires_grad_()
+    b64 = bn.bias.detach().cpu().double().requires_grad_()
+    y64 = F.batch_norm(x64, None, None, w64, b64, True, 0.0, 1e-5)
+    y64.backward(dy.double())
+    assert (y.detach().cpu().double() - y64.detach()).abs().max().item() < 2e-5
+    # dx is what is left of dy after two projections; with a handful of values per channel nearly all of
+    # it cancels, so the bound is set by the size of the terms that cancel (gamma / std * |dy|), as for
+    # any fp32 evaluation, and not by the size of the result
+    dims_ = [0] + list(range(2, len(shape)))
+    istd = 1.0 / torch.sqrt(x.double().var(dim=dims_, unbiased=False) + 1e-5)
+    terms = (w64.detach().abs() * istd).max().item() * dy.abs().max().item()
+    assert (xd.grad.cpu().double() - x64.grad).abs().max().item() <= 1e-5 * x64.grad.abs().max().item() + 2e-6 * terms
+    n_per_channel = x.numel() // C
+    assert (bn.weight.grad.cpu().double() - w64.grad).abs().max().item() \
+        <= 1e-5 * w64.grad.abs().max().item() + 2e-6 * n_per_channel ** 0.5 * dy.abs().max().item()
+    assert max_rel_to_peak(bn.bias.grad, b64.grad) < 1e-5
+    # chunks = 1: this one micro-batch was committed (momentum 0.1, biased variance as the reference keeps it)
+    dims = [0] + list(range(2, len(shape)))
+    mean = x.double().mean(dim=dims)
+    var = x.double().var(dim=dims, unbiased=False)
+    # a mean near zero is itself a cancelled sum: bounded against the size of the values, not of the mean
+    assert ((bn.running_mean.cpu().double() - 0.1 * mean).abs() <= 1e-6 * 0.1 * (mean.abs() + var.sqrt())).all()
+    assert _rel(bn.running_var, 0.9 + 0.1 * var) < 1e-5
+    _check_workspace(bn)
+
+
 def test_deferred_bn_interleaved_forwards_and_backwards(device):
     # a pipeline runs several micro-batches forward before the first backward, and backward
     # in another order: the layer's forward and backward calls share one alternating workspace
