@@ -268,6 +268,43 @@ def test_byol_special_cases(device):
     assert rel_err(l1, want) < 1e-5
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_byol_and_cosine_over_row_counts_and_widths(device, dtype):
+    # a row is a wavefront's work in both kernels (four rows to a workgroup): widths below, at and above
+    # what 64 lanes hold in one and in several 16-byte vectors, odd widths (rows off a 16-byte boundary),
+    # row counts that leave a workgroup partly empty
+    tol = 1e-5 if dtype == torch.float32 else 1e-3
+    for n, c in ((1, 1), (2, 3), (5, 64), (3, 65), (7, 255), (4, 256), (9, 257), (6, 768), (2, 1001), (3, 4099)):
+        g = seeded(7000 + n + c)
+        o1, o2, t1, t2 = [torch.randn(n, c, generator=g).to(dtype) for _ in range(4)]
+        want, (g1, g2) = _oracle_grad(ts_oracle.byol_contrastive_loss, o1, o2, others=(t1, t2))
+        d1, d2 = o1.to(device).requires_grad_(), o2.to(device).requires_grad_()
+        loss = ta.byol_contrastive_loss(d1, d2, t1.to(device), t2.to(device), None, None)
+        loss.backward()
+        case = f"byol n={n} c={c}"
+        assert rel_err(loss.item(), want) < tol or abs(loss.item() - want) < 1e-6, case
+        for got, ref, x in ((d1.grad, g1, o1), (d2.grad, g2, o2)):
+            slack = ref.abs() * (2.0 ** -8 if dtype != torch.float32 else 0.0)
+            # the gradient is a difference of terms of size 2 / (n |x|) per row; at width 1 all of it cancels
+            terms = 2.0 / (n * x.double().norm(dim=1, keepdim=True))
+            assert ((got.cpu().double() - ref).abs() <= tol * ref.abs().max().item() + slack + tol * 0.1 * terms).all(), case
+        # cosine embedding loss with target +1 on the same rows, every other row masked out
+        keep = torch.arange(n) % 2 == 0
+
+        def ref_cos(a, b):
+            return 1.5 * torch.nn.CosineEmbeddingLoss()(a[keep], b[keep], a.new_ones(int(keep.sum())))
+        want, (gx,) = _oracle_grad(ref_cos, o1, others=(t1,))
+        xd = o1.to(device).requires_grad_()
+        loss = ta.cosine_embedding_loss(xd, t1.to(device), keep.to(device), 1.5)
+        loss.backward()
+        case = f"cosine n={n} c={c}"
+        assert rel_err(loss.item(), want) < tol or abs(loss.item() - want) < 1e-6, case
+        slack = gx.abs() * (2.0 ** -8 if dtype != torch.float32 else 0.0)
+        terms = 1.5 / (int(keep.sum()) * o1.double().norm(dim=1, keepdim=True))
+        assert ((xd.grad.cpu().double() - gx).abs() <= tol * gx.abs().max().item() + slack + tol * 0.1 * terms).all(), case
+        assert (xd.grad.cpu()[~keep] == 0).all(), case
+
+
 def _nce_inputs(n, c, seed, dtype):
     g = seeded(seed)
     q = torch.nn.functional.normalize(torch.randn(n, c, generator=g), dim=1).to(dtype)
