@@ -438,6 +438,23 @@ def test_infonce_any_width_and_temperature(device, dtype, n, c, tau):
     assert (err <= 1e-4 * peak + gw.abs() * store + (2.0 ** -24 if dtype == torch.float16 else 0.0)).all()
 
 
+def test_infonce_fp32_path_over_widths_and_row_counts(device):
+    # the fp32-MFMA kernels pad the width to the matrix instruction's step and run widths above 256 as two
+    # feature groups; rows come in tiles of 32 per wavefront, 128 per workgroup: every edge of both
+    for n, c in ((1, 1), (2, 2), (31, 3), (33, 5), (32, 31), (129, 33), (127, 63), (5, 65), (64, 127), (65, 129),
+                 (40, 255), (128, 257), (130, 320), (3, 511), (97, 512)):
+        q, k = _nce_inputs(n, c, 5000 + n + c, torch.float32)
+        want, (gw,) = _oracle_grad(lambda a, b: ts_oracle.infonce(a, b, 0.2), q, others=(k,))
+        qd = q.to(device).requires_grad_()
+        loss = ta.infonce_loss(qd, k.to(device), 0.2)
+        loss.backward()
+        case = f"n={n} c={c}"
+        assert rel_err(loss.item(), want) < 2e-5 or abs(loss.item() - want) < 1e-6, case
+        # at width 1 the whole gradient is the projected-out component: bounded by its terms, 2 tau / (n tau |q|)
+        terms = 2.0 / (n * q.double().norm(dim=1, keepdim=True))
+        assert ((qd.grad.cpu().double() - gw).abs() <= 1e-4 * gw.abs().max().item() + 1e-6 * terms).all(), case
+
+
 @pytest.mark.parametrize("n,c,tau", [(1000, 256, 0.2), (4096, 256, 0.2), (300, 128, 0.07), (130, 64, 0.5), (1, 64, 0.2)])
 def test_infonce_fp32_inputs_in_fp32_arithmetic(device, n, c, tau):
     # the reference's TSPipe MoCo run is fp32 end to end (benchmarks/moco-v3/main.py:151-160, no autocast):
