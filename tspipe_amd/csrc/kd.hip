@@ -386,15 +386,14 @@ __global__ __launch_bounds__(BLOCK, (KREG * GROUP > 1024 ? 4 : 1)) void kd_rows_
         const Vec16<T> lt = load16(trow + g.head + v * VEC), ls = load16(srow + g.head + v * VEC);
         __builtin_memcpy(&stage_t[v], &lt, 16);
         __builtin_memcpy(&stage_s[v], &ls, 16);
-      } else if constexpr (GROUP <= kWave) {
-        // rows that a wavefront or less holds: short-lived workgroups streaming through, where
-        // non-temporal loads pay (32768 x 1000 fp32: 75.0 -> 71.0 us; 65536 x 100: 22.7 -> 22.4); on the
-        // workgroup-wide rows they cost (4096 x 30522 bf16 under a 15 % mask: 83 against 77)
+      } else {
+        // The logits are read once: non-temporal loads.  On working sets beyond the last-level cache,
+        // us per call: 32768 x 1000 fp32 75.0 -> 71.0, 16384 x 4000 fp32 144 -> 128, 8192 x 16000 fp32
+        // 283 -> 264, 4096 x 30522 bf16 with and without a mask unchanged.  (A loop on one set of logits
+        // that fits that cache loses, 8192 x 4096 bf16 45 -> 52: its own plain loads were what kept the
+        // set there from call to call.)
         rt[j] = load16_stream(trow + g.head + v * VEC);
         rs[j] = load16_stream(srow + g.head + v * VEC);
-      } else {
-        rt[j] = load16(trow + g.head + v * VEC);
-        rs[j] = load16(srow + g.head + v * VEC);
       }
     }
   }

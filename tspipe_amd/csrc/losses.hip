@@ -415,7 +415,7 @@ __global__ __launch_bounds__(1024) void mse_finalize_kernel(const float* __restr
 // leaves it out.  No counting launch in front: a workgroup that computes
 // counts the mask's few kilobytes itself while its loads are in flight.
 // 4096 x 30522 bf16, us per call under a 15 % mask / without a mask (two sets
-// of logits in turn): 74 / 147 against 119 / - for the span kernel above;
+// of logits in turn, plain loads): 74 / 147 against 119 / - for the span kernel above;
 // threads x vectors in flight 256 x 8: 77 / 157, 256 x 4: 80 / 165, 512 x 4:
 // 77 / 147, 512 x 2: 78 / 152, 1024 x 4: 74 / 138 (but the zero-fill half alone
 // 58 against 54), 1024 x 2: 78 / 140.
@@ -478,8 +478,9 @@ __global__ __launch_bounds__(kMseLongBlock) void mse_long_rows_kernel(const RowP
     for (int j = 0; j < REGS; ++j) {
       const int64_t v = base + tid + (int64_t)j * kMseLongBlock;
       if (v < nvec) {
-        vs[j] = load16(s4 + v * VEC);
-        vt[j] = load16(t4 + v * VEC);
+        // read once: non-temporal loads (us per call, 15 % / 50 % / no mask: 73.6 / 112 / 146.5 -> 71 / 99.5 / 140.5)
+        vs[j] = load16_stream(s4 + v * VEC);
+        vt[j] = load16_stream(t4 + v * VEC);
         if (acc_g) vg[ACC ? j : 0] = load16(g4 + v * VEC);
       }
     }
