@@ -584,6 +584,38 @@ def test_kd_ce_mse_at_every_row_width_boundary(device, dtype):
             assert (sd.grad.cpu()[4] == 0).all(), case   # neither masked in nor labelled
 
 
+@pytest.mark.parametrize("rows", [77, 1027, 8195])
+def test_kd_ce_counts_from_a_mask_that_starts_off_an_8_byte_boundary(device, rows):
+    # short rows under a mask and with labels take a counting launch that reads the mask eight rows at a
+    # time when it can; a mask that is a view three bytes into a buffer cannot, and must count the same
+    g = seeded(930 + rows)
+    V = 50
+    s = torch.randn(rows, V, generator=g).to(device)
+    t = torch.randn(rows, V, generator=g).to(device)
+    mask = (torch.rand(rows, generator=g) < 0.4).to(device)
+    y = torch.randint(0, V, (rows,), generator=g)
+    y[torch.rand(rows, generator=g) < 0.5] = -100
+    y = y.to(device)
+    big = torch.zeros(rows + 16, dtype=torch.bool, device=device)
+    off = big[3:3 + rows]
+    off.copy_(mask)
+    assert off.data_ptr() % 8 == 3 and mask.data_ptr() % 8 == 0
+    a = s.clone().requires_grad_()
+    la = ta.kd_ce_loss(a, t, y, 2.0, kd_weight=0.5, ce_weight=2.0, row_mask=mask)
+    la.backward()
+    b = s.clone().requires_grad_()
+    lb = ta.kd_ce_loss(b, t, y, 2.0, kd_weight=0.5, ce_weight=2.0, row_mask=off)
+    lb.backward()
+    assert torch.equal(la, lb) and torch.equal(a.grad, b.grad)
+    # and against the closed form of the two means
+    sm, tm = s.cpu().double(), t.cpu().double()
+    m, yy = mask.cpu(), y.cpu()
+    kd = torch.nn.functional.kl_div(torch.log_softmax(sm[m] / 2.0, -1), torch.softmax(tm[m] / 2.0, -1),
+                                    reduction="batchmean") * 4.0
+    ce = torch.nn.functional.cross_entropy(sm, yy, ignore_index=-100)
+    assert rel_err(la.item(), (0.5 * kd + 2.0 * ce).item()) < 1e-5
+
+
 def test_cosine_embedding_loss(device):
     g = seeded(220)
     x = torch.randn(3, 7, 48, generator=g)

@@ -152,6 +152,38 @@ __device__ __forceinline__ float block_sum(float v, float* lds) {
   return r;
 }
 
+// This thread's share of sum(v[0..n)) when NT threads of one workgroup walk the
+// array together, in a fixed order.  One workgroup has to get through the whole
+// array, so the walk is bound by memory latency: 16-byte loads, eight of them
+// in flight per thread (65536 values are two round trips; element by element
+// they were 64, and the final sum of a 65536-row loss took 18 us instead of 5).
+template <int NT>
+__device__ __forceinline__ float thread_share_of_sum(const float* __restrict__ v, int64_t n) {
+  constexpr int kInFlight = 8;
+  float acc = 0.f;
+  int64_t done = 0;
+  if (((uintptr_t)v & 15u) == 0) {
+    const int64_t n4 = n / 4;
+    const f32x4* v4 = reinterpret_cast<const f32x4*>(v);
+    f32x4 s4 = {0.f, 0.f, 0.f, 0.f};
+    for (int64_t i0 = threadIdx.x; i0 < n4; i0 += (int64_t)NT * kInFlight) {
+      f32x4 a[kInFlight];
+#pragma unroll
+      for (int j = 0; j < kInFlight; ++j) {
+        const int64_t i = i0 + (int64_t)j * NT;
+        a[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (i < n4) a[j] = v4[i];
+      }
+#pragma unroll
+      for (int j = 0; j < kInFlight; ++j) s4 += a[j];
+    }
+    acc = (s4[0] + s4[1]) + (s4[2] + s4[3]);
+    done = n4 * 4;
+  }
+  for (int64_t i = done + threadIdx.x; i < n; i += NT) acc += v[i];
+  return acc;
+}
+
 // Number of non-zero mask bytes, counted by the calling workgroup (every
 // thread gets the result; `lds` holds NT / 64 floats).  The mask of a batch is
 // a few kilobytes, so this is an L2-resident read and one block reduction --
@@ -162,13 +194,23 @@ __device__ __forceinline__ float mask_count_block(const uint8_t* __restrict__ ma
   int c = 0;
   const int64_t n8 = ((uintptr_t)mask & 7u) == 0 ? n / 8 : 0;
   const uint64_t* m8 = reinterpret_cast<const uint64_t*>(mask);
-  for (int64_t i = threadIdx.x; i < n8; i += NT) {
-    uint64_t v = m8[i];
-    // a byte counts when any of its bits is set
-    v |= v >> 4;
-    v |= v >> 2;
-    v |= v >> 1;
-    c += __popcll(v & 0x0101010101010101ull);
+  constexpr int kInFlight = 4;  // loads per thread and trip: one workgroup walks the whole mask
+  for (int64_t i0 = threadIdx.x; i0 < n8; i0 += (int64_t)NT * kInFlight) {
+    uint64_t w[kInFlight];
+#pragma unroll
+    for (int j = 0; j < kInFlight; ++j) {
+      const int64_t i = i0 + (int64_t)j * NT;
+      w[j] = i < n8 ? m8[i] : 0;
+    }
+#pragma unroll
+    for (int j = 0; j < kInFlight; ++j) {
+      uint64_t v = w[j];
+      // a byte counts when any of its bits is set
+      v |= v >> 4;
+      v |= v >> 2;
+      v |= v >> 1;
+      c += __popcll(v & 0x0101010101010101ull);
+    }
   }
   for (int64_t i = n8 * 8 + threadIdx.x; i < n; i += NT) c += mask[i] != 0;
   // per-thread counts stay far below 2^24 for any n the launchers accept: the float sum is exact

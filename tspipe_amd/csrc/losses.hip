@@ -11,9 +11,7 @@ __global__ __launch_bounds__(1024) void sum_scale_kernel(const float* __restrict
                                                          float scale, const int* __restrict__ denom_dev,
                                                          float denom, float* __restrict__ out) {
   __shared__ float lds[1024 / kWave];
-  float acc = 0.f;
-  for (int64_t i = threadIdx.x; i < n; i += 1024) acc += v[i];
-  const float tot = block_sum<1024 / kWave>(acc, lds);
+  const float tot = block_sum<1024 / kWave>(thread_share_of_sum<1024>(v, n), lds);
   if (threadIdx.x == 0) {
     const float d = denom_dev ? (float)(*denom_dev) : denom;
     *out = scale * (tot / d);
@@ -105,10 +103,7 @@ __global__ __launch_bounds__(256) void byol_rows_kernel(const ByolArgs args, int
 __global__ __launch_bounds__(1024) void mask_count_kernel(const uint8_t* __restrict__ mask, int64_t n,
                                                           int* __restrict__ out) {
   __shared__ float lds[1024 / kWave];
-  int c = 0;
-  for (int64_t i = threadIdx.x; i < n; i += 1024) c += mask[i] != 0;
-  // per-thread counts stay below 2^14 for any n the launchers accept, so the float sum is exact
-  const float tot = block_sum<1024 / kWave>((float)c, lds);
+  const float tot = mask_count_block<1024>(mask, n, lds);  // exact in float for any n the launchers accept
   if (threadIdx.x == 0) *out = (int)tot;
 }
 
@@ -263,21 +258,27 @@ __global__ __launch_bounds__(1024) void cosine_finalize_kernel(const float* __re
                                                                float* __restrict__ out) {
   __shared__ float lds[1024 / kWave];
   const float n_sel = mask ? mask_count_block<1024>(mask, n, lds) : (float)n;
-  float acc = 0.f;
-  for (int64_t i = threadIdx.x; i < n; i += 1024) acc += row_loss[i];
-  const float tot = block_sum<1024 / kWave>(acc, lds);
+  const float tot = block_sum<1024 / kWave>(thread_share_of_sum<1024>(row_loss, n), lds);
   if (threadIdx.x == 0) *out = weight * (tot / n_sel);
 }
 
 // ---- squared error between logits (fused backward) -----------------------
 //   loss = weight * sum over selected rows, all columns of (s - t)^2 / denom
 //   grad = d loss / d s = (2 weight / denom)(s - t) on selected rows, 0 elsewhere
-// denom = selected rows (x V when the mean runs over elements).  A workgroup
-// owns kMseSpan elements of one row and leaves one partial sum.
+// denom = selected rows (x V when the mean runs over elements).  Every row
+// leaves one partial sum; a last single-workgroup launch adds them in a fixed
+// order.
+// Rows below kMseLongMin elements: GROUP lanes of a wavefront own a row (16
+// lanes for rows of up to 32 16-byte vectors, a whole wavefront beyond), four
+// wavefronts to a workgroup, no LDS and no barrier: each lane keeps up to four
+// vectors per operand in flight, the row's sum is a shuffle reduction.
+// 32768 x 1000 fp32, us per call without a mask / under a 15 % mask: 71 / 49
+// against 115 / 110 for the form this replaces (a 256-thread workgroup per
+// 4096 elements of a row with a block reduction: 250 of 1024 vector slots used
+// at that width).  kMseSpan only sizes the workspace now.
 constexpr int kMseBlock = 256;
-// 4096 x 30522 bf16 under a 15 % mask, us per call: span 2048: 154, 4096: 122, 8192: 148, 16384: 201;
-// 512 threads x 4096: 159, 512 x 8192: 131, 1024 x 8192: 223, 1024 x 16384: 149
 constexpr int kMseSpan = 4096;
+constexpr int kMseShortRegs = 4;
 
 // One element: its squared difference into acc, its gradient (or a zero) out.
 template <typename T>
@@ -287,103 +288,92 @@ __device__ __forceinline__ T mse_grad_one(T sv, T tv, T gold, float k, int accum
   return from_f32<T>(accumulate ? to_f32(gold) + k * d : k * d);
 }
 
-// A workgroup owns kMseSpan elements of one row.  Where s, t and the gradient
-// row sit at the same offset from a 16-byte boundary (the usual case) these
-// are the span's 16-byte vectors of the row's aligned middle, and the first
-// workgroup of the row also takes the few elements in front of and behind
-// that middle; otherwise the span is walked element by element.
-template <typename T>
+template <typename T, int GROUP, bool ACC>
 __global__ __launch_bounds__(kMseBlock) void mse_rows_kernel(const RowPieces tab, const uint8_t* __restrict__ mask,
                                                               const int* __restrict__ n_sel_dev, int64_t n_rows,
-                                                              int64_t V, float weight, int per_element, int accumulate,
+                                                              int64_t V, float weight, int per_element,
                                                               float* __restrict__ partial) {
   constexpr int VEC = 16 / sizeof(T);
-  constexpr int kVecSpan = kMseSpan / VEC;          // vectors per workgroup
-  constexpr int kPerThread = kVecSpan / kMseBlock;  // vectors per thread (2 for 16-bit types, 4 for fp32)
-  static_assert(kPerThread >= 1 && kVecSpan % kMseBlock == 0, "span and block do not fit the vector width");
-  __shared__ float lds[kMseBlock / kWave];
-  const int64_t parts = gridDim.x;
+  constexpr int accumulate = ACC ? 1 : 0;
+  const int gtid = threadIdx.x % GROUP;
+  const int64_t row = (int64_t)blockIdx.x * (kMseBlock / GROUP) + threadIdx.x / GROUP;
+  if (row >= n_rows) return;  // whole groups leave together; nothing below synchronises across groups
+  const bool sel = !mask || mask[row] != 0;
+  const RowPtrs<T> rp = row_ptrs<T>(tab, row);
+  const T* sr = rp.a;
+  const T* tr = rp.b;
+  T* gr = rp.g;
+  const T zero = from_f32<T>(0.f);
+  if (!sel) {
+    if (gtid == 0) partial[row] = 0.f;
+    if (!gr || ACC) return;
+    const uint32_t mis = (uint32_t)((uintptr_t)gr & 15u);
+    int64_t head = (int64_t)(((16u - mis) & 15u) / sizeof(T));
+    if (head > V) head = V;
+    const int64_t nvec = (V - head) / VEC, tail0 = head + nvec * VEC;
+    Vec16<T> z;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) z.v[e] = zero;
+    if (gtid < head) gr[gtid] = zero;
+    for (int64_t v = gtid; v < nvec; v += GROUP) store16(gr + head + v * VEC, z);  // plain stores: a zero-fill
+    if (tail0 + gtid < V) gr[tail0 + gtid] = zero;
+    return;
+  }
   const float rows_sel = n_sel_dev ? (float)(*n_sel_dev) : (float)n_rows;
-  const float denom = per_element ? rows_sel * (float)V : rows_sel;
-  const float k = 2.f * weight / denom;
-  const int tid = threadIdx.x;
-  for (int64_t row = blockIdx.y; row < n_rows; row += gridDim.y) {
-    const bool sel = !mask || mask[row] != 0;
-    float acc = 0.f;
-    const RowPtrs<T> rp = row_ptrs<T>(tab, row);
-    const T* sr = rp.a;
-    const T* tr = rp.b;
-    T* gr = rp.g;
-    if (sel || (gr && !accumulate)) {
-      const uint32_t mis = (uint32_t)((uintptr_t)sr & 15u);
-      const bool alike = mis == (uint32_t)((uintptr_t)tr & 15u) && (!gr || mis == (uint32_t)((uintptr_t)gr & 15u)) &&
-                         mis % sizeof(T) == 0;
-      int64_t head = alike ? (int64_t)(((16u - mis) & 15u) / sizeof(T)) : V;
-      if (head > V) head = V;
-      const int64_t nvec = (V - head) / VEC, tail0 = head + nvec * VEC;
-      const T zero = from_f32<T>(0.f);
-      auto one = [&](int64_t i) {
-        if (sel) {
-          const T gv = mse_grad_one<T>(sr[i], tr[i], (gr && accumulate) ? gr[i] : zero, k, accumulate, acc);
-          if (gr) gr[i] = gv;
-        } else {
-          gr[i] = zero;
-        }
-      };
-      if (!alike) {
-        // consecutive lanes, consecutive elements
-        const int64_t i0 = (int64_t)blockIdx.x * kMseSpan + tid;
+  const float k = 2.f * weight / (per_element ? rows_sel * (float)V : rows_sel);
+  const uint32_t mis = (uint32_t)((uintptr_t)sr & 15u);
+  const bool alike = mis == (uint32_t)((uintptr_t)tr & 15u) && (!gr || mis == (uint32_t)((uintptr_t)gr & 15u)) &&
+                     mis % sizeof(T) == 0;
+  int64_t head = alike ? (int64_t)(((16u - mis) & 15u) / sizeof(T)) : V;
+  if (head > V) head = V;
+  const int64_t nvec = (V - head) / VEC, tail0 = head + nvec * VEC;
+  const bool acc_g = gr && ACC;
+  float acc = 0.f;
+  // the few elements in front of and behind the row's aligned middle (all of the row when the operands
+  // are aligned differently)
+  for (int64_t i = gtid; i < head; i += GROUP) {
+    const T gv = mse_grad_one<T>(sr[i], tr[i], acc_g ? gr[i] : zero, k, accumulate, acc);
+    if (gr) gr[i] = gv;
+  }
+  if (tail0 + gtid < V) {
+    const int64_t i = tail0 + gtid;
+    const T gv = mse_grad_one<T>(sr[i], tr[i], acc_g ? gr[i] : zero, k, accumulate, acc);
+    if (gr) gr[i] = gv;
+  }
+  const T* s4 = sr + head;
+  const T* t4 = tr + head;
+  T* g4 = gr + head;
+  for (int64_t base = 0; base < nvec; base += (int64_t)GROUP * kMseShortRegs) {
+    Vec16<T> vs[kMseShortRegs], vt[kMseShortRegs], vg[ACC ? kMseShortRegs : 1];
 #pragma unroll
-        for (int j = 0; j < kMseSpan / kMseBlock; ++j)
-          if (i0 + j * kMseBlock < V) one(i0 + j * kMseBlock);
-      } else {
-        if (blockIdx.x == 0) {
-          if (tid < head) one(tid);
-          if (tail0 + tid < V) one(tail0 + tid);
-        }
-        const T* s4 = sr + head;
-        const T* t4 = tr + head;
-        T* g4 = gr + head;
-        const int64_t v0 = (int64_t)blockIdx.x * kVecSpan + tid;
-        Vec16<T> vs[kPerThread], vt[kPerThread], vg[kPerThread];
+    for (int j = 0; j < kMseShortRegs; ++j) {
+      const int64_t v = base + gtid + (int64_t)j * GROUP;
+      if (v < nvec) {
+        vs[j] = load16_stream(s4 + v * VEC);  // read once
+        vt[j] = load16_stream(t4 + v * VEC);
+        if (acc_g) vg[ACC ? j : 0] = load16(g4 + v * VEC);
+      }
+    }
 #pragma unroll
-        for (int j = 0; j < kPerThread; ++j) {
-          const int64_t v = v0 + j * kMseBlock;
-          if (v < nvec && sel) {
-            vs[j] = load16(s4 + v * VEC);
-            vt[j] = load16(t4 + v * VEC);
-            if (gr && accumulate) vg[j] = load16(g4 + v * VEC);
-          }
-        }
+    for (int j = 0; j < kMseShortRegs; ++j) {
+      const int64_t v = base + gtid + (int64_t)j * GROUP;
+      if (v < nvec) {
+        Vec16<T> o;
 #pragma unroll
-        for (int j = 0; j < kPerThread; ++j) {
-          const int64_t v = v0 + j * kMseBlock;
-          if (v < nvec) {
-            Vec16<T> o;
-#pragma unroll
-            for (int e = 0; e < VEC; ++e)
-              o.v[e] = sel ? mse_grad_one<T>(vs[j].v[e], vt[j].v[e], (gr && accumulate) ? vg[j].v[e] : zero, k,
-                                             accumulate, acc)
-                           : zero;
-            if (gr) {
-              // a computed gradient streams out; a zero-fill keeps plain stores (as in the KD kernels)
-              if (sel && !accumulate)
-                store16_stream(g4 + v * VEC, o);
-              else
-                store16(g4 + v * VEC, o);
-            }
-          }
+        for (int e = 0; e < VEC; ++e)
+          o.v[e] = mse_grad_one<T>(vs[j].v[e], vt[j].v[e], acc_g ? vg[ACC ? j : 0].v[e] : zero, k, accumulate, acc);
+        if (gr) {
+          if (ACC)
+            store16(g4 + v * VEC, o);
+          else
+            store16_stream(g4 + v * VEC, o);
         }
       }
     }
-    if (!sel) {  // uniform: the workgroup shares the row; nothing to add up
-      if (tid == 0) partial[row * parts + blockIdx.x] = 0.f;
-      continue;
-    }
-    const float tot = block_sum<kMseBlock / kWave>(acc, lds);
-    if (tid == 0) partial[row * parts + blockIdx.x] = tot;
-    __syncthreads();  // lds is reused by the next row
   }
+#pragma unroll
+  for (int off = GROUP / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off, kWave);
+  if (gtid == 0) partial[row] = acc;
 }
 
 // out (+)= weight * sum(partial) / denom, fixed summation order
@@ -395,9 +385,7 @@ __global__ __launch_bounds__(1024) void mse_finalize_kernel(const float* __restr
   __shared__ float lds[1024 / kWave];
   // no counting launch ran in front (the long-row route): the selected rows are counted here
   const float counted = (!n_sel_dev && mask) ? mask_count_block<1024>(mask, n_rows, lds) : (float)n_rows;
-  float acc = 0.f;
-  for (int64_t i = threadIdx.x; i < n; i += 1024) acc += partial[i];
-  const float tot = block_sum<1024 / kWave>(acc, lds);
+  const float tot = block_sum<1024 / kWave>(thread_share_of_sum<1024>(partial, n), lds);
   if (threadIdx.x == 0) {
     const float rows_sel = n_sel_dev ? (float)(*n_sel_dev) : counted;
     const float denom = per_element ? rows_sel * (float)V : rows_sel;
@@ -557,14 +545,26 @@ int launch_mse(const RowPieces& tab, const uint8_t* mask, int64_t n_rows, int64_
     int rc = check_launch();
     if (rc) return rc;
   }
-  const int64_t parts = mse_parts(V);
-  const int64_t gy = n_rows < 65535 ? n_rows : 65535;
-  hipLaunchKernelGGL((mse_rows_kernel<T>), dim3((unsigned)parts, (unsigned)gy), dim3(kMseBlock), 0, stream, tab, mask,
-                     mask ? n_sel : (const int*)nullptr, n_rows, V, weight, per_element, accumulate, partial);
+  // rows of up to 32 vectors (a ragged first and last one counted): 16 lanes each, else a wavefront
+  const int64_t vecs = (V + Vec16<T>::N - 1) / Vec16<T>::N + 1;
+  const int group = vecs <= 32 ? 16 : kWave;
+  const int64_t per_block = kMseBlock / group;
+  const int64_t blocks = (n_rows + per_block - 1) / per_block;
+  if (blocks * kMseBlock > 0xffffffffLL) return TS_ERR_RANGE;
+  const int* n_sel_arg = mask ? n_sel : (const int*)nullptr;
+#define TS_MSE_LAUNCH(GROUP, ACC)                                                                              \
+  hipLaunchKernelGGL((mse_rows_kernel<T, GROUP, ACC>), dim3((unsigned)blocks), dim3(kMseBlock), 0, stream, tab, \
+                     mask, n_sel_arg, n_rows, V, weight, per_element, partial)
+  if (group == 16) {
+    if (accumulate) TS_MSE_LAUNCH(16, true); else TS_MSE_LAUNCH(16, false);
+  } else {
+    if (accumulate) TS_MSE_LAUNCH(kWave, true); else TS_MSE_LAUNCH(kWave, false);
+  }
+#undef TS_MSE_LAUNCH
   int rc = check_launch();
   if (rc) return rc;
-  hipLaunchKernelGGL(mse_finalize_kernel, dim3(1), dim3(1024), 0, stream, partial, n_rows * parts,
-                     mask ? n_sel : (const int*)nullptr, mask, n_rows, V, weight, per_element, accumulate, loss_out);
+  hipLaunchKernelGGL(mse_finalize_kernel, dim3(1), dim3(1024), 0, stream, partial, n_rows, n_sel_arg, mask, n_rows, V,
+                     weight, per_element, accumulate, loss_out);
   return check_launch();
 }
 
