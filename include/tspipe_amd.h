@@ -399,7 +399,10 @@ int ts_infonce_pieces_fwd_bwd(const void* const* q1_pieces, const void* const* k
 /* ------------------------------------------------------------------------ */
 /* DeferredBatchNorm (tspipe/batchnorm.py).                           */
 /* x, y, dy, dx: fp32 [N, C, HW] contiguous (NCHW with HW = prod of the      */
-/* trailing dims).                                                           */
+/* trailing dims).  Two families of kernels behind every call: planes of     */
+/* more than 256 elements are dealt a wavefront each; smaller ones (the late  */
+/* stages of a ResNet, [N, C, 1, 1]) are walked as flat ranges of a sample    */
+/* when C*HW is a multiple of 4 and the tensors sit on 16-byte boundaries.    */
 /* ------------------------------------------------------------------------ */
 
 /* _track (batchnorm.py:45-59) fused with the statistics F.batch_norm(
@@ -410,7 +413,7 @@ int ts_infonce_pieces_fwd_bwd(const void* const* q1_pieces, const void* const* k
  *   - turned into ub_mean = S/cnt and ub_invstd = 1/sqrt(max(Q/cnt - mean^2,0)
  *     + eps), cnt = N*HW, unless those are NULL.
  * One launch: the last workgroup of a channel to finish does the channel's
- * bookkeeping.  ws: ts_bn_stats_workspace_bytes(C) bytes (3*C floats: two
+ * bookkeeping (small planes: two short launches).  ws: ts_bn_stats_workspace_bytes(C) bytes (3*C floats: two
  * sums and a ticket counter per channel) that are ZERO on entry; the call
  * leaves them zero again.  Calls that share a ws must not overlap on the
  * device (the last workgroup of a channel reads and clears what the others

@@ -138,7 +138,12 @@ def test_deferred_bn_backward(device):
 
 
 @pytest.mark.parametrize("shape", [(2, 3, 1), (2, 5, 1, 1), (1, 2, 130, 130), (3, 4, 64, 64), (5, 3, 257),
-                                   (33, 2, 7, 7), (2, 70, 3, 3), (9, 1, 4, 5), (17, 6, 2)])
+                                   (33, 2, 7, 7), (2, 70, 3, 3), (9, 1, 4, 5), (17, 6, 2),
+                                   # planes of up to 256 elements with C * HW a multiple of 4: the flat-tile kernels
+                                   # (tiles that cut channels, one-element planes, a thread and a wavefront per
+                                   # channel in the final sums, more than one tile and more than one slab)
+                                   (64, 512, 7, 7), (37, 2048, 1, 1), (40, 24, 4, 4), (7, 36, 17), (3, 5, 16, 16),
+                                   (130, 260, 3, 3), (5, 1028, 1)])
 def test_deferred_bn_forward_and_backward_over_plane_and_batch_sizes(device, shape):
     # planes of one element, planes longer than one round of a wavefront's loads, planes that start off a
     # 16-byte boundary (odd sizes), more samples than a workgroup's slab, a single channel, many channels:
@@ -331,13 +336,14 @@ def test_a_refused_call_leaves_the_next_forward_correct(device, monkeypatch):
     assert (y.cpu().double() - want).abs().max() < 2e-5
 
 
-def test_stand_alone_statistics_pass_is_one_launch_that_cleans_up(device):
+@pytest.mark.parametrize("N,C,H,W", [(16, 24, 56, 56), (48, 512, 7, 7), (300, 64, 1, 1)])
+def test_stand_alone_statistics_pass_is_one_launch_that_cleans_up(device, N, C, H, W):
     # ts_bn_stats with several workgroups per channel: the last one to finish does the channel's
-    # bookkeeping and leaves the 3C-float workspace (sums and ticket counters) zero again
+    # bookkeeping and leaves the 3C-float workspace (sums and ticket counters) zero again; on small
+    # planes (the second and third shape) a second short launch does that instead
     from tspipe_amd import _lib
     lib = _lib.lib()
     st = torch.cuda.current_stream(device).cuda_stream
-    N, C, H, W = 16, 24, 56, 56
     g = seeded(91)
     z = lambda n: torch.zeros(n, device=device)  # noqa: E731
     ws, acc_s, acc_q, mean, inv = z(3 * C), z(C), z(C), z(C), z(C)

@@ -408,6 +408,416 @@ __global__ __launch_bounds__(kBnBlock) void bn_bwd_dx_kernel(const float* __rest
   }
 }
 
+// ---------------------------------------------------------------------------
+// Small planes (HW <= kBnFlatMaxHW): flat tiles.  A plane of a late ResNet
+// stage is 49 or 16 elements; a wavefront per plane leaves most lanes idle
+// there (and a [N, C, 1, 1] input one lane in 64).  But the C planes of one
+// sample are contiguous, so a workgroup takes a range of kBnFlatElems
+// consecutive floats of every sample of its slab -- whole 16-byte vectors,
+// one per thread and sample, fully coalesced, no index arithmetic in the loop --
+// whatever channels that range covers.  A thread's four elements keep the same
+// channels from sample to sample, so it accumulates per element in registers;
+// at the end the per-position partial sums go through LDS, a thread (planes of
+// up to 16 elements) or a wavefront per channel adds up that channel's
+// positions, and one atomic add per channel and quantity leaves the workgroup,
+// as in the kernels above.  Needs C * HW to be a multiple of 4 and the tensors
+// on 16-byte boundaries; everything else keeps the plane kernels.
+// Through the C ABI, us: [256, 512, 7, 7] training forward 134 -> 20 and backward
+// 160 -> 26; [256, 2048, 7, 7] 316 -> 55-61; [512, 512, 4, 4] 122 -> 14;
+// [4096, 512, 1, 1] 794 -> 30.
+// ---------------------------------------------------------------------------
+constexpr int kBnFlatElems = kBnBlock * 4;
+constexpr int64_t kBnFlatMaxHW = 256;
+constexpr int kBnFlatMaxCh = kBnFlatElems + 1;  // channels a tile can touch (HW = 1, plus one cut at the front)
+constexpr int kBnFlatShiftN = 16;
+constexpr int kBnFlatInFlight = 16;  // samples a thread has in flight (one 16-byte vector each); half per operand with two
+#ifndef TS_BN_FLAT_SLABS
+#define TS_BN_FLAT_SLABS 16
+#endif
+constexpr int64_t kBnFlatMaxSlabs = TS_BN_FLAT_SLABS;
+
+struct FlatTile {
+  uint32_t f0;     // first float of the tile inside a sample
+  int nelem;       // floats of the tile (a multiple of 4)
+  uint32_t c_lo;   // first channel the tile touches
+  int nch;         // channels it touches
+  bool valid;      // this thread's vector lies inside the tile
+  int ch[4];       // tile-local channel of each of the thread's four elements
+};
+
+__device__ __forceinline__ FlatTile flat_tile(int64_t C, int64_t HW) {
+  FlatTile t;
+  const uint32_t E = (uint32_t)(C * HW), hw = (uint32_t)HW;
+  t.f0 = blockIdx.x * (uint32_t)kBnFlatElems;
+  t.nelem = (int)((E - t.f0 < (uint32_t)kBnFlatElems) ? E - t.f0 : (uint32_t)kBnFlatElems);
+  t.c_lo = t.f0 / hw;
+  t.nch = (int)((t.f0 + (uint32_t)t.nelem - 1) / hw - t.c_lo) + 1;
+  const int e0 = 4 * (int)threadIdx.x;
+  t.valid = e0 < t.nelem;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) t.ch[j] = t.valid ? (int)((t.f0 + (uint32_t)(e0 + j)) / hw - t.c_lo) : 0;
+  return t;
+}
+
+// The shift of a channel on this path: the mean of its first (up to) 16
+// values in (sample, position) order, added up serially -- the same loads and
+// the same order wherever it is computed, so the statistics and the
+// normalising launch agree on it to the bit.
+__device__ __forceinline__ float flat_shift(const float* __restrict__ x, uint32_t c, int64_t N, int64_t C,
+                                            int64_t HW) {
+  const int64_t avail = N * HW;
+  const int m = avail < kBnFlatShiftN ? (int)avail : kBnFlatShiftN;
+  float v[kBnFlatShiftN];
+  int64_t n = 0, i = 0;
+#pragma unroll
+  for (int j = 0; j < kBnFlatShiftN; ++j) {
+    v[j] = j < m ? x[(n * C + c) * HW + i] : 0.f;
+    if (++i == HW) {
+      i = 0;
+      ++n;
+    }
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int j = 0; j < kBnFlatShiftN; ++j) s += v[j];
+  return s / (float)m;
+}
+
+// Adds up, per channel of the tile, the per-position partial sums in la / lb
+// (kBnFlatElems floats each, zeros beyond the tile) and hands (channel, a, b)
+// to emit on one thread per channel.
+template <typename F>
+__device__ __forceinline__ void flat_reduce_channels(const FlatTile& t, int64_t HW, const float* la, const float* lb,
+                                                     F emit) {
+  const uint32_t hw = (uint32_t)HW;
+  auto range = [&](int lc, int& lo, int& hi) {
+    const uint32_t c = t.c_lo + (uint32_t)lc;
+    const uint32_t b = c * hw, e = b + hw, end = t.f0 + (uint32_t)t.nelem;
+    lo = (int)((b > t.f0 ? b : t.f0) - t.f0);
+    hi = (int)((e < end ? e : end) - t.f0);
+  };
+  if (HW <= 16) {
+    for (int lc = threadIdx.x; lc < t.nch; lc += kBnBlock) {
+      int lo, hi;
+      range(lc, lo, hi);
+      float a = 0.f, b = 0.f;
+      for (int i = lo; i < hi; ++i) {
+        a += la[i];
+        b += lb[i];
+      }
+      emit(t.c_lo + (uint32_t)lc, a, b);
+    }
+  } else {
+    const int lane = threadIdx.x % kWave, w = threadIdx.x / kWave;
+    for (int lc = w; lc < t.nch; lc += kBnBlock / kWave) {
+      int lo, hi;
+      range(lc, lo, hi);
+      float a = 0.f, b = 0.f;
+      for (int i = lo + lane; i < hi; i += kWave) {
+        a += la[i];
+        b += lb[i];
+      }
+      a = wave_sum(a);
+      b = wave_sum(b);
+      if (lane == 0) emit(t.c_lo + (uint32_t)lc, a, b);
+    }
+  }
+}
+
+// First launch of the fused training forward on small planes: sum(x - k) and
+// sum((x - k)^2) per channel into ws.  gridDim = (tiles of a sample, slabs).
+__global__ __launch_bounds__(kBnBlock) void bn_flat_stats_kernel(const float* __restrict__ x, int64_t N, int64_t C,
+                                                                 int64_t HW, int64_t slab, float* __restrict__ ws) {
+  __shared__ float lk[kBnFlatMaxCh];
+  __shared__ float ls[kBnFlatElems], lq[kBnFlatElems];
+  const FlatTile t = flat_tile(C, HW);
+  const int64_t n0 = (int64_t)blockIdx.y * slab;
+  const int64_t n1 = (n0 + slab < N) ? n0 + slab : N;
+  const int64_t stride4 = C * HW / 4;  // 16-byte vectors per sample
+  const f32x4* p = reinterpret_cast<const f32x4*>(x + t.f0) + threadIdx.x;
+  // A workgroup's lifetime is a chain of memory round trips (every workgroup of the launch is resident
+  // at once), so the first round of loads is on its way before the shifts are worked out, and a round
+  // is up to 16 samples.
+  constexpr int U = kBnFlatInFlight;
+  f32x4 v[U];
+  if (t.valid) {
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (n0 + u < n1) v[u] = p[(n0 + u) * stride4];  // plain loads: the normalising launch reads x again
+  }
+  for (int lc = threadIdx.x; lc < t.nch; lc += kBnBlock) lk[lc] = flat_shift(x, t.c_lo + (uint32_t)lc, N, C, HW);
+  __syncthreads();
+  float k[4], S[4] = {0.f, 0.f, 0.f, 0.f}, Q[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int j = 0; j < 4; ++j) k[j] = lk[t.ch[j]];
+  if (t.valid) {
+    for (int64_t n = n0; n < n1; n += U) {
+      if (n != n0) {
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+          if (n + u < n1) v[u] = p[(n + u) * stride4];
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if (n + u < n1) {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const float d = v[u][j] - k[j];
+            S[j] += d;
+            Q[j] += d * d;
+          }
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    ls[4 * threadIdx.x + j] = S[j];
+    lq[4 * threadIdx.x + j] = Q[j];
+  }
+  __syncthreads();
+  flat_reduce_channels(t, HW, ls, lq, [&](uint32_t c, float a, float b) {
+    unsafeAtomicAdd(ws + c, a);
+    unsafeAtomicAdd(ws + C + c, b);
+  });
+}
+
+// Stand-alone statistics pass on small planes, second launch: one thread per
+// channel does what the last workgroup of a channel does in bn_stats_kernel
+// (the channel's bookkeeping from the two sums), and clears the sums again.
+__global__ __launch_bounds__(kBnBlock) void bn_flat_stats_finish_kernel(const float* __restrict__ x, int64_t N,
+                                                                        int64_t C, int64_t HW, float cnt,
+                                                                        float* __restrict__ ws, float* sum,
+                                                                        float* sum_squares, float* ub_mean,
+                                                                        float* ub_invstd, float eps) {
+  const int64_t c = (int64_t)blockIdx.x * kBnBlock + threadIdx.x;
+  if (c >= C) return;
+  const float k = flat_shift(x, (uint32_t)c, N, C, HW);
+  const float St = ws[c], Qt = ws[C + c];
+  ws[c] = 0.f;
+  ws[C + c] = 0.f;
+  if (sum) sum[c] += fmaf(cnt, k, St);
+  if (sum_squares) sum_squares[c] += fmaf(k, fmaf(cnt, k, 2.f * St), Qt);
+  const float dm = St / cnt;  // mean - k
+  if (ub_mean) ub_mean[c] = k + dm;
+  if (ub_invstd) ub_invstd[c] = 1.f / sqrtf(fmaxf(Qt / cnt - dm * dm, 0.f) + eps);
+}
+
+// y = (x - mu) * a + b with per-element constants; MODE 0: fixed statistics
+// (mean, invstd or var), MODE 1: second launch of the fused training forward
+// (statistics from ws_in; the channel's bookkeeping is done by the workgroup
+// of the first slab whose tile holds the channel's first element).
+template <int MODE>
+__global__ __launch_bounds__(kBnBlock) void bn_flat_apply_kernel(
+    const float* __restrict__ x, float* __restrict__ y, const float* __restrict__ mean,
+    const float* __restrict__ invstd_or_var, const float* __restrict__ gamma, const float* __restrict__ beta,
+    int64_t N, int64_t C, int64_t HW, int64_t slab, int is_var, float cnt, float eps, const float* __restrict__ ws_in,
+    float* __restrict__ ws_clear, float* sum, float* sum_squares, float* ub_mean, float* ub_invstd) {
+  __shared__ float l_mu[kBnFlatMaxCh], l_a[kBnFlatMaxCh], l_b[kBnFlatMaxCh];
+  const FlatTile t = flat_tile(C, HW);
+  for (int lc = threadIdx.x; lc < t.nch; lc += kBnBlock) {
+    const uint32_t c = t.c_lo + (uint32_t)lc;
+    float mu, istd;
+    if (MODE == 0) {
+      mu = mean[c];
+      istd = is_var ? 1.f / sqrtf(invstd_or_var[c] + eps) : invstd_or_var[c];
+    } else {
+      const float k = flat_shift(x, c, N, C, HW);  // the statistics launch took its sums about the same value
+      const float S = ws_in[c], Q = ws_in[C + c];
+      const float dm = S / cnt;  // mean - k
+      mu = k + dm;
+      istd = 1.f / sqrtf(fmaxf(Q / cnt - dm * dm, 0.f) + eps);
+      if (blockIdx.y == 0 && c * (uint32_t)HW >= t.f0) {
+        if (sum) sum[c] += fmaf(cnt, k, S);
+        if (sum_squares) sum_squares[c] += fmaf(k, fmaf(cnt, k, 2.f * S), Q);
+        if (ub_mean) ub_mean[c] = mu;
+        if (ub_invstd) ub_invstd[c] = istd;
+        ws_clear[c] = 0.f;
+        ws_clear[C + c] = 0.f;
+      }
+    }
+    l_mu[lc] = mu;
+    l_a[lc] = gamma ? istd * gamma[c] : istd;
+    l_b[lc] = beta ? beta[c] : 0.f;
+  }
+  __syncthreads();
+  if (!t.valid) return;
+  float mu[4], a[4], b[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    mu[j] = l_mu[t.ch[j]];
+    a[j] = l_a[t.ch[j]];
+    b[j] = l_b[t.ch[j]];
+  }
+  const int64_t n0 = (int64_t)blockIdx.y * slab;
+  const int64_t n1 = (n0 + slab < N) ? n0 + slab : N;
+  const int64_t stride4 = C * HW / 4;
+  const f32x4* p = reinterpret_cast<const f32x4*>(x + t.f0) + threadIdx.x;
+  f32x4* o = reinterpret_cast<f32x4*>(y + t.f0) + threadIdx.x;
+  constexpr int U = kBnFlatInFlight;
+  for (int64_t n = n0; n < n1; n += U) {
+    f32x4 v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (n + u < n1) v[u] = __builtin_nontemporal_load(p + (n + u) * stride4);  // last reader of x in this call
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (n + u < n1) {
+        f32x4 r;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) r[j] = (v[u][j] - mu[j]) * a[j] + b[j];
+        __builtin_nontemporal_store(r, o + (n + u) * stride4);
+      }
+    }
+  }
+}
+
+// Backward on small planes, level 1: per-channel sum(dy) and sum(dy * xhat) into ws.
+__global__ __launch_bounds__(kBnBlock) void bn_flat_bwd_reduce_kernel(const float* __restrict__ x,
+                                                                      const float* __restrict__ dy,
+                                                                      const float* __restrict__ mean,
+                                                                      const float* __restrict__ invstd, int64_t N,
+                                                                      int64_t C, int64_t HW, int64_t slab,
+                                                                      float* __restrict__ ws) {
+  __shared__ float l_mu[kBnFlatMaxCh], l_is[kBnFlatMaxCh];
+  __shared__ float ls[kBnFlatElems], lq[kBnFlatElems];
+  const FlatTile t = flat_tile(C, HW);
+  for (int lc = threadIdx.x; lc < t.nch; lc += kBnBlock) {
+    l_mu[lc] = mean[t.c_lo + (uint32_t)lc];
+    l_is[lc] = invstd[t.c_lo + (uint32_t)lc];
+  }
+  __syncthreads();
+  float mu[4], is[4], A[4] = {0.f, 0.f, 0.f, 0.f}, B[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    mu[j] = l_mu[t.ch[j]];
+    is[j] = l_is[t.ch[j]];
+  }
+  const int64_t n0 = (int64_t)blockIdx.y * slab;
+  const int64_t n1 = (n0 + slab < N) ? n0 + slab : N;
+  const int64_t stride4 = C * HW / 4;
+  const f32x4* px = reinterpret_cast<const f32x4*>(x + t.f0) + threadIdx.x;
+  const f32x4* pg = reinterpret_cast<const f32x4*>(dy + t.f0) + threadIdx.x;
+  constexpr int U = kBnFlatInFlight / 2;
+  if (t.valid) {
+    for (int64_t n = n0; n < n1; n += U) {
+      f32x4 v[U], g[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if (n + u < n1) {
+          v[u] = px[(n + u) * stride4];  // plain loads: the dx launch reads both again
+          g[u] = pg[(n + u) * stride4];
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if (n + u < n1) {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            A[j] += g[u][j];
+            B[j] += g[u][j] * ((v[u][j] - mu[j]) * is[j]);
+          }
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    ls[4 * threadIdx.x + j] = A[j];
+    lq[4 * threadIdx.x + j] = B[j];
+  }
+  __syncthreads();
+  flat_reduce_channels(t, HW, ls, lq, [&](uint32_t c, float a, float b) {
+    unsafeAtomicAdd(ws + c, a);
+    unsafeAtomicAdd(ws + C + c, b);
+  });
+}
+
+// Backward on small planes, level 2: dx, and dbeta / dgamma / the clearing of
+// the other workspace half by the owner of each channel (as in the forward).
+__global__ __launch_bounds__(kBnBlock) void bn_flat_bwd_dx_kernel(
+    const float* __restrict__ x, const float* __restrict__ dy, const float* __restrict__ mean,
+    const float* __restrict__ invstd, const float* __restrict__ gamma, const float* __restrict__ ws_sums,
+    float* __restrict__ ws_clear, float* __restrict__ dgamma, float* __restrict__ dbeta, float* __restrict__ dx,
+    int64_t N, int64_t C, int64_t HW, int64_t slab, float inv_cnt /* 0: fixed statistics */) {
+  __shared__ float l_mu[kBnFlatMaxCh], l_is[kBnFlatMaxCh], l_gi[kBnFlatMaxCh], l_mb[kBnFlatMaxCh], l_mg[kBnFlatMaxCh];
+  const FlatTile t = flat_tile(C, HW);
+  for (int lc = threadIdx.x; lc < t.nch; lc += kBnBlock) {
+    const uint32_t c = t.c_lo + (uint32_t)lc;
+    const float istd = invstd[c];
+    const float sum_dy = ws_sums[c], sum_dyx = ws_sums[C + c];
+    if (blockIdx.y == 0 && c * (uint32_t)HW >= t.f0) {
+      dbeta[c] = sum_dy;
+      dgamma[c] = sum_dyx;
+      ws_clear[c] = 0.f;
+      ws_clear[C + c] = 0.f;
+    }
+    l_mu[lc] = mean[c];
+    l_is[lc] = istd;
+    l_gi[lc] = (gamma ? gamma[c] : 1.f) * istd;
+    l_mb[lc] = sum_dy * inv_cnt;
+    l_mg[lc] = sum_dyx * inv_cnt;
+  }
+  __syncthreads();
+  if (!t.valid) return;
+  float mu[4], is[4], gi[4], mb[4], mg[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    mu[j] = l_mu[t.ch[j]];
+    is[j] = l_is[t.ch[j]];
+    gi[j] = l_gi[t.ch[j]];
+    mb[j] = l_mb[t.ch[j]];
+    mg[j] = l_mg[t.ch[j]];
+  }
+  const int64_t n0 = (int64_t)blockIdx.y * slab;
+  const int64_t n1 = (n0 + slab < N) ? n0 + slab : N;
+  const int64_t stride4 = C * HW / 4;
+  const f32x4* px = reinterpret_cast<const f32x4*>(x + t.f0) + threadIdx.x;
+  const f32x4* pg = reinterpret_cast<const f32x4*>(dy + t.f0) + threadIdx.x;
+  f32x4* pd = reinterpret_cast<f32x4*>(dx + t.f0) + threadIdx.x;
+  constexpr int U = kBnFlatInFlight / 2;
+  for (int64_t n = n0; n < n1; n += U) {
+    f32x4 v[U], g[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (n + u < n1) {
+        v[u] = __builtin_nontemporal_load(px + (n + u) * stride4);  // second and last pass over x and dy
+        g[u] = __builtin_nontemporal_load(pg + (n + u) * stride4);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (n + u < n1) {
+        f32x4 r;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) r[j] = gi[j] * (g[u][j] - mb[j] - ((v[u][j] - mu[j]) * is[j]) * mg[j]);
+        __builtin_nontemporal_store(r, pd + (n + u) * stride4);
+      }
+    }
+  }
+}
+
+// Whether a call takes the flat kernels, and how many samples a workgroup gets.
+inline bool bn_flat_ok(int64_t C, int64_t HW, uintptr_t ptr_bits) {
+  return HW <= kBnFlatMaxHW && (C * HW) % 4 == 0 && (ptr_bits & 15u) == 0;
+}
+
+inline void bn_flat_grid(int64_t N, int64_t C, int64_t HW, dim3* grid, int64_t* slab) {
+  const int64_t tiles = (C * HW + kBnFlatElems - 1) / kBnFlatElems;
+  // About 1024 workgroups, but at most kBnFlatMaxSlabs slabs: every slab's workgroup sends one atomic
+  // add per channel and quantity to the same few addresses, and those are served one after the other
+  // (64 slabs on [256, 512, 7, 7]: 36 us for the statistics, most of it that queue).
+  int64_t slabs = (1024 + tiles - 1) / tiles;
+  // (with only a few tiles the slabs are all the parallelism there is: twice the cap)
+  const int64_t cap = tiles >= 16 ? kBnFlatMaxSlabs : 2 * kBnFlatMaxSlabs;
+  if (slabs > cap) slabs = cap;
+  if (slabs > (N + 3) / 4) slabs = (N + 3) / 4;
+  if (slabs < 1) slabs = 1;
+  const int64_t per = (N + slabs - 1) / slabs;
+  *slab = per;
+  *grid = dim3((unsigned)tiles, (unsigned)((N + per - 1) / per));
+}
+
 // Samples per workgroup: about 8K elements each, so small feature maps do
 // not degenerate into one workgroup per few hundred bytes.
 // Samples per workgroup: about `target` elements.  The fused passes use 8192;
@@ -445,6 +855,19 @@ int ts_bn_stats(const float* x, int64_t N, int64_t C, int64_t HW, float* ws, flo
   if ((uintptr_t)x & 3u) return TS_ERR_ALIGN;
   hipStream_t st = (hipStream_t)stream;
   const float cnt = (float)((double)N * (double)HW);
+  if (ts::bn_flat_ok(C, HW, (uintptr_t)x)) {
+    // small planes: the flat-tile sums, then a launch of one thread per channel (two short launches
+    // instead of the one below, which would leave most of its lanes idle on such planes)
+    dim3 fgrid;
+    int64_t fslab;
+    ts::bn_flat_grid(N, C, HW, &fgrid, &fslab);
+    hipLaunchKernelGGL(ts::bn_flat_stats_kernel, fgrid, dim3(ts::kBnBlock), 0, st, x, N, C, HW, fslab, ws);
+    rc = ts::check_launch();
+    if (rc) return rc;
+    hipLaunchKernelGGL(ts::bn_flat_stats_finish_kernel, dim3((unsigned)((C + ts::kBnBlock - 1) / ts::kBnBlock)),
+                       dim3(ts::kBnBlock), 0, st, x, N, C, HW, cnt, ws, sum, sum_squares, ub_mean, ub_invstd, eps);
+    return ts::check_launch();
+  }
   const int64_t slab = ts::bn_slab(N, HW, 16384);
   dim3 grid((unsigned)((N + slab - 1) / slab), (unsigned)C);
   hipLaunchKernelGGL(ts::bn_stats_kernel<true>, grid, dim3(ts::kBnBlock), 0, st, x, N, C, HW, slab,
@@ -471,6 +894,15 @@ int ts_bn_apply(const float* x, float* y, const float* mean, const float* invstd
   int rc = ts::bn_check_dims(N, C, HW);
   if (rc) return rc;
   if (((uintptr_t)x | (uintptr_t)y) & 3u) return TS_ERR_ALIGN;
+  if (ts::bn_flat_ok(C, HW, (uintptr_t)x | (uintptr_t)y)) {
+    dim3 fgrid;
+    int64_t fslab;
+    ts::bn_flat_grid(N, C, HW, &fgrid, &fslab);
+    hipLaunchKernelGGL(ts::bn_flat_apply_kernel<0>, fgrid, dim3(ts::kBnBlock), 0, (hipStream_t)stream, x, y, mean,
+                       invstd_or_var, gamma, beta, N, C, HW, fslab, is_var, 0.f, eps, (const float*)nullptr,
+                       (float*)nullptr, (float*)nullptr, (float*)nullptr, (float*)nullptr, (float*)nullptr);
+    return ts::check_launch();
+  }
   const int64_t slab = ts::bn_slab(N, HW);
   dim3 grid((unsigned)((N + slab - 1) / slab), (unsigned)C);
   hipLaunchKernelGGL(ts::bn_apply_kernel, grid, dim3(ts::kBnBlock), 0, (hipStream_t)stream, x, y, mean,
@@ -490,6 +922,18 @@ int ts_bn_forward_train(const float* x, float* y, const float* gamma, const floa
   hipStream_t st = (hipStream_t)stream;
   float* ws_now = ws + (int64_t)parity * 2 * C;
   float* ws_other = ws + (int64_t)(1 - parity) * 2 * C;
+  if (ts::bn_flat_ok(C, HW, (uintptr_t)x | (uintptr_t)y)) {
+    dim3 fgrid;
+    int64_t fslab;
+    ts::bn_flat_grid(N, C, HW, &fgrid, &fslab);
+    hipLaunchKernelGGL(ts::bn_flat_stats_kernel, fgrid, dim3(ts::kBnBlock), 0, st, x, N, C, HW, fslab, ws_now);
+    rc = ts::check_launch();
+    if (rc) return rc;
+    hipLaunchKernelGGL(ts::bn_flat_apply_kernel<1>, fgrid, dim3(ts::kBnBlock), 0, st, x, y, (const float*)nullptr,
+                       (const float*)nullptr, gamma, beta, N, C, HW, fslab, 0, (float)((double)N * (double)HW), eps,
+                       (const float*)ws_now, ws_other, sum, sum_squares, ub_mean, ub_invstd);
+    return ts::check_launch();
+  }
   hipLaunchKernelGGL(ts::bn_stats_kernel<false>, grid, dim3(ts::kBnBlock), 0, st, x, N, C, HW, slab, 0.f, ws_now,
                      (float*)nullptr, (float*)nullptr, (float*)nullptr, (float*)nullptr, 0.f);
   rc = ts::check_launch();
@@ -512,6 +956,19 @@ int ts_bn_backward(const float* x, const float* dy, const float* ub_mean, const 
   hipStream_t st = (hipStream_t)stream;
   float* ws_now = ws + (int64_t)parity * 2 * C;
   float* ws_other = ws + (int64_t)(1 - parity) * 2 * C;
+  if (ts::bn_flat_ok(C, HW, (uintptr_t)x | (uintptr_t)dy | (uintptr_t)dx)) {
+    dim3 fgrid;
+    int64_t fslab;
+    ts::bn_flat_grid(N, C, HW, &fgrid, &fslab);
+    hipLaunchKernelGGL(ts::bn_flat_bwd_reduce_kernel, fgrid, dim3(ts::kBnBlock), 0, st, x, dy, ub_mean, ub_invstd, N, C,
+                       HW, fslab, ws_now);
+    rc = ts::check_launch();
+    if (rc) return rc;
+    hipLaunchKernelGGL(ts::bn_flat_bwd_dx_kernel, fgrid, dim3(ts::kBnBlock), 0, st, x, dy, ub_mean, ub_invstd, gamma,
+                       (const float*)ws_now, ws_other, dgamma, dbeta, dx, N, C, HW, fslab,
+                       training ? (float)(1.0 / ((double)N * (double)HW)) : 0.f);
+    return ts::check_launch();
+  }
   hipLaunchKernelGGL(ts::bn_bwd_reduce_kernel, grid, dim3(ts::kBnBlock), 0, st, x, dy, ub_mean, ub_invstd,
                      N, C, HW, slab, ws_now);
   rc = ts::check_launch();
