@@ -191,5 +191,14 @@ def time_next_launch(device):
 
 
 def current_stream_ptr(device) -> int:
+    """Raw handle of torch's current stream on `device` (a torch.device or an
+    index).  Through torch's C binding where it has one: building a Stream
+    object costs the adapters more host time than some of the kernels take."""
     import torch
+    raw = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+    if raw is not None:
+        index = device if isinstance(device, int) else device.index
+        if index is None:
+            index = torch.cuda.current_device()
+        return raw(index)
     return torch.cuda.current_stream(device).cuda_stream

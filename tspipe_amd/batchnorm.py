@@ -36,6 +36,42 @@ def _ptr(t: Optional[Tensor]) -> Optional[int]:
     return None if t is None else t.data_ptr()
 
 
+class _on_device:
+    """``with torch.cuda.device(dev)`` only when `dev` is not already the
+    current device: the context manager costs a training forward on a small
+    feature map about as much host time as the rest of the call."""
+
+    __slots__ = ("ctx",)
+
+    def __init__(self, dev: torch.device):
+        self.ctx = None if dev.index == torch.cuda.current_device() else torch.cuda.device(dev)
+
+    def __enter__(self):
+        if self.ctx is not None:
+            self.ctx.__enter__()
+
+    def __exit__(self, *exc):
+        if self.ctx is not None:
+            return self.ctx.__exit__(*exc)
+        return False
+
+
+class _LayerState:
+    """Per-layer bookkeeping that changes on every call, kept off the module
+    object itself: ``nn.Module.__setattr__`` is a slow path (several
+    ``isinstance`` checks per assignment), and a forward used to take it four
+    times."""
+
+    __slots__ = ("counter", "tracked", "chunks", "parity", "ws_stream")
+
+    def __init__(self, chunks: int):
+        self.counter = 0
+        self.tracked = 0
+        self.chunks = chunks
+        self.parity = 0
+        self.ws_stream = None  # raw handle of the stream whose kernels last used the workspace
+
+
 def _dims(x: Tensor):
     n, c = int(x.shape[0]), int(x.shape[1])
     hw = x.numel() // (n * c) if n * c else 0
@@ -60,7 +96,7 @@ class _NormalizeFn(torch.autograd.Function):
     def forward(ctx, x, weight, bias, mean, spread, layer: "DeferredBatchNorm", training: bool, eps: float):
         n, c, hw = _dims(x)
         y = torch.empty_like(x)
-        with torch.cuda.device(x.device):
+        with _on_device(x.device):
             status = _lib.lib().ts_bn_apply(x.data_ptr(), y.data_ptr(), mean.data_ptr(), spread.data_ptr(),
                                             _ptr(weight), _ptr(bias), n, c, hw, 0 if training else 1, eps,
                                             _lib.current_stream_ptr(x.device))
@@ -79,12 +115,12 @@ class _NormalizeFn(torch.autograd.Function):
         n, c, hw = _dims(x)
         dy = dy.contiguous()
         dx = torch.empty_like(x)
-        dgamma = torch.empty(c, dtype=torch.float32, device=x.device)
-        dbeta = torch.empty(c, dtype=torch.float32, device=x.device)
+        dgb = torch.empty((2, c), dtype=torch.float32, device=x.device)
+        dgamma, dbeta = dgb[0], dgb[1]
         layer = ctx.layer
         ws = layer._workspace(x)
-        parity = layer._parity  # shared with the training forward: the calls of a layer alternate
-        with torch.cuda.device(x.device):
+        parity = layer._st.parity  # shared with the training forward: the calls of a layer alternate
+        with _on_device(x.device):
             status = _lib.lib().ts_bn_backward(x.data_ptr(), dy.data_ptr(), mean.data_ptr(), invstd.data_ptr(),
                                                _ptr(weight), dx.data_ptr(), dgamma.data_ptr(), dbeta.data_ptr(),
                                                ws.data_ptr() + 12 * c, parity, n, c, hw, 1 if ctx.training else 0,
@@ -103,11 +139,11 @@ class _TrainForwardFn(torch.autograd.Function):
     def forward(ctx, x, weight, bias, layer: "DeferredBatchNorm"):
         n, c, hw = _dims(x)
         y = torch.empty_like(x)
-        mean = torch.empty(c, dtype=torch.float32, device=x.device)
-        invstd = torch.empty(c, dtype=torch.float32, device=x.device)
+        stats = torch.empty((2, c), dtype=torch.float32, device=x.device)
+        mean, invstd = stats[0], stats[1]
         ws = layer._workspace(x)
-        parity = layer._parity
-        with torch.cuda.device(x.device):
+        parity = layer._st.parity
+        with _on_device(x.device):
             status = _lib.lib().ts_bn_forward_train(
                 x.data_ptr(), y.data_ptr(), _ptr(weight), _ptr(bias), n, c, hw, layer.sum.data_ptr(),
                 layer.sum_squares.data_ptr(), mean.data_ptr(), invstd.data_ptr(), ws.data_ptr() + 12 * c, parity,
@@ -143,11 +179,13 @@ class DeferredBatchNorm(_BatchNorm):
         # the training forward and the backward alternate between
         # (``_parity`` says which one the next call reduces into)
         self.register_buffer("_ws", torch.zeros(7 * num_features), persistent=False)
-        self._parity = 0
-        self._ws_stream = None  # the stream whose kernels last used the workspace
-        self.counter = 0
-        self.tracked = 0
-        self.chunks = chunks
+        object.__setattr__(self, "_st", _LayerState(chunks))
+
+    # the reference's public counters (tspipe/batchnorm.py:36-38), kept in the state object
+    counter = property(lambda self: self._st.counter, lambda self, v: setattr(self._st, "counter", v))
+    tracked = property(lambda self: self._st.tracked, lambda self, v: setattr(self._st, "tracked", v))
+    chunks = property(lambda self: self._st.chunks, lambda self, v: setattr(self._st, "chunks", v))
+    _parity = property(lambda self: self._st.parity, lambda self, v: setattr(self._st, "parity", v))
 
     def _check_input_dim(self, input: Tensor) -> None:
         if input.dim() <= 2:
@@ -159,10 +197,18 @@ class DeferredBatchNorm(_BatchNorm):
         with ``.half()`` / ``.double()`` or left on another device is refused
         here, as ``F.batch_norm`` refuses mixed types, instead of letting a
         kernel write 4-byte values into narrower buffers."""
-        state = [("sum", self.sum), ("sum_squares", self.sum_squares), ("running_mean", self.running_mean),
-                 ("running_var", self.running_var)]
-        if self.affine:
-            state += [("weight", self.weight), ("bias", self.bias)]
+        dev, f32 = x.device, torch.float32
+        bufs, params = self._buffers, self._parameters
+        a, b, c, d = bufs["sum"], bufs["sum_squares"], bufs["running_mean"], bufs["running_var"]
+        w, bias = params.get("weight"), params.get("bias")
+        ok = (a.dtype is f32 and b.dtype is f32 and c.dtype is f32 and d.dtype is f32 and a.device == dev
+              and b.device == dev and c.device == dev and d.device == dev
+              and (w is None or (w.dtype is f32 and w.device == dev))
+              and (bias is None or (bias.dtype is f32 and bias.device == dev)))
+        nbt = bufs.get("num_batches_tracked")
+        if ok and (nbt is None or (nbt.dtype is torch.int64 and nbt.device == dev)):
+            return
+        state = [("sum", a), ("sum_squares", b), ("running_mean", c), ("running_var", d), ("weight", w), ("bias", bias)]
         for name, t in state:
             if t is None:
                 continue
@@ -170,25 +216,25 @@ class DeferredBatchNorm(_BatchNorm):
                 raise TypeError(f"DeferredBatchNorm kernels are fp32: {name} is {t.dtype} (input {x.dtype})")
             if t.device != x.device:
                 raise TypeError(f"DeferredBatchNorm: {name} is on {t.device}, the input on {x.device}")
-        nbt = self.num_batches_tracked
-        if nbt is not None and (nbt.dtype != torch.int64 or nbt.device != x.device):
-            raise TypeError(f"DeferredBatchNorm: num_batches_tracked must be int64 on {x.device}")
+        raise TypeError(f"DeferredBatchNorm: num_batches_tracked must be int64 on {x.device}")
 
     def _workspace(self, x: Tensor) -> Tensor:
         """The layer's reduction workspace, on x's device.  Its alternating
         halves assume that the layer's calls run one after the other on the
         device, so a call on a stream other than the previous call's first
         waits for that stream."""
-        if self._ws.device != x.device or self._ws.numel() != 7 * self.num_features or self._ws.dtype != torch.float32:
+        st = self._st
+        ws = self._buffers["_ws"]
+        if ws.device != x.device or ws.numel() != 7 * self.num_features or ws.dtype is not torch.float32:
             # moved, resized, or cast along with the module (module.half()): start from zeros
-            self._ws = torch.zeros(7 * self.num_features, dtype=torch.float32, device=x.device)
-            self._parity = 0
-            self._ws_stream = None
-        stream = torch.cuda.current_stream(x.device)
-        if self._ws_stream is not None and self._ws_stream != stream:
-            stream.wait_stream(self._ws_stream)
-        self._ws_stream = stream
-        return self._ws
+            ws = self._ws = torch.zeros(7 * self.num_features, dtype=torch.float32, device=x.device)
+            st.parity = 0
+            st.ws_stream = None
+        stream = _lib.current_stream_ptr(x.device)
+        if st.ws_stream is not None and st.ws_stream != stream:
+            torch.cuda.current_stream(x.device).wait_stream(torch.cuda.ExternalStream(st.ws_stream, device=x.device))
+        st.ws_stream = stream
+        return ws
 
     def _after_launch(self, status: int, parity: int, what: str) -> None:
         """The half the next call reduces into alternates only once this call
@@ -196,16 +242,16 @@ class DeferredBatchNorm(_BatchNorm):
         its launches, so the workspace starts again from zeros."""
         if status < 0:
             self._ws = torch.zeros(7 * self.num_features, dtype=torch.float32, device=self._ws.device)
-            self._parity = 0
+            self._st.parity = 0
             _lib.check(status, what)
-        self._parity = 1 - parity
+        self._st.parity = 1 - parity
 
     def _stats(self, x: Tensor, accumulate: bool):
         """One pass over x: micro-batch mean / invstd, optionally ``sum += ...``."""
         n, c, hw = _dims(x)
         mean = torch.empty(c, dtype=torch.float32, device=x.device)
         invstd = torch.empty(c, dtype=torch.float32, device=x.device)
-        with torch.cuda.device(x.device):
+        with _on_device(x.device):
             status = _lib.lib().ts_bn_stats(
                 x.data_ptr(), n, c, hw, self._workspace(x).data_ptr(),
                 self.sum.data_ptr() if accumulate else None,
@@ -222,9 +268,10 @@ class DeferredBatchNorm(_BatchNorm):
         self._require_state(x)
         x = x if x.is_contiguous() else x.contiguous()
         self._last_stats = self._stats(x, accumulate=True)
-        self.counter += input.size().numel() // input.size(1)
-        self.tracked += 1
-        return self.tracked == self.chunks
+        st = self._st
+        st.counter += input.numel() // input.size(1)
+        st.tracked += 1
+        return st.tracked == st.chunks
 
     def _commit(self) -> None:
         """Folds the accumulated sums into the running statistics
@@ -233,15 +280,15 @@ class DeferredBatchNorm(_BatchNorm):
         if not self.sum.is_cuda:
             raise TypeError("DeferredBatchNorm kernels need device buffers (no host fallback)")
         self._require_state(self.sum)
-        with torch.cuda.device(dev):
+        with _on_device(dev):
             status = _lib.lib().ts_bn_commit(
                 self.sum.data_ptr(), self.sum_squares.data_ptr(), self.running_mean.data_ptr(),
                 self.running_var.data_ptr(), self.num_batches_tracked.data_ptr(), self.num_features,
                 float(self.counter), -1.0 if self.momentum is None else float(self.momentum),
                 _lib.current_stream_ptr(dev))
         _lib.check(status, "ts_bn_commit")
-        self.counter = 0
-        self.tracked = 0
+        self._st.counter = 0
+        self._st.tracked = 0
 
     def forward(self, input: Tensor) -> Tensor:  # type: ignore[override]
         self._check_input_dim(input)
@@ -262,9 +309,10 @@ class DeferredBatchNorm(_BatchNorm):
         # (tspipe/batchnorm.py:45-59) and its normalisation (111-120), fused;
         # the commit (61-85) follows once ``chunks`` micro-batches are in
         y = _TrainForwardFn.apply(x, weight, bias, self)
-        self.counter += input.size().numel() // input.size(1)
-        self.tracked += 1
-        if self.tracked == self.chunks:
+        st = self._st
+        st.counter += input.numel() // input.size(1)
+        st.tracked += 1
+        if st.tracked == st.chunks:
             self._commit()
         return y
 
