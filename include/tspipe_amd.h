@@ -151,6 +151,16 @@ int64_t ts_copy_plan(const void* const* src, void* const* dst, const int64_t* by
 int ts_copy_segments(const ts_copy_chunk* table_dev, int64_t n_chunks, int64_t chunk_bytes,
                      ts_stream_t stream);
 
+/* The same copy for up to 16 segments without a table: src, dst, bytes are
+ * HOST arrays of n_segments entries (device pointers, byte counts; zero-length
+ * segments are skipped) that travel in the kernel's arguments, so nothing is
+ * planned or uploaded first.  For the small gathers of a pipeline -- the
+ * torch.cat of a few micro-batch outputs of some kilobytes each,
+ * tspipe/batch_ops.py:192,198 -- where the table's upload costs more than the
+ * copy.  More than 16 segments: TS_ERR_RANGE (use the table). */
+int ts_copy_few(const void* const* src, void* const* dst, const int64_t* bytes, int n_segments,
+                ts_stream_t stream);
+
 /* ------------------------------------------------------------------------ */
 /* KD soft-target loss, forward and backward in one pass over rows.   */
 /*                                                                          */

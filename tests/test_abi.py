@@ -171,6 +171,13 @@ def test_device_entry_points_validate_before_launching():
     assert lib.ts_ema_multi(p, 1, 1024 * (1 << 24), 0.9, 0.1, None) == -5
     assert lib.ts_copy_segments(p, 1 << 25, 4096, None) == -5
     assert lib.ts_copy_segments(None, 3, 16384, None) == -1
+    import ctypes
+    three = (ctypes.c_void_p * 3)(p, p, p)
+    assert lib.ts_copy_few(three, three, (ctypes.c_int64 * 3)(1, 2, 3), 17, None) == -5   # the table form takes more
+    assert lib.ts_copy_few(None, three, (ctypes.c_int64 * 3)(1, 2, 3), 3, None) == -1
+    assert lib.ts_copy_few(three, three, (ctypes.c_int64 * 3)(1, -2, 3), 3, None) == -1
+    assert lib.ts_copy_few(three, three, (ctypes.c_int64 * 3)(0, 0, 0), 3, None) == 0        # nothing to copy
+    assert lib.ts_copy_few(None, None, None, 0, None) == 0
     assert lib.ts_copy_segments(p, 0, 16384, None) == 0
     assert lib.ts_kd_fwd_bwd(None, p, None, 4, 10, 10, 10, 1.0, 1.0, p, p, None, 10, 0, None) == -1
     assert lib.ts_kd_fwd_bwd(p, p, None, 4, 10, 9, 10, 1.0, 1.0, p, p, None, 10, 0, None) == -1   # ld < V

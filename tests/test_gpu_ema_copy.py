@@ -166,6 +166,22 @@ def test_gather_tuple_and_unaligned_segments(device):
     assert bits_equal(ta.gather([ta.Batch(p) for p in parts]), torch.cat([p.cpu() for p in parts]))
 
 
+@pytest.mark.parametrize("n_pieces", [2, 16, 17, 40])
+def test_gather_of_few_and_of_many_small_pieces(device, n_pieces):
+    # up to 16 small segments travel in the kernel's own arguments, more (or longer ones) through a
+    # planned table: same bytes either way, with ragged row counts, an empty piece, byte-sized elements
+    # and pieces that start off a 16-byte boundary
+    g = seeded(700 + n_pieces)
+    for dtype, width in ((torch.float32, 33), (torch.uint8, 7), (torch.bfloat16, 129)):
+        pieces = []
+        for i in range(n_pieces):
+            rows = 0 if i == 1 else 1 + (i * 5) % 9
+            base = (torch.randn(rows * width + 3, generator=g) * 50).to(dtype).to(device)
+            pieces.append(base[3:].view(rows, width) if i % 3 == 2 else base[:rows * width].view(rows, width))
+        got = ta.gather([ta.Batch(p) for p in pieces])
+        assert torch.equal(got, torch.cat(pieces))
+
+
 def test_gather_autograd_routes_gradients(device):
     g = seeded(24)
     leaves = [torch.randn(r, 4, generator=g).to(device).requires_grad_() for r in (2, 3, 1)]

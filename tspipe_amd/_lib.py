@@ -63,6 +63,7 @@ SIGNATURES = {
     "ts_byol_pieces_fwd_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                                        c_int64, c_void_p, c_void_p, c_int, c_void_p]),
     "ts_infonce_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int]),
+    "ts_copy_few": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
     "ts_infonce_set_workgroup_target": (c_int, [c_int]),
     "ts_infonce_set_fp32_arithmetic": (c_int, [c_int]),
     "ts_infonce_fwd_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_float,

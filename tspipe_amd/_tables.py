@@ -7,6 +7,7 @@ A small ring of (pinned, device) buffer pairs per thread and device lets the
 host run ahead of the GPU: a pair is reused only after the launch that last
 read it has finished.
 """
+import ctypes
 import threading
 from collections import OrderedDict
 from typing import List, Sequence
@@ -199,13 +200,33 @@ def stage_copy(src_ptrs: np.ndarray, dst_ptrs: np.ndarray, nbytes_arr: np.ndarra
     return StagedTable(slot, count, chunk_bytes, device)
 
 
+FEW_SEGMENTS = 16            # what ts_copy_few takes
+FEW_MAX_BYTES = 16 << 20     # longer segments go through the planned table (balanced chunks)
+
+
 def copy_segments(srcs: Sequence[torch.Tensor], dsts: Sequence[torch.Tensor]) -> None:
     """dsts[i] <- srcs[i] (contiguous device tensors of equal byte size), one launch."""
     if not srcs:
         return
-    device = dsts[0].device
-    nbytes = np.fromiter((s.numel() * s.element_size() for s in srcs), dtype=np.int64, count=len(srcs))
-    table = stage_copy(ptr_array(srcs), ptr_array(dsts), nbytes, device)
+    copy_segments_raw([s.data_ptr() for s in srcs], [d.data_ptr() for d in dsts],
+                      [s.numel() * s.element_size() for s in srcs], dsts[0].device)
+
+
+def copy_segments_raw(src_ptrs: Sequence[int], dst_ptrs: Sequence[int], sizes: Sequence[int],
+                      device: torch.device) -> None:
+    """The same on device addresses and byte counts (the caller keeps the
+    tensors alive until the launch is enqueued)."""
+    n = len(src_ptrs)
+    if n == 0:
+        return
+    if n <= FEW_SEGMENTS and kernel_events is None and max(sizes) <= FEW_MAX_BYTES:
+        # a handful of small segments: described in the launch's own arguments, nothing planned or uploaded
+        _lib.check(_lib.lib().ts_copy_few((ctypes.c_void_p * n)(*src_ptrs), (ctypes.c_void_p * n)(*dst_ptrs),
+                                          (ctypes.c_int64 * n)(*sizes), n, _lib.current_stream_ptr(device)),
+                   "ts_copy_few")
+        return
+    nbytes = np.asarray(sizes, dtype=np.int64)
+    table = stage_copy(np.asarray(src_ptrs, dtype=np.uint64), np.asarray(dst_ptrs, dtype=np.uint64), nbytes, device)
     timed = kernel_events is not None
     if timed:
         start, end = _lib.time_next_launch(device)

@@ -121,8 +121,9 @@ def check(input: Any) -> None:
 # dim-0 concatenation on the device: one launch for any number of outputs
 # ---------------------------------------------------------------------------
 
-def _cat_plan(pieces: Sequence[Tensor]) -> Tuple[Tensor, List[Tensor], List[Tensor]]:
-    """Allocates the result of concatenating ``pieces`` and lists (src, dst-view) pairs."""
+def _cat_plan(pieces: Sequence[Tensor]) -> Tuple[Tensor, List[Tensor], List[int], List[int]]:
+    """Allocates the result of concatenating ``pieces``; lists the source
+    tensors, their destination addresses inside the result and byte counts."""
     first = pieces[0]
     if any(not torch.is_tensor(p) for p in pieces):
         raise TypeError("gather expects tensors")
@@ -138,13 +139,18 @@ def _cat_plan(pieces: Sequence[Tensor]) -> Tuple[Tensor, List[Tensor], List[Tens
                 f"(got {tuple(p.shape)} {p.dtype} vs {tuple(first.shape)} {first.dtype})")
     rows = [int(p.shape[0]) for p in pieces]
     out = torch.empty((sum(rows),) + tuple(tail), dtype=first.dtype, device=first.device)
-    srcs, dsts, r0 = [], [], 0
+    # destination addresses by arithmetic: a view of `out` per piece costs more host time than the
+    # copy of a small piece takes
+    row_bytes = (out.numel() // out.shape[0] if out.shape[0] else 0) * out.element_size()
+    base = out.data_ptr()
+    srcs, dsts, sizes, r0 = [], [], [], 0
     for p, r in zip(pieces, rows):
         if r:
-            srcs.append(p.detach() if p.is_contiguous() else p.detach().contiguous())
-            dsts.append(out[r0:r0 + r])
+            srcs.append(p if p.is_contiguous() else p.detach().contiguous())
+            dsts.append(base + r0 * row_bytes)
+            sizes.append(r * row_bytes)
         r0 += r
-    return out, srcs, dsts
+    return out, srcs, dsts, sizes
 
 
 class _CatMany(torch.autograd.Function):
@@ -154,18 +160,24 @@ class _CatMany(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, group_sizes: Tuple[int, ...], *pieces: Tensor):
-        outs, srcs, dsts, rows = [], [], [], []
+        outs, srcs, dsts, sizes, rows = [], [], [], [], []
         i = 0
         for g in group_sizes:
             group = pieces[i:i + g]
             i += g
-            out, s, d = _cat_plan(group)
+            out, s, d, b = _cat_plan(group)
             outs.append(out)
             srcs += s
             dsts += d
+            sizes += b
             rows.append([int(p.shape[0]) for p in group])
-        with torch.cuda.device(outs[0].device):
-            _tables.copy_segments(srcs, dsts)
+        dev = outs[0].device
+        src_ptrs = [t.data_ptr() for t in srcs]  # `srcs` keeps contiguous copies alive until the launch is enqueued
+        if dev.index == torch.cuda.current_device():
+            _tables.copy_segments_raw(src_ptrs, dsts, sizes, dev)
+        else:
+            with torch.cuda.device(dev):
+                _tables.copy_segments_raw(src_ptrs, dsts, sizes, dev)
         ctx.rows = rows
         return tuple(outs)
 
