@@ -16,7 +16,7 @@ from typing import Any, Callable, Iterator, List, Sequence, Tuple, Union
 import torch
 from torch import Tensor
 
-from . import _tables
+from . import _lib, _tables
 from .utils import traverse_tensor_map
 
 Tensors = Union[Tuple[Tensor, ...], dict]
@@ -176,7 +176,7 @@ class _CatMany(torch.autograd.Function):
         if dev.index == torch.cuda.current_device():
             _tables.copy_segments_raw(src_ptrs, dsts, sizes, dev)
         else:
-            with torch.cuda.device(dev):
+            with _lib.on_device(dev):
                 _tables.copy_segments_raw(src_ptrs, dsts, sizes, dev)
         ctx.rows = rows
         return tuple(outs)
@@ -230,7 +230,7 @@ def scatter_copy(input: TensorOrTensors, chunks: int) -> List[Batch]:
     dsts = [torch.empty_like(t, memory_format=torch.contiguous_format) for t in srcs]
     live = [(s.detach() if s.is_contiguous() else s.detach().contiguous(), d)
             for s, d in zip(srcs, dsts) if s.numel()]
-    with torch.cuda.device(srcs[0].device):
+    with _lib.on_device(srcs[0].device):
         _tables.copy_segments([s for s, _ in live], [d for _, d in live])
     it = iter(dsts)
     return [Batch(next(it)) if b.atomic else Batch(tuple(next(it) for _ in b)) for b in views]

@@ -36,26 +36,6 @@ def _ptr(t: Optional[Tensor]) -> Optional[int]:
     return None if t is None else t.data_ptr()
 
 
-class _on_device:
-    """``with torch.cuda.device(dev)`` only when `dev` is not already the
-    current device: the context manager costs a training forward on a small
-    feature map about as much host time as the rest of the call."""
-
-    __slots__ = ("ctx",)
-
-    def __init__(self, dev: torch.device):
-        self.ctx = None if dev.index == torch.cuda.current_device() else torch.cuda.device(dev)
-
-    def __enter__(self):
-        if self.ctx is not None:
-            self.ctx.__enter__()
-
-    def __exit__(self, *exc):
-        if self.ctx is not None:
-            return self.ctx.__exit__(*exc)
-        return False
-
-
 class _LayerState:
     """Per-layer bookkeeping that changes on every call, kept off the module
     object itself: ``nn.Module.__setattr__`` is a slow path (several
@@ -96,7 +76,7 @@ class _NormalizeFn(torch.autograd.Function):
     def forward(ctx, x, weight, bias, mean, spread, layer: "DeferredBatchNorm", training: bool, eps: float):
         n, c, hw = _dims(x)
         y = torch.empty_like(x)
-        with _on_device(x.device):
+        with _lib.on_device(x.device):
             status = _lib.lib().ts_bn_apply(x.data_ptr(), y.data_ptr(), mean.data_ptr(), spread.data_ptr(),
                                             _ptr(weight), _ptr(bias), n, c, hw, 0 if training else 1, eps,
                                             _lib.current_stream_ptr(x.device))
@@ -120,7 +100,7 @@ class _NormalizeFn(torch.autograd.Function):
         layer = ctx.layer
         ws = layer._workspace(x)
         parity = layer._st.parity  # shared with the training forward: the calls of a layer alternate
-        with _on_device(x.device):
+        with _lib.on_device(x.device):
             status = _lib.lib().ts_bn_backward(x.data_ptr(), dy.data_ptr(), mean.data_ptr(), invstd.data_ptr(),
                                                _ptr(weight), dx.data_ptr(), dgamma.data_ptr(), dbeta.data_ptr(),
                                                ws.data_ptr() + 12 * c, parity, n, c, hw, 1 if ctx.training else 0,
@@ -143,7 +123,7 @@ class _TrainForwardFn(torch.autograd.Function):
         mean, invstd = stats[0], stats[1]
         ws = layer._workspace(x)
         parity = layer._st.parity
-        with _on_device(x.device):
+        with _lib.on_device(x.device):
             status = _lib.lib().ts_bn_forward_train(
                 x.data_ptr(), y.data_ptr(), _ptr(weight), _ptr(bias), n, c, hw, layer.sum.data_ptr(),
                 layer.sum_squares.data_ptr(), mean.data_ptr(), invstd.data_ptr(), ws.data_ptr() + 12 * c, parity,
@@ -251,7 +231,7 @@ class DeferredBatchNorm(_BatchNorm):
         n, c, hw = _dims(x)
         mean = torch.empty(c, dtype=torch.float32, device=x.device)
         invstd = torch.empty(c, dtype=torch.float32, device=x.device)
-        with _on_device(x.device):
+        with _lib.on_device(x.device):
             status = _lib.lib().ts_bn_stats(
                 x.data_ptr(), n, c, hw, self._workspace(x).data_ptr(),
                 self.sum.data_ptr() if accumulate else None,
@@ -280,7 +260,7 @@ class DeferredBatchNorm(_BatchNorm):
         if not self.sum.is_cuda:
             raise TypeError("DeferredBatchNorm kernels need device buffers (no host fallback)")
         self._require_state(self.sum)
-        with _on_device(dev):
+        with _lib.on_device(dev):
             status = _lib.lib().ts_bn_commit(
                 self.sum.data_ptr(), self.sum_squares.data_ptr(), self.running_mean.data_ptr(),
                 self.running_var.data_ptr(), self.num_batches_tracked.data_ptr(), self.num_features,

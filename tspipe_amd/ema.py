@@ -78,7 +78,7 @@ def _launch(m: float, students: Sequence[torch.Tensor], teachers: Sequence[torch
             out_ptrs: np.ndarray, numels: np.ndarray) -> None:
     device = teachers[0].device
     code = _DTYPE_CODES[teachers[0].dtype]
-    with torch.cuda.device(device):
+    with _lib.on_device(device):
         table = _tables.stage_ema(_ptrs(teachers), _ptrs(students), out_ptrs, numels, device, dtype=code)
         timed = kernel_events is not None
         if timed:
@@ -131,7 +131,7 @@ def _fast_update(m: float, online, target) -> Optional[List[torch.Tensor]]:
     if arena.numels.size != n or not np.array_equal(arena.numels, nn[:n]):
         return None  # hash collision between different lists: take the exact path
     device = teachers[0].device
-    with torch.cuda.device(device):
+    with _lib.on_device(device):
         table = _tables.stage_ema(tp[:n], sp[:n], arena.ptrs, arena.numels, device)
         timed = kernel_events is not None
         if timed:
@@ -334,7 +334,7 @@ def clone_and_update(m: float, online_param: Iterable[torch.Tensor], target_para
     clone_arena, clone_views = _acquire_arena(teachers, shapes)
     offset = clone_arena.flat.data_ptr() - ema_arena.flat.data_ptr()
     device = teachers[0].device
-    with torch.cuda.device(device):
+    with _lib.on_device(device):
         table = _tables.stage_ema(_ptrs(teachers), _ptrs(students), ema_arena.ptrs, ema_arena.numels, device)
         timed = kernel_events is not None
         if timed:
@@ -387,7 +387,7 @@ def clone_params(params: Iterable[torch.Tensor]) -> List[torch.Tensor]:
         for i, piece in zip(idx, flat.split(padded)):
             outs[i] = piece[:dense[i].numel()].view(dense[i].shape)
     live = [(s, o) for s, o in zip(dense, outs) if s.numel()]
-    with torch.cuda.device(dense[0].device):
+    with _lib.on_device(dense[0].device):
         _tables.copy_segments([s for s, _ in live], [o for _, o in live])
     return outs  # type: ignore[return-value]
 
@@ -403,7 +403,7 @@ def copy_params_(dst_params: Iterable[torch.Tensor], src_params: Iterable[torch.
     live = [(s, d) for s, d in zip(srcs, dsts) if s.numel()]
     if not live:
         return
-    with torch.cuda.device(dsts[0].device):
+    with _lib.on_device(dsts[0].device):
         _tables.copy_segments([s for s, _ in live], [d for _, d in live])
 
 

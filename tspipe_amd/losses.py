@@ -37,7 +37,7 @@ def _scale_saved_grad(grad: Tensor, grad_output: Tensor, rows: int, cols: int) -
     """grad *= grad_output on the device, without a host sync; the kernel
     returns immediately when grad_output is 1."""
     g = grad_output.detach().to(torch.float32).reshape(1)
-    with torch.cuda.device(grad.device):
+    with _lib.on_device(grad.device):
         status = _lib.lib().ts_scale_rows(grad.data_ptr(), rows, cols, cols, g.data_ptr(),
                                           _lib.dtype_code(grad.dtype), _lib.current_stream_ptr(grad.device))
     _lib.check(status, "ts_scale_rows")
@@ -93,7 +93,7 @@ class _KDSoftTargetFn(torch.autograd.Function):
         ws = torch.empty(lib.ts_kd_workspace_bytes(rows, V, code), dtype=torch.uint8, device=dev)
         loss = torch.empty((), dtype=torch.float32, device=dev)
         grad = torch.empty_like(s) if need_grad else None
-        with torch.cuda.device(dev):
+        with _lib.on_device(dev):
             status = lib.ts_kdce_fwd_bwd(s.data_ptr(), t.data_ptr(), mask_ptr, label_ptr, int(ignore_index), rows, V,
                                          V, V, 1.0 / T, T * T * weight, float(ce_weight), ws.data_ptr(),
                                          loss.data_ptr(), None if grad is None else grad.data_ptr(), V, code,
@@ -101,7 +101,7 @@ class _KDSoftTargetFn(torch.autograd.Function):
         _lib.check(status, "ts_kdce_fwd_bwd")
         if mse_weight > 0.0:
             ws2 = torch.empty(lib.ts_mse_workspace_bytes(rows, V), dtype=torch.uint8, device=dev)
-            with torch.cuda.device(dev):
+            with _lib.on_device(dev):
                 status = lib.ts_mse_fwd_bwd(s.data_ptr(), t.data_ptr(), mask_ptr, rows, V, V, V, float(mse_weight),
                                             1 if mse_per_element else 0, 1,
                                             ws2.data_ptr(), loss.data_ptr(), None if grad is None else grad.data_ptr(),
@@ -215,7 +215,7 @@ class _KDPiecesFn(torch.autograd.Function):
         ws = torch.empty(lib.ts_kd_workspace_bytes(total, V, code), dtype=torch.uint8, device=dev)
         loss = torch.empty((), dtype=torch.float32, device=dev)
         ptrs = lambda ts: (ctypes.c_void_p * n)(*[t.data_ptr() for t in ts])
-        with torch.cuda.device(dev):
+        with _lib.on_device(dev):
             status = lib.ts_kdce_pieces_fwd_bwd(ptrs(s_flat), ptrs(t_flat), None if grads is None else ptrs(grads),
                                                 (ctypes.c_int64 * n)(*rows), n, mask_ptr, label_ptr, int(ignore_index),
                                                 V, 1.0 / T, T * T * weight, float(ce_weight), ws.data_ptr(),
@@ -224,7 +224,7 @@ class _KDPiecesFn(torch.autograd.Function):
         if mse_weight > 0.0:
             # the squared-error term joins loss and gradient in place, piece by piece
             ws2 = torch.empty(lib.ts_mse_workspace_bytes(total, V), dtype=torch.uint8, device=dev)
-            with torch.cuda.device(dev):
+            with _lib.on_device(dev):
                 status = lib.ts_mse_pieces_fwd_bwd(ptrs(s_flat), ptrs(t_flat), None if grads is None else ptrs(grads),
                                                    (ctypes.c_int64 * n)(*rows), n, mask_ptr, V, float(mse_weight),
                                                    1 if mse_per_element else 0, 1, ws2.data_ptr(), loss.data_ptr(),
@@ -292,7 +292,7 @@ class _LogitsMSEFn(torch.autograd.Function):
         ws = torch.empty(lib.ts_mse_workspace_bytes(rows, V), dtype=torch.uint8, device=dev)
         loss = torch.empty((), dtype=torch.float32, device=dev)
         grad = torch.empty_like(s) if ctx.needs_input_grad[0] else None
-        with torch.cuda.device(dev):
+        with _lib.on_device(dev):
             status = lib.ts_mse_fwd_bwd(s.data_ptr(), t.data_ptr(), mask_ptr, rows, V, V, V, float(weight),
                                         1 if per_element else 0, 0, ws.data_ptr(), loss.data_ptr(),
                                         None if grad is None else grad.data_ptr(), V, _lib.dtype_code(s.dtype),
@@ -353,7 +353,7 @@ class _CosineFn(torch.autograd.Function):
         ws = torch.empty(lib.ts_cosine_workspace_bytes(n), dtype=torch.uint8, device=dev)
         loss = torch.empty((), dtype=torch.float32, device=dev)
         gx = torch.empty_like(xs) if ctx.needs_input_grad[0] else None
-        with torch.cuda.device(dev):
+        with _lib.on_device(dev):
             status = lib.ts_cosine_fwd_bwd(xs.data_ptr(), ys.data_ptr(), mask_ptr, n, c, weight, ws.data_ptr(),
                                            loss.data_ptr(), None if gx is None else gx.data_ptr(),
                                            _lib.dtype_code(xs.dtype), _lib.current_stream_ptr(dev))
@@ -411,7 +411,7 @@ class _CosinePiecesFn(torch.autograd.Function):
         ws = torch.empty(lib.ts_cosine_workspace_bytes(total), dtype=torch.uint8, device=dev)
         loss = torch.empty((), dtype=torch.float32, device=dev)
         ptrs = lambda ts: (ctypes.c_void_p * n)(*[t.data_ptr() for t in ts])  # noqa: E731
-        with torch.cuda.device(dev):
+        with _lib.on_device(dev):
             status = lib.ts_cosine_pieces_fwd_bwd(ptrs(x_flat), ptrs(y_flat), None if grads is None else ptrs(grads),
                                                   (ctypes.c_int64 * n)(*rows), n, mask_ptr, c, float(weight),
                                                   ws.data_ptr(), loss.data_ptr(), _lib.dtype_code(dtype),
@@ -464,7 +464,7 @@ class _BYOLFn(torch.autograd.Function):
         loss = torch.empty((), dtype=torch.float32, device=dev)
         g1 = torch.empty_like(prep[0]) if ctx.needs_input_grad[0] else None
         g2 = torch.empty_like(prep[2]) if (x2 is not None and ctx.needs_input_grad[2]) else None
-        with torch.cuda.device(dev):
+        with _lib.on_device(dev):
             status = _lib.lib().ts_byol_fwd_bwd(
                 prep[0].data_ptr(), prep[1].data_ptr(),
                 prep[2].data_ptr() if x2 is not None else None,
@@ -537,7 +537,7 @@ class _InfoNCEFn(torch.autograd.Function):
         loss = torch.empty((), dtype=torch.float32, device=dev)
         g1 = torch.empty_like(prep[0]) if ctx.needs_input_grad[0] else None
         g2 = torch.empty_like(prep[2]) if (q2 is not None and ctx.needs_input_grad[2]) else None
-        with torch.cuda.device(dev):
+        with _lib.on_device(dev):
             status = lib.ts_infonce_fwd_bwd(
                 prep[0].data_ptr(), prep[1].data_ptr(),
                 prep[2].data_ptr() if q2 is not None else None,
@@ -645,7 +645,7 @@ class _PairPiecesFn(torch.autograd.Function):
         loss = torch.empty((), dtype=torch.float32, device=dev)
         ptrs = lambda ts: None if ts is None else (ctypes.c_void_p * n)(*[t.data_ptr() for t in ts])  # noqa: E731
         rows_arr = (ctypes.c_int64 * n)(*rows)
-        with torch.cuda.device(dev):
+        with _lib.on_device(dev):
             stream = _lib.current_stream_ptr(dev)
             if kind == "infonce":
                 if c > 512:
