@@ -259,6 +259,53 @@ def test_deferred_bn_module_contract(device):
     assert out.shape == (2, 4, 6, 6)
 
 
+def test_cpp_autograd_node_and_python_function_agree(device, monkeypatch):
+    # the training forward runs from a C++ autograd node when the host helper is built, from a Python
+    # autograd.Function otherwise: same launches, same bits, same bookkeeping, interleaved on one layer
+    from tspipe_amd import _lib
+    from tspipe_amd import batchnorm as bn_mod
+    if _lib.host_helper() is None or not hasattr(_lib.host_helper(), "bn_train"):
+        pytest.skip("host helper not built")
+    g = seeded(610)
+    results = {}
+    for use_node in (True, False):
+        monkeypatch.setattr(bn_mod, "_HOST_NODE", use_node)
+        bn = ta.DeferredBatchNorm(12, chunks=2).to(device)
+        with torch.no_grad():
+            bn.weight.copy_(torch.linspace(0.5, 1.5, 12))
+            bn.bias.copy_(torch.linspace(-0.2, 0.2, 12))
+        outs = []
+        for step in range(5):
+            x = _make((6, 12, 7, 7), 620 + step).to(device).requires_grad_()
+            dy = torch.randn(6, 12, 7, 7, generator=seeded(640 + step)).to(device)
+            y = bn(x)
+            y.backward(dy)
+            outs.append((y.detach().clone(), x.grad.clone(), bn.weight.grad.clone(), bn.bias.grad.clone()))
+        outs.append((bn.running_mean.clone(), bn.running_var.clone(), bn.sum.clone(), bn.sum_squares.clone()))
+        _check_workspace(bn)
+        assert bn.tracked == 1 and int(bn.num_batches_tracked) == 2
+        results[use_node] = outs
+    for a_, b_ in zip(results[True], results[False]):
+        for u, v in zip(a_, b_):
+            assert torch.equal(u, v)
+    # the two paths on ONE layer, alternating: the shared parity keeps the workspace halves in step
+    bn = ta.DeferredBatchNorm(12, chunks=1 << 30).to(device)
+    for step in range(6):
+        monkeypatch.setattr(bn_mod, "_HOST_NODE", step % 2 == 0)
+        x = _make((6, 12, 7, 7), 660 + step).to(device).requires_grad_()
+        y = bn(x)
+        y.backward(torch.ones_like(y))
+        want = F.batch_norm(x.detach().cpu().double(), None, None, bn.weight.detach().cpu().double(),
+                            bn.bias.detach().cpu().double(), True, 0.0, 1e-5)
+        assert (y.detach().cpu().double() - want).abs().max() < 2e-5
+    _check_workspace(bn)
+    import copy
+    twin = copy.deepcopy(bn)
+    assert twin._parity == bn._parity and twin._st.shared.data_ptr() != bn._st.shared.data_ptr()
+    twin._parity = 1 - twin._parity
+    assert twin._st.shared[0].item() == twin._parity != bn._parity
+
+
 def test_fused_training_forward_equals_the_two_calls(device):
     # ts_bn_forward_train against ts_bn_stats + ts_bn_apply through the C ABI: bit for bit,
     # over several calls so that both workspace halves are used and cleared
@@ -295,6 +342,9 @@ def test_fused_training_forward_equals_the_two_calls(device):
 
 def test_a_refused_call_leaves_the_next_forward_correct(device, monkeypatch):
     from tspipe_amd import _lib
+    from tspipe_amd import batchnorm as bn_mod
+    # the Python path is the one whose library handle can be swapped for a refusing one
+    monkeypatch.setattr(bn_mod, "_HOST_NODE", False)
     bn = ta.DeferredBatchNorm(6, chunks=8).to(device)
     xs = [_make((4, 6, 5, 5), 70 + i) for i in range(3)]
     bn(xs[0].to(device))
@@ -308,10 +358,10 @@ def test_a_refused_call_leaves_the_next_forward_correct(device, monkeypatch):
             return -4  # TS_ERR_ALIGN, nothing enqueued
 
     parity = bn._parity
-    monkeypatch.setattr(_lib, "lib", lambda: Refusing())
-    with pytest.raises(_lib.TSPipeAmdError):
-        bn(xs[1].to(device))
-    monkeypatch.undo()
+    with monkeypatch.context() as swapped:
+        swapped.setattr(_lib, "lib", lambda: Refusing())
+        with pytest.raises(_lib.TSPipeAmdError):
+            bn(xs[1].to(device))
     assert bn._parity in (0, parity)  # not advanced by the refused call
     _check_workspace(bn)
     y = bn(xs[2].to(device))

@@ -137,6 +137,8 @@ def host_helper():
                     addr = lambda fn: ctypes.cast(fn, c_void_p).value  # noqa: E731
                     mod.bind_abi(addr(handle.ts_infonce_workspace_bytes), addr(handle.ts_infonce_fwd_bwd),
                                  addr(handle.ts_scale_rows))
+                    if hasattr(mod, "bind_bn"):
+                        mod.bind_bn(addr(handle.ts_bn_forward_train), addr(handle.ts_bn_backward))
                 _host = mod
             _host_tried = True
     return _host

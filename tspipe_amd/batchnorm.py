@@ -21,6 +21,7 @@ and the converter's sharing of parameters and running buffers are unchanged.
 """
 from typing import Optional, TypeVar, cast
 
+import numpy as np
 import torch
 from torch import Tensor, nn
 from torch.nn.modules.batchnorm import _BatchNorm
@@ -28,6 +29,10 @@ from torch.nn.modules.batchnorm import _BatchNorm
 from . import _lib
 
 __all__ = ["DeferredBatchNorm"]
+
+# the C++ autograd node of the optional host helper takes the training forward when it is there
+# (tests switch it off to exercise the Python path)
+_HOST_NODE = True
 
 TModule = TypeVar("TModule", bound=nn.Module)
 
@@ -42,14 +47,50 @@ class _LayerState:
     ``isinstance`` checks per assignment), and a forward used to take it four
     times."""
 
-    __slots__ = ("counter", "tracked", "chunks", "parity", "ws_stream")
+    __slots__ = ("counter", "tracked", "chunks", "_np", "shared")
 
     def __init__(self, chunks: int):
         self.counter = 0
         self.tracked = 0
         self.chunks = chunks
-        self.parity = 0
-        self.ws_stream = None  # raw handle of the stream whose kernels last used the workspace
+        # [0]: which half of the reduction workspace the next call uses; [1]: raw handle of the stream
+        # whose kernels used the workspace last (0: none yet).  One piece of host memory seen as a numpy
+        # array here and as a tensor by the C++ autograd node, which updates it from autograd's thread.
+        self._np = np.zeros(2, dtype=np.int64)
+        self.shared = torch.from_numpy(self._np)
+
+    @property
+    def parity(self) -> int:
+        return int(self._np[0])
+
+    @parity.setter
+    def parity(self, v: int) -> None:
+        self._np[0] = v
+
+    @property
+    def ws_stream(self):
+        v = int(self._np[1])
+        return v if v else None
+
+    @ws_stream.setter
+    def ws_stream(self, v) -> None:
+        self._np[1] = v if v else 0
+
+    def __deepcopy__(self, memo):
+        new = _LayerState(self.chunks)
+        new.counter, new.tracked = self.counter, self.tracked
+        new._np[:] = self._np
+        return new
+
+    def __reduce__(self):
+        return (_restore_state, (self.chunks, self.counter, self.tracked, int(self._np[0])))
+
+
+def _restore_state(chunks, counter, tracked, parity):
+    st = _LayerState(chunks)
+    st.counter, st.tracked = counter, tracked
+    st._np[0] = parity
+    return st
 
 
 def _dims(x: Tensor):
@@ -288,8 +329,23 @@ class DeferredBatchNorm(_BatchNorm):
         # statistics of this micro-batch into the accumulators
         # (tspipe/batchnorm.py:45-59) and its normalisation (111-120), fused;
         # the commit (61-85) follows once ``chunks`` micro-batches are in
-        y = _TrainForwardFn.apply(x, weight, bias, self)
         st = self._st
+        y = None
+        host = _lib.host_helper()
+        if host is not None and _HOST_NODE:
+            # the same two launches and the same backward from a C++ autograd node (no interpreter in
+            # backward); it shares the parity / last-stream words with this object
+            ws = self._workspace(x)
+            try:
+                y = host.bn_train(x, weight, bias, self.sum, self.sum_squares, ws, st.shared, float(self.eps),
+                                  st.ws_stream or 0)
+            except RuntimeError:
+                # a refused call may have run part of its launches: the workspace starts again from zeros
+                self._ws = torch.zeros(7 * self.num_features, dtype=torch.float32, device=ws.device)
+                st.parity = 0
+                raise
+        if y is None:
+            y = _TrainForwardFn.apply(x, weight, bias, self)
         st.counter += input.numel() // input.size(1)
         st.tracked += 1
         if st.tracked == st.chunks:

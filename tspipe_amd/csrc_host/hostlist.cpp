@@ -4,6 +4,7 @@
 // EMA kernel itself; here it is one call.  No GPU work happens in this module.
 #include <torch/extension.h>
 #include <torch/csrc/autograd/python_variable.h>
+#include <ATen/detail/CUDAHooksInterface.h>
 
 #include <cstdint>
 #include <vector>
@@ -189,6 +190,105 @@ py::object infonce(const at::Tensor& q1, const at::Tensor& k1, const c10::option
   return py::cast(loss);
 }
 
+// ---------------------------------------------------------------------------
+// DeferredBatchNorm's training forward as a C++ autograd node, for the same
+// reason: on the feature maps of a network's late stages the kernels take
+// 10-30 us and a Python autograd.Function around them 100.  The layer's
+// state that changes with every launch -- which half of the reduction
+// workspace the next call uses, and the stream that used the workspace last --
+// lives in a two-element int64 host tensor shared with the Python module
+// (state[0] = parity, state[1] = stream handle), so that Python-side calls of
+// the same layer (evaluation mode, the stand-alone statistics) stay in step.
+// ---------------------------------------------------------------------------
+typedef int (*bn_fwd_fn)(const float*, float*, const float*, const float*, int64_t, int64_t, int64_t, float*, float*,
+                         float*, float*, float*, int, float, void*);
+typedef int (*bn_bwd_fn)(const float*, const float*, const float*, const float*, const float*, float*, float*, float*,
+                         float*, int, int64_t, int64_t, int64_t, int, void*);
+static bn_fwd_fn g_bn_fwd = nullptr;
+static bn_bwd_fn g_bn_bwd = nullptr;
+
+void bind_bn(uintptr_t fwd, uintptr_t bwd) {
+  g_bn_fwd = reinterpret_cast<bn_fwd_fn>(fwd);
+  g_bn_bwd = reinterpret_cast<bn_bwd_fn>(bwd);
+}
+
+struct BnTrainNode : public torch::autograd::Function<BnTrainNode> {
+  static at::Tensor forward(torch::autograd::AutogradContext* ctx, const at::Tensor& x,
+                            const c10::optional<at::Tensor>& weight, const c10::optional<at::Tensor>& bias,
+                            const at::Tensor& sum, const at::Tensor& sum_squares, const at::Tensor& ws,
+                            const at::Tensor& state, double eps, int64_t stream) {
+    const int64_t N = x.size(0), C = x.size(1), HW = (N * C) ? x.numel() / (N * C) : 0;
+    c10::DeviceGuard guard(x.device());
+    at::Tensor y = at::empty_like(x);
+    at::Tensor stats = at::empty({2, C}, x.options());  // micro-batch mean, inverse standard deviation
+    int64_t* st = state.data_ptr<int64_t>();
+    const int parity = (int)st[0];
+    const bool has_w = weight.has_value() && weight->defined(), has_b = bias.has_value() && bias->defined();
+    const int rc = g_bn_fwd(x.data_ptr<float>(), y.data_ptr<float>(), has_w ? weight->data_ptr<float>() : nullptr,
+                            has_b ? bias->data_ptr<float>() : nullptr, N, C, HW, sum.data_ptr<float>(),
+                            sum_squares.data_ptr<float>(), stats.data_ptr<float>(), stats.data_ptr<float>() + C,
+                            ws.data_ptr<float>() + 3 * C, parity, (float)eps, reinterpret_cast<void*>(stream));
+    TORCH_CHECK(rc == 0, "ts_bn_forward_train: status ", rc);
+    st[0] = 1 - parity;
+    st[1] = stream;
+    ctx->save_for_backward({x, stats, has_w ? *weight : at::Tensor()});
+    ctx->saved_data["ws"] = ws;
+    ctx->saved_data["state"] = state;
+    ctx->saved_data["stream"] = stream;
+    ctx->saved_data["has_w"] = has_w;
+    ctx->saved_data["has_b"] = has_b;
+    return y;
+  }
+
+  static torch::autograd::variable_list backward(torch::autograd::AutogradContext* ctx,
+                                                 torch::autograd::variable_list grad_out) {
+    const auto saved = ctx->get_saved_variables();
+    const at::Tensor& x = saved[0];
+    const at::Tensor& stats = saved[1];
+    const at::Tensor& weight = saved[2];
+    const bool has_w = ctx->saved_data["has_w"].toBool(), has_b = ctx->saved_data["has_b"].toBool();
+    const int64_t stream = ctx->saved_data["stream"].toInt();
+    at::Tensor ws = ctx->saved_data["ws"].toTensor(), state = ctx->saved_data["state"].toTensor();
+    const int64_t N = x.size(0), C = x.size(1), HW = (N * C) ? x.numel() / (N * C) : 0;
+    c10::DeviceGuard guard(x.device());
+    at::Tensor dy = grad_out[0].contiguous();
+    if (dy.scalar_type() != at::kFloat) dy = dy.to(at::kFloat);
+    at::Tensor dx = at::empty_like(x);
+    at::Tensor dgb = at::empty({2, C}, x.options());
+    int64_t* st = state.data_ptr<int64_t>();
+    if (st[1] != 0 && st[1] != stream) {
+      // the layer's last call ran on another stream: its use of the workspace must be over first
+      // (rare; the Python side orders the two streams with an event instead of this wait)
+      at::detail::getCUDAHooks().deviceSynchronize(x.device().index());
+    }
+    const int parity = (int)st[0];
+    const int rc = g_bn_bwd(x.data_ptr<float>(), dy.data_ptr<float>(), stats.data_ptr<float>(),
+                            stats.data_ptr<float>() + C, weight.defined() ? weight.data_ptr<float>() : nullptr,
+                            dx.data_ptr<float>(), dgb.data_ptr<float>(), dgb.data_ptr<float>() + C,
+                            ws.data_ptr<float>() + 3 * C, parity, N, C, HW, 1, reinterpret_cast<void*>(stream));
+    TORCH_CHECK(rc == 0, "ts_bn_backward: status ", rc);
+    st[0] = 1 - parity;
+    st[1] = stream;
+    return {dx, has_w ? dgb[0] : at::Tensor(), has_b ? dgb[1] : at::Tensor(), at::Tensor(), at::Tensor(),
+            at::Tensor(), at::Tensor(), at::Tensor(), at::Tensor()};
+  }
+};
+
+// Returns None when the call is not of the plain kind (then the Python path
+// takes it): contiguous fp32 device tensors, state on the host.
+py::object bn_train(const at::Tensor& x, const c10::optional<at::Tensor>& weight,
+                    const c10::optional<at::Tensor>& bias, const at::Tensor& sum, const at::Tensor& sum_squares,
+                    const at::Tensor& ws, const at::Tensor& state, double eps, int64_t stream) {
+  if (!g_bn_fwd || !g_bn_bwd) return py::none();
+  if (!x.is_cuda() || x.scalar_type() != at::kFloat || !x.is_contiguous() || x.dim() < 3) return py::none();
+  if (state.is_cuda() || state.scalar_type() != at::kLong || state.numel() != 2 || !state.is_contiguous())
+    return py::none();
+  const int64_t C = x.size(1);
+  if (ws.numel() != 7 * C || ws.scalar_type() != at::kFloat || ws.device() != x.device()) return py::none();
+  at::Tensor y = BnTrainNode::apply(x, weight, bias, sum, sum_squares, ws, state, eps, stream);
+  return py::cast(y);
+}
+
 // Test aid: a C++ owner of a tensor that Python cannot see.  hold() keeps the
 // tensor alive inside this module until drop() is called.
 static std::vector<at::Tensor> g_held;
@@ -203,6 +303,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("all_refcounts_equal", &all_refcounts_equal);
   m.def("bind_abi", &bind_abi);
   m.def("infonce", &infonce);
+  m.def("bind_bn", &bind_bn);
+  m.def("bn_train", &bn_train);
   m.def("hold", &hold);
   m.def("drop", &drop);
 }
