@@ -306,6 +306,45 @@ def test_cpp_autograd_node_and_python_function_agree(device, monkeypatch):
     assert twin._st.shared[0].item() == twin._parity != bn._parity
 
 
+@pytest.mark.parametrize("shape", [(9, 12, 7, 7), (5, 64, 4, 4), (3, 8, 16, 16), (33, 20, 1, 1)])
+def test_small_planes_flat_and_plane_kernels_agree(device, shape):
+    # the same values once on a 16-byte boundary (flat-tile kernels) and once four bytes off it (the
+    # wavefront-per-plane kernels): outputs, statistics and gradients agree to fp32 rounding
+    from tspipe_amd import _lib
+    lib = _lib.lib()
+    st = torch.cuda.current_stream(device).cuda_stream
+    N, C = shape[0], shape[1]
+    HW = shape[2] * shape[3]
+    n = N * C * HW
+    g = seeded(810 + HW)
+    xv = (torch.randn(n, generator=g) * 1.5 + 0.5)
+    dyv = torch.randn(n, generator=g)
+    gamma = (torch.rand(C, generator=g) + 0.5).to(device)
+    beta = (torch.randn(C, generator=g) * 0.1).to(device)
+    outs = []
+    for off in (0, 1):
+        buf = lambda: torch.zeros(n + 4, device=device)  # noqa: E731
+        x, dy, y, dx = buf()[off:off + n], buf()[off:off + n], buf()[off:off + n], buf()[off:off + n]
+        x.copy_(xv)
+        dy.copy_(dyv)
+        assert x.data_ptr() % 16 == 4 * off
+        z = lambda k: torch.zeros(k, device=device)  # noqa: E731
+        acc_s, acc_q, mean, inv, ws, dg, db = z(C), z(C), z(C), z(C), z(4 * C), z(C), z(C)
+        _lib.check(lib.ts_bn_forward_train(x.data_ptr(), y.data_ptr(), gamma.data_ptr(), beta.data_ptr(), N, C, HW,
+                                           acc_s.data_ptr(), acc_q.data_ptr(), mean.data_ptr(), inv.data_ptr(),
+                                           ws.data_ptr(), 0, 1e-5, st), "forward")
+        _lib.check(lib.ts_bn_backward(x.data_ptr(), dy.data_ptr(), mean.data_ptr(), inv.data_ptr(), gamma.data_ptr(),
+                                      dx.data_ptr(), dg.data_ptr(), db.data_ptr(), ws.data_ptr(), 1, N, C, HW, 1, st),
+                   "backward")
+        torch.cuda.synchronize()
+        assert (ws[:2 * C] == 0).all()  # the forward's half, cleared by the backward (whose own half the next call clears)
+        outs.append([t.clone() for t in (y, dx, acc_s, acc_q, mean, inv, dg, db)])
+    names = ("y", "dx", "sum", "sum_squares", "mean", "invstd", "dgamma", "dbeta")
+    for name, a_, b_ in zip(names, *outs):
+        scale = a_.abs().max().item() + 1e-12
+        assert (a_ - b_).abs().max().item() <= 2e-5 * scale + 2e-6, name
+
+
 def test_fused_training_forward_equals_the_two_calls(device):
     # ts_bn_forward_train against ts_bn_stats + ts_bn_apply through the C ABI: bit for bit,
     # over several calls so that both workspace halves are used and cleared
