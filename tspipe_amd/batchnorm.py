@@ -323,6 +323,17 @@ class DeferredBatchNorm(_BatchNorm):
 
         if not self.training:
             # fixed running statistics (tspipe/batchnorm.py:88-99)
+            if not (torch.is_grad_enabled() and (x.requires_grad or (weight is not None and weight.requires_grad)
+                                                 or (bias is not None and bias.requires_grad))):
+                # nothing to differentiate (a teacher network under no_grad): the launch alone
+                n, c, hw = _dims(x)
+                y = torch.empty_like(x)
+                with _lib.on_device(x.device):
+                    status = _lib.lib().ts_bn_apply(x.data_ptr(), y.data_ptr(), self.running_mean.data_ptr(),
+                                                    self.running_var.data_ptr(), _ptr(weight), _ptr(bias), n, c, hw,
+                                                    1, float(self.eps), _lib.current_stream_ptr(x.device))
+                _lib.check(status, "ts_bn_apply")
+                return y
             return _NormalizeFn.apply(x, weight, bias, self.running_mean, self.running_var,
                                       self, False, float(self.eps))
 
