@@ -468,6 +468,34 @@ def run_kernel_table(dev, with_cpu=True, with_eager=True):
     cpu("kd_256x100_f32", kd_cpu(s, t, 4.0))
     eager("kd_256x100_f32", kd_cpu(s, t, 4.0, device=dev))
 
+    # the soft-target benchmark's whole loss at the same shape: hard-label CE + lambda * KD in one pass
+    y = torch.randint(0, 100, (256,), generator=g).to(dev)
+    g_ce = torch.empty_like(s)
+    ws_ce = torch.empty(lib.ts_kd_workspace_bytes(256, 100, _lib.TS_F32), dtype=torch.uint8, device=dev)
+    loss_ce = torch.empty((), device=dev)
+
+    def f_kdce():
+        _lib.check(lib.ts_kdce_fwd_bwd(s.data_ptr(), t.data_ptr(), None, y.data_ptr(), -100, 256, 100, 100, 100, 0.25,
+                                       16.0 * 0.7, 1.0, ws_ce.data_ptr(), loss_ce.data_ptr(), g_ce.data_ptr(), 100,
+                                       _lib.TS_F32, stream), "ts_kdce_fwd_bwd")
+    out["kdce_256x100_f32"] = entry(3 * 256 * 100 * 4, _time_stream(f_kdce),
+                                    "cfg2's shape with the plug-in's hard-label term (train_kd.py:439-453): CE + 0.7 * KD in "
+                                    "one pass; latency-bound: two launches, every workgroup counts the labels itself", 2,
+                                    working_set=3 * 256 * 100 * 4)
+    s_e = s.detach().clone().requires_grad_()
+
+    def kdce_eager():
+        s_e.grad = None
+        ts_oracle.soft_target_tspipe_loss(s_e, t, y, 4.0, 0.7).backward()
+    eager("kdce_256x100_f32", kdce_eager)
+    if with_cpu:
+        s_c, t_c, y_c = s.detach().cpu().requires_grad_(), t.cpu(), y.cpu()
+
+        def kdce_cpu():
+            s_c.grad = None
+            ts_oracle.soft_target_tspipe_loss(s_c, t_c, y_c, 4.0, 0.7).backward()
+        cpu("kdce_256x100_f32", kdce_cpu)
+
     def kd_sets(rows, V, n_sets):
         fns = []
         for _ in range(n_sets):
