@@ -18,6 +18,9 @@
  *     pair armed by ts_time_next_launch; per process, the address of the
  *     fixed scratch array of ts_kd_fwd_bwd_static, looked up once per GPU;
  *   - workspaces are caller-provided; sizes are stated per function;
+ *   - a loss over zero rows (n_rows / n = 0) is accepted, its input and
+ *     gradient pointers may then be null: loss = NaN, a mean over nothing, as
+ *     the reference's kl_div 'batchmean', cross entropy and row means give;
  *   - "plan" functions are pure host code (no GPU needed): they turn tensor
  *     lists into the chunk tables the kernels walk.
  */

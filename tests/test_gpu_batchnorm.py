@@ -451,3 +451,48 @@ def test_stand_alone_statistics_pass_is_one_launch_that_cleans_up(device, N, C, 
         v64 = x64.var(dim=(0, 2, 3), unbiased=False)
         assert _rel(acc_s, tot_s) < 1e-6 and _rel(acc_q, tot_q) < 1e-6
         assert _rel(mean, m64) < 1e-5 and _rel(inv, 1.0 / torch.sqrt(v64 + 1e-5)) < 1e-6
+
+
+def test_empty_micro_batch_and_one_value_per_channel_follow_the_reference(device):
+    """An empty micro-batch passes through, counts as tracked and commits 0/0 = NaN
+    running statistics; one value per channel in training is tracked, committed and
+    then refused as F.batch_norm refuses it (tspipe/batchnorm.py:103-120); in
+    evaluation mode it is normalised like any input."""
+    ref = ts_oracle.DeferredBNOracle(3, chunks=2)
+    bn = ta.DeferredBatchNorm(3, chunks=2).to(device)
+    g = torch.Generator().manual_seed(5)
+    full = torch.randn(4, 3, 5, generator=g)
+    empty = torch.randn(0, 3, 5)
+    for x in (full, empty):
+        want = ref.forward(x)
+        got = bn(x.to(device))
+        assert got.shape == want.shape
+    assert bn.tracked == ref.tracked == 0 and int(bn.num_batches_tracked) == int(ref.num_batches_tracked) == 1
+    # 4 x 5 values and an empty micro-batch; means near zero are sums that cancel, so the bound is on the largest
+    assert max_rel_to_peak(bn.running_mean, ref.running_mean) < 1e-6
+    xe = empty.to(device).requires_grad_()
+    bn(xe).sum().backward()
+    assert xe.grad.shape == xe.shape
+    # two empty micro-batches: a commit over no values
+    for _ in range(2):
+        ref.forward(empty)
+        bn(empty.to(device))
+    assert torch.isnan(ref.running_mean).all() and torch.isnan(bn.running_mean).all()
+    assert torch.isnan(ref.running_var).all() and torch.isnan(bn.running_var).all()
+
+    ref = ts_oracle.DeferredBNOracle(3, chunks=1)
+    bn = ta.DeferredBatchNorm(3, chunks=1).to(device)
+    one = torch.randn(1, 3, 1, generator=g)
+    with pytest.raises(ValueError, match="Expected more than 1 value per channel") as want_err:
+        ref.forward(one)
+    with pytest.raises(ValueError, match="Expected more than 1 value per channel") as got_err:
+        bn(one.to(device))
+    assert str(got_err.value) == str(want_err.value)
+    assert int(bn.num_batches_tracked) == int(ref.num_batches_tracked) == 1     # tracked and committed before the refusal
+    assert max_rel_to_peak(bn.running_mean, ref.running_mean) < 1e-6
+    assert max_rel_to_peak(bn.running_var, ref.running_var) < 1e-6
+    ref.training = False
+    bn.eval()
+    with torch.no_grad():
+        assert (bn(one.to(device)).cpu() - ref.forward(one)).abs().max() < 2e-5
+    assert bn(empty.to(device)).shape == empty.shape

@@ -403,3 +403,22 @@ def test_ema_more_chunks_than_a_grid_dimension_holds(device):
     torch.cuda.synchronize()
     want = t * torch.tensor(0.99, dtype=torch.float32) + s * torch.tensor(1.0 - 0.99, dtype=torch.float32)
     assert torch.equal(out, want)
+
+
+def test_empty_lists_tensors_and_pieces_pass_through(device):
+    """What the reference's loops and torch.cat / chunk do with nothing in hand."""
+    g = seeded(3)
+    t = [torch.randn(5, generator=g), torch.randn(0), torch.randn(0, 3), torch.randn(2, 2, generator=g)]
+    s = [torch.randn(x.shape, generator=g) for x in t]
+    want = ts_oracle.ema_update(0.9, s, t)
+    got = ta.calculate_target_network_parameters(0.9, [x.to(device) for x in s], [x.to(device) for x in t])
+    assert len(got) == len(want) and all(bits_equal(a, b) for a, b in zip(got, want))
+    assert ta.calculate_target_network_parameters(0.9, [], []) == []
+    pieces = [torch.randn(2, 3, generator=g), torch.randn(0, 3), torch.randn(1, 3, generator=g)]
+    assert bits_equal(ta.gather([ta.Batch(p.to(device)) for p in pieces]), ts_oracle.gather(pieces))
+    nothing = [torch.randn(0, 3), torch.randn(0, 3)]
+    out = ta.gather([ta.Batch(p.to(device)) for p in nothing])
+    assert out.shape == (0, 3) and out.is_cuda
+    got = [b.value for b in ta.scatter(torch.randn(0, 3).to(device), 2)]
+    want = ts_oracle.scatter(torch.randn(0, 3), 2)
+    assert [tuple(x.shape) for x in got] == [tuple(x.shape) for x in want]

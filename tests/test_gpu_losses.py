@@ -1033,3 +1033,35 @@ def test_byol_loss_on_pieces_equals_the_gathered_loss(device):
     nine = [torch.randn(4, c, generator=g).to(device) for _ in range(9)]
     with pytest.raises(Exception):
         ta.byol_contrastive_loss_pieces(nine, nine, nine, nine)
+
+
+def test_losses_over_a_batch_without_rows_give_nan_and_empty_gradients(device):
+    """kl_div 'batchmean', cross entropy and the row means of the reference all
+    divide a zero sum by zero rows: NaN loss, empty gradient, no error."""
+    from argparse import Namespace
+
+    def run(fn, *xs):
+        xs = [x.clone().requires_grad_() if x.is_floating_point() else x for x in xs]
+        loss = fn(*xs)
+        loss.backward()
+        return loss.detach().cpu(), xs[0].grad
+
+    z, zl = torch.randn(0, 100), torch.zeros(0, dtype=torch.long)
+    e, q = torch.randn(0, 128), torch.randn(0, 256)
+    ns = Namespace(T=4.0, lambda_kd=0.7, kd_mode="st", moco_t=0.2)
+    cases = [
+        (lambda a, b: ts_oracle.kd_soft_target(a, b, 4.0), lambda a, b: ta.kd_soft_target_loss(a, b, 4.0), (z, z)),
+        (lambda a, b, y: ts_oracle.soft_target_tspipe_loss(a, b, y, 4.0, 0.7),
+         lambda a, b, y: ta.soft_target_tspipe_loss(a, b, y, None, ns, 0), (z, z, zl)),
+        (ts_oracle.logits_mse, ta.logits_mse_loss, (z, z)),
+        (ts_oracle.byol_contrastive_loss, ta.byol_contrastive_loss, (e, e, e, e)),
+        (lambda a, b, c, d: ts_oracle.moco_contrastive_loss(a, b, c, d, 0.2),
+         lambda a, b, c, d: ta.moco_contrastive_loss(a, b, c, d, None, ns), (q, q, q, q)),
+        (lambda a, b, c, d: ts_oracle.moco_contrastive_loss(a, b, c, d, 0.2),
+         lambda a, b, c, d: ta.moco_contrastive_loss(a, b, c, d, None, ns), (q.bfloat16(), ) * 4),
+    ]
+    for ref_fn, got_fn, xs in cases:
+        ref_loss, ref_grad = run(ref_fn, *xs)
+        got_loss, got_grad = run(got_fn, *[x.to(device) for x in xs])
+        assert torch.isnan(ref_loss) and torch.isnan(got_loss)
+        assert got_grad.shape == ref_grad.shape and got_grad.dtype == ref_grad.dtype and got_grad.is_cuda

@@ -320,6 +320,9 @@ class DeferredBatchNorm(_BatchNorm):
         x = input if input.is_contiguous() else input.contiguous()
         weight = self.weight if self.affine else None
         bias = self.bias if self.affine else None
+        per_channel = input.numel() // input.size(1) if input.size(1) else 0
+        if per_channel <= 1 and (self.training or per_channel == 0):
+            return self._forward_without_a_batch(input, x, per_channel)
 
         if not self.training:
             # fixed running statistics (tspipe/batchnorm.py:88-99)
@@ -362,6 +365,25 @@ class DeferredBatchNorm(_BatchNorm):
         if st.tracked == st.chunks:
             self._commit()
         return y
+
+    def _forward_without_a_batch(self, input: Tensor, x: Tensor, per_channel: int) -> Tensor:
+        """The two inputs no kernel normalises.  An empty micro-batch comes back
+        empty; in training it still counts as tracked, and a commit over zero
+        values leaves NaN running statistics (0/0), as tspipe/batchnorm.py:45-85
+        does.  One value per channel in training is tracked and committed like
+        any micro-batch (batchnorm.py:103-108) and then refused with the error
+        that ``F.batch_norm(training=True)`` raises at batchnorm.py:111-120."""
+        if self.training:
+            if per_channel:
+                self._stats(x.detach(), accumulate=True)
+            st = self._st
+            st.counter += per_channel
+            st.tracked += 1
+            if st.tracked == st.chunks:
+                self._commit()
+            if per_channel:
+                raise ValueError(f"Expected more than 1 value per channel when training, got input size {input.size()}")
+        return x.clone()
 
     @classmethod
     def convert_deferred_batch_norm(cls, module: TModule, chunks: int = 1) -> TModule:

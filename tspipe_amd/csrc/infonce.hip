@@ -992,7 +992,7 @@ size_t ts_infonce_workspace_bytes(int64_t n, int64_t c, int n_pairs) {
 int ts_infonce_fwd_bwd(const void* q1, const void* k1, const void* q2, const void* k2, int64_t n, int64_t c,
                        float tau, void* workspace, float* loss_out, void* dq1, void* dq2, int dtype,
                        ts_stream_t stream) {
-  if (!q1 || !k1 || !workspace || !loss_out) return TS_ERR_ARG;
+  if (!loss_out || (n > 0 && (!q1 || !k1 || !workspace))) return TS_ERR_ARG;
   if ((q2 == nullptr) != (k2 == nullptr)) return TS_ERR_ARG;
   if (n < 0 || !(tau > 0.f) || c < 1) return TS_ERR_ARG;
   if (dtype != TS_F32 && dtype != TS_BF16 && dtype != TS_F16) return TS_ERR_ARG;

@@ -651,7 +651,8 @@ size_t ts_cosine_workspace_bytes(int64_t n) {
 
 int ts_cosine_fwd_bwd(const void* x, const void* y, const uint8_t* row_mask, int64_t n, int64_t c, float weight,
                       void* workspace, float* loss_out, void* gx, int dtype, ts_stream_t stream) {
-  if (!x || !y || !workspace || !loss_out) return TS_ERR_ARG;
+  // no rows, nothing to point at: the loss is then a mean over nothing, NaN
+  if (!loss_out || (n > 0 && (!x || !y || !workspace))) return TS_ERR_ARG;
   if (n < 0 || c <= 0) return TS_ERR_ARG;
   if (dtype != TS_F32 && dtype != TS_BF16 && dtype != TS_F16) return TS_ERR_ARG;
   if (n > (1 << 24)) return TS_ERR_RANGE;
@@ -683,7 +684,7 @@ size_t ts_mse_workspace_bytes(int64_t n_rows, int64_t V) {
 int ts_mse_fwd_bwd(const void* s, const void* t, const uint8_t* row_mask, int64_t n_rows, int64_t V, int64_t ld_s,
                    int64_t ld_t, float weight, int per_element, int accumulate, void* workspace, float* loss_out,
                    void* grad, int64_t ld_g, int dtype, ts_stream_t stream) {
-  if (!s || !t || !workspace || !loss_out) return TS_ERR_ARG;
+  if (!loss_out || (n_rows > 0 && (!s || !t || !workspace))) return TS_ERR_ARG;
   if (n_rows < 0 || V <= 0 || ld_s < V || ld_t < V || (grad && ld_g < V)) return TS_ERR_ARG;
   if (dtype != TS_F32 && dtype != TS_BF16 && dtype != TS_F16) return TS_ERR_ARG;
   if (n_rows > (1 << 24) || n_rows * ts::mse_parts(V) > 0x7fffffffLL) return TS_ERR_RANGE;
@@ -715,9 +716,10 @@ int ts_mse_pieces_fwd_bwd(const void* const* s_pieces, const void* const* t_piec
 
 int ts_scale_rows(void* grad, int64_t n_rows, int64_t V, int64_t ld_g, const float* g_dev, int dtype,
                   ts_stream_t stream) {
-  if (!grad || !g_dev || n_rows < 0 || V < 0 || ld_g < V) return TS_ERR_ARG;
+  if (!g_dev || n_rows < 0 || V < 0 || ld_g < V) return TS_ERR_ARG;
   if (dtype != TS_F32 && dtype != TS_BF16 && dtype != TS_F16) return TS_ERR_ARG;
   if (n_rows == 0 || V == 0) return TS_OK;
+  if (!grad) return TS_ERR_ARG;
   // a contiguous matrix is one long row: keeps gridDim.y within 65535
   if (ld_g == V) {
     V = n_rows * V;
@@ -746,7 +748,7 @@ int ts_scale_rows(void* grad, int64_t n_rows, int64_t V, int64_t ld_g, const flo
 int ts_byol_fwd_bwd(const void* x1, const void* y1, const void* x2, const void* y2, int64_t n,
                     int64_t c, float* workspace, float* loss_out, void* gx1, void* gx2, int dtype,
                     ts_stream_t stream) {
-  if (!x1 || !y1 || !workspace || !loss_out) return TS_ERR_ARG;
+  if (!loss_out || (n > 0 && (!x1 || !y1 || !workspace))) return TS_ERR_ARG;
   if ((x2 == nullptr) != (y2 == nullptr)) return TS_ERR_ARG;
   if (n < 0 || c <= 0) return TS_ERR_ARG;
   if (dtype != TS_F32 && dtype != TS_BF16 && dtype != TS_F16) return TS_ERR_ARG;
