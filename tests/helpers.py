@@ -20,6 +20,8 @@ def bits_equal(a: torch.Tensor, b: torch.Tensor) -> bool:
     a, b = a.detach().cpu().contiguous(), b.detach().cpu().contiguous()
     if a.shape != b.shape or a.dtype != b.dtype:
         return False
+    if a.dim() == 0:
+        a, b = a.reshape(1), b.reshape(1)
     return bool(torch.equal(a.view(torch.uint8), b.view(torch.uint8)))
 
 

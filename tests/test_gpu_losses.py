@@ -10,7 +10,7 @@ import pytest
 import torch
 
 import tspipe_amd as ta
-from helpers import max_rel_to_peak, rel_err, seeded
+from helpers import bits_equal, max_rel_to_peak, rel_err, seeded
 from oracle import ts_oracle
 
 pytestmark = pytest.mark.gpu
@@ -1065,3 +1065,58 @@ def test_losses_over_a_batch_without_rows_give_nan_and_empty_gradients(device):
         got_loss, got_grad = run(got_fn, *[x.to(device) for x in xs])
         assert torch.isnan(ref_loss) and torch.isnan(got_loss)
         assert got_grad.shape == ref_grad.shape and got_grad.dtype == ref_grad.dtype and got_grad.is_cuda
+
+
+def test_cpp_autograd_node_and_python_functions_of_the_row_losses_agree(device, monkeypatch):
+    """The plain calls of the KD / squared-error / cosine / BYOL plug-ins run as a
+    C++ autograd node of the host helper; it makes the same calls on the same entry
+    points as the Python autograd.Functions, so loss and gradients agree bit for bit,
+    also under a scaled grad_output, N-D inputs, masks and labels."""
+    from tspipe_amd import _lib, losses
+    if _lib.host_helper() is None or not hasattr(_lib.host_helper(), "row_loss"):
+        pytest.skip("host helper not built")
+    g = seeded(21)
+
+    def both(fn, n_leaves, *xs):
+        results = []
+        for node in (True, False):
+            monkeypatch.setattr(losses, "_HOST_NODE", node)
+            leaves = [x.clone().requires_grad_() for x in xs[:n_leaves]]
+            loss = fn(*leaves, *xs[n_leaves:])
+            assert ("RowLossNode" in loss.grad_fn.name()) == node, loss.grad_fn.name()
+            (loss * 0.37).backward()
+            results.append((loss.detach(), [x.grad for x in leaves]))
+        (la, ga), (lb, gb) = results
+        assert bits_equal(la, lb)
+        assert all(bits_equal(a, b) for a, b in zip(ga, gb))
+        assert all(a.shape == x.shape for a, x in zip(ga, xs))
+
+    for dtype in (torch.float32, torch.bfloat16):
+        s = (torch.randn(6, 50, 100, generator=g) * 2).to(device, dtype)
+        t = (torch.randn(6, 50, 100, generator=g) * 2).to(device, dtype)
+        mask = (torch.rand(6, 50, generator=g) < 0.4).to(device)
+        labels = torch.randint(0, 100, (6, 50), generator=g).to(device)
+        labels[0, :7] = -100
+        both(lambda a, b: ta.kd_soft_target_loss(a, b, 4.0), 1, s, t)
+        both(lambda a, b: ta.distil_ce_loss(a, b, mask, 2.0, 5.0), 1, s, t)
+        both(lambda a, b: ta.kd_ce_loss(a, b, labels, 2.0, 5.0, 2.0, row_mask=mask, mse_weight=0.5), 1, s, t)
+        both(lambda a, b: ta.logits_mse_loss(a, b), 1, s, t)
+        both(lambda a, b: ta.logits_mse_loss(a, b, mask, 0.5, False), 1, s, t)
+        both(lambda a, b: ta.cosine_embedding_loss(a, b, mask, 1.5), 1, s, t)
+        x = [torch.randn(77, 128, generator=g).to(device, dtype) for _ in range(4)]
+        both(lambda a, b, c, d: ta.byol_contrastive_loss(a, b, c, d), 2, *x)
+        both(lambda a, b: losses.regression_loss_mean(a, b), 1, x[0], x[2])
+    # without gradient mode and without a leaf: a loss and nothing else
+    monkeypatch.setattr(losses, "_HOST_NODE", True)
+    with torch.no_grad():
+        a = ta.kd_soft_target_loss(s.clone().requires_grad_(), t, 4.0)
+    b = ta.kd_soft_target_loss(s, t, 4.0)
+    assert a.grad_fn is None and b.grad_fn is None and bits_equal(a, b)
+    # calls that are not plain take the Python path and its errors
+    with pytest.raises(ValueError):
+        ta.kd_soft_target_loss(s, t[:, :, :50], 4.0)
+    with pytest.raises(TypeError):
+        ta.kd_soft_target_loss(s.cpu(), t.cpu(), 4.0)
+    strided = s.transpose(0, 1).requires_grad_()
+    loss = ta.kd_soft_target_loss(strided, t.transpose(0, 1), 4.0)
+    assert "RowLossNode" not in loss.grad_fn.name()

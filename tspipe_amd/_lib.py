@@ -139,6 +139,11 @@ def host_helper():
                                  addr(handle.ts_scale_rows))
                     if hasattr(mod, "bind_bn"):
                         mod.bind_bn(addr(handle.ts_bn_forward_train), addr(handle.ts_bn_backward))
+                    if hasattr(mod, "bind_losses"):
+                        mod.bind_losses(addr(handle.ts_kd_workspace_bytes), addr(handle.ts_kdce_fwd_bwd),
+                                        addr(handle.ts_mse_workspace_bytes), addr(handle.ts_mse_fwd_bwd),
+                                        addr(handle.ts_cosine_workspace_bytes), addr(handle.ts_cosine_fwd_bwd),
+                                        addr(handle.ts_byol_fwd_bwd))
                 _host = mod
             _host_tried = True
     return _host

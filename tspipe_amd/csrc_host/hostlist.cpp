@@ -6,6 +6,7 @@
 #include <torch/csrc/autograd/python_variable.h>
 #include <ATen/detail/CUDAHooksInterface.h>
 
+#include <algorithm>
 #include <cstdint>
 #include <vector>
 
@@ -289,6 +290,187 @@ py::object bn_train(const at::Tensor& x, const c10::optional<at::Tensor>& weight
   return py::cast(y);
 }
 
+// ---------------------------------------------------------------------------
+// The row losses (KD with its cross-entropy and squared-error riders, squared
+// error alone, cosine, BYOL) as one C++ autograd node, for the same reason as
+// the two above: at the batch sizes of the CIFAR-sized benchmarks the kernels
+// take 7-12 us and a Python autograd.Function around them 50-300.  Each kind
+// is the same call sequence as its Python Function, on the same C entry
+// points, so both give the same bits.
+// ---------------------------------------------------------------------------
+typedef size_t (*kd_ws_fn)(int64_t, int64_t, int);
+typedef int (*kdce_fn)(const void*, const void*, const uint8_t*, const int64_t*, int64_t, int64_t, int64_t, int64_t,
+                       int64_t, float, float, float, void*, float*, void*, int64_t, int, void*);
+typedef size_t (*mse_ws_fn)(int64_t, int64_t);
+typedef int (*mse_fn)(const void*, const void*, const uint8_t*, int64_t, int64_t, int64_t, int64_t, float, int, int,
+                      void*, float*, void*, int64_t, int, void*);
+typedef size_t (*cos_ws_fn)(int64_t);
+typedef int (*cos_fn)(const void*, const void*, const uint8_t*, int64_t, int64_t, float, void*, float*, void*, int,
+                      void*);
+typedef int (*byol_fn)(const void*, const void*, const void*, const void*, int64_t, int64_t, float*, float*, void*,
+                       void*, int, void*);
+static kd_ws_fn g_kd_ws = nullptr;
+static kdce_fn g_kdce = nullptr;
+static mse_ws_fn g_mse_ws = nullptr;
+static mse_fn g_mse = nullptr;
+static cos_ws_fn g_cos_ws = nullptr;
+static cos_fn g_cos = nullptr;
+static byol_fn g_byol = nullptr;
+
+void bind_losses(uintptr_t kd_ws, uintptr_t kdce, uintptr_t mse_ws, uintptr_t mse, uintptr_t cos_ws, uintptr_t cos,
+                 uintptr_t byol) {
+  g_kd_ws = reinterpret_cast<kd_ws_fn>(kd_ws);
+  g_kdce = reinterpret_cast<kdce_fn>(kdce);
+  g_mse_ws = reinterpret_cast<mse_ws_fn>(mse_ws);
+  g_mse = reinterpret_cast<mse_fn>(mse);
+  g_cos_ws = reinterpret_cast<cos_ws_fn>(cos_ws);
+  g_cos = reinterpret_cast<cos_fn>(cos);
+  g_byol = reinterpret_cast<byol_fn>(byol);
+}
+
+enum LossKind : int64_t { kLossKd = 0, kLossMse = 1, kLossCosine = 2, kLossByol = 3 };
+
+struct RowLossNode : public torch::autograd::Function<RowLossNode> {
+  // x1 (and x2, BYOL's second student) may require gradients; y1, y2, mask and labels never do.
+  // f: kind-specific numbers (see row_loss below); n: kind-specific integers.
+  static at::Tensor forward(torch::autograd::AutogradContext* ctx, const at::Tensor& x1, const at::Tensor& y1,
+                            const c10::optional<at::Tensor>& x2o, const c10::optional<at::Tensor>& y2o,
+                            const c10::optional<at::Tensor>& mask, const c10::optional<at::Tensor>& labels,
+                            int64_t kind, std::vector<double> f, std::vector<int64_t> n, int64_t stream) {
+    const int64_t V = x1.size(-1), rows = V ? x1.numel() / V : 0;
+    const int code = dtype_code(x1.scalar_type());
+    c10::DeviceGuard guard(x1.device());
+    void* st = reinterpret_cast<void*>(stream);
+    const uint8_t* mask_ptr = mask.has_value() ? static_cast<const uint8_t*>(mask->data_ptr()) : nullptr;
+    at::Tensor loss = at::empty({}, x1.options().dtype(at::kFloat));
+    at::Tensor g1, g2, ws;
+    if (x1.requires_grad()) g1 = at::empty_like(x1);
+    auto bytes = [&](size_t b) { return at::empty({(int64_t)b}, x1.options().dtype(at::kByte)); };
+    int rc = 0;
+    const char* what = "";
+    switch (kind) {
+      case kLossKd: {
+        // f = {T, weight, ce_weight, mse_weight}; n = {ignore_index, mse_per_element}
+        const double T = f[0];
+        ws = bytes(g_kd_ws(rows, V, code));
+        what = "ts_kdce_fwd_bwd";
+        rc = g_kdce(x1.data_ptr(), y1.data_ptr(), mask_ptr,
+                    labels.has_value() ? labels->data_ptr<int64_t>() : nullptr, n[0], rows, V, V, V, (float)(1.0 / T),
+                    (float)(T * T * f[1]), (float)f[2], ws.data_ptr(), loss.data_ptr<float>(),
+                    g1.defined() ? g1.data_ptr() : nullptr, V, code, st);
+        if (rc == 0 && f[3] > 0.0) {
+          at::Tensor ws2 = bytes(g_mse_ws(rows, V));
+          what = "ts_mse_fwd_bwd";
+          rc = g_mse(x1.data_ptr(), y1.data_ptr(), mask_ptr, rows, V, V, V, (float)f[3], (int)n[1], 1, ws2.data_ptr(),
+                     loss.data_ptr<float>(), g1.defined() ? g1.data_ptr() : nullptr, V, code, st);
+        }
+        break;
+      }
+      case kLossMse:
+        // f = {weight}; n = {per_element}
+        ws = bytes(g_mse_ws(rows, V));
+        what = "ts_mse_fwd_bwd";
+        rc = g_mse(x1.data_ptr(), y1.data_ptr(), mask_ptr, rows, V, V, V, (float)f[0], (int)n[0], 0, ws.data_ptr(),
+                   loss.data_ptr<float>(), g1.defined() ? g1.data_ptr() : nullptr, V, code, st);
+        break;
+      case kLossCosine:
+        // f = {weight}
+        ws = bytes(g_cos_ws(rows));
+        what = "ts_cosine_fwd_bwd";
+        rc = g_cos(x1.data_ptr(), y1.data_ptr(), mask_ptr, rows, V, (float)f[0], ws.data_ptr(), loss.data_ptr<float>(),
+                   g1.defined() ? g1.data_ptr() : nullptr, code, st);
+        break;
+      default: {
+        const bool two = x2o.has_value();
+        if (two && x2o->requires_grad()) g2 = at::empty_like(*x2o);
+        ws = at::empty({2 * std::max<int64_t>(rows, 1)}, x1.options().dtype(at::kFloat));
+        what = "ts_byol_fwd_bwd";
+        rc = g_byol(x1.data_ptr(), y1.data_ptr(), two ? x2o->data_ptr() : nullptr, two ? y2o->data_ptr() : nullptr,
+                    rows, V, ws.data_ptr<float>(), loss.data_ptr<float>(), g1.defined() ? g1.data_ptr() : nullptr,
+                    g2.defined() ? g2.data_ptr() : nullptr, code, st);
+      }
+    }
+    TORCH_CHECK(rc == 0, what, ": status ", rc);
+    ctx->saved_data["g1"] = g1;
+    ctx->saved_data["g2"] = g2;
+    ctx->saved_data["stream"] = stream;
+    ctx->saved_data["done"] = false;
+    return loss;
+  }
+
+  static torch::autograd::variable_list backward(torch::autograd::AutogradContext* ctx,
+                                                 torch::autograd::variable_list grad_out) {
+    TORCH_CHECK(!ctx->saved_data["done"].toBool(),
+                "the fused loss keeps one gradient buffer: backward can run once per forward");
+    ctx->saved_data["done"] = true;
+    // the context lets go of the buffers, so that autograd can adopt them as .grad instead of copying
+    at::Tensor g1 = ctx->saved_data["g1"].toTensor(), g2 = ctx->saved_data["g2"].toTensor();
+    ctx->saved_data["g1"] = at::Tensor();
+    ctx->saved_data["g2"] = at::Tensor();
+    void* stream = reinterpret_cast<void*>(ctx->saved_data["stream"].toInt());
+    at::Tensor go = grad_out[0];
+    if (go.scalar_type() != at::kFloat) go = go.to(at::kFloat);
+    for (at::Tensor* g : {&g1, &g2}) {
+      if (!g->defined() || g->numel() == 0) continue;
+      const int64_t V = g->size(-1);
+      const int rc = g_scale(g->data_ptr(), g->numel() / V, V, V, go.data_ptr<float>(), dtype_code(g->scalar_type()),
+                             stream);
+      TORCH_CHECK(rc == 0, "ts_scale_rows: status ", rc);
+    }
+    return {g1,           at::Tensor(), g2,           at::Tensor(), at::Tensor(),
+            at::Tensor(), at::Tensor(), at::Tensor(), at::Tensor(), at::Tensor()};
+  }
+};
+
+// kind 0 (KD): f = {T, weight, ce_weight, mse_weight}, n = {ignore_index, mse_per_element};
+// kind 1 (squared error): f = {weight}, n = {per_element}; kind 2 (cosine): f = {weight};
+// kind 3 (BYOL): x2 / y2 the second pair or None.
+// Returns None when the call is not of the plain kind, and the Python autograd.Function takes it
+// (and raises the proper errors): dense device tensors of one shape and floating dtype with at
+// least one row, teachers without gradients, a bool / uint8 mask with one entry per row, int64 labels.
+py::object row_loss(int64_t kind, const at::Tensor& x1, const at::Tensor& y1, const c10::optional<at::Tensor>& x2,
+                    const c10::optional<at::Tensor>& y2, const c10::optional<at::Tensor>& mask,
+                    const c10::optional<at::Tensor>& labels, std::vector<double> f, std::vector<int64_t> n,
+                    int64_t stream) {
+  if (!g_kdce || !g_mse || !g_cos || !g_byol || !g_scale) return py::none();
+  if (kind < kLossKd || kind > kLossByol) return py::none();
+  if (f.size() < (kind == kLossKd ? 4u : kind == kLossByol ? 0u : 1u)) return py::none();
+  if (n.size() < (kind == kLossKd ? 2u : kind == kLossMse ? 1u : 0u)) return py::none();
+  if (x2.has_value() != y2.has_value() || (x2.has_value() && kind != kLossByol)) return py::none();
+  if (x1.dim() < 1 || (kind == kLossByol && x1.dim() != 2) || x1.numel() == 0) return py::none();
+  if (dtype_code(x1.scalar_type()) < 0) return py::none();
+  const at::Tensor* all[4] = {&x1, &y1, x2.has_value() ? &*x2 : nullptr, y2.has_value() ? &*y2 : nullptr};
+  for (const at::Tensor* t : all) {
+    if (!t) continue;
+    if (!t->is_cuda() || !t->is_contiguous() || t->sizes() != x1.sizes() || t->scalar_type() != x1.scalar_type() ||
+        t->device() != x1.device())
+      return py::none();
+  }
+  if (y1.requires_grad() || (y2.has_value() && y2->requires_grad())) return py::none();
+  const int64_t rows = x1.numel() / x1.size(-1);
+  if (mask.has_value()) {
+    if (kind == kLossByol) return py::none();
+    const at::Tensor& m = *mask;
+    // (masks of other types mean "not zero" and are converted by the Python path)
+    if (!m.is_cuda() || m.device() != x1.device() || !m.is_contiguous() || m.numel() != rows ||
+        m.scalar_type() != at::kBool)
+      return py::none();
+  }
+  if (labels.has_value()) {
+    const at::Tensor& l = *labels;
+    if (kind != kLossKd || !l.is_cuda() || l.device() != x1.device() || !l.is_contiguous() || l.numel() != rows ||
+        l.scalar_type() != at::kLong)
+      return py::none();
+  }
+  if (kind == kLossKd && !(f[0] > 0.0)) return py::none();
+  // without gradient mode nothing is recorded, so no gradient buffer is wanted either
+  const bool record = at::GradMode::is_enabled();
+  c10::optional<at::Tensor> s2 = x2;
+  if (!record && x2.has_value()) s2 = x2->detach();
+  at::Tensor loss = RowLossNode::apply(record ? x1 : x1.detach(), y1, s2, y2, mask, labels, kind, f, n, stream);
+  return py::cast(loss);
+}
+
 // Test aid: a C++ owner of a tensor that Python cannot see.  hold() keeps the
 // tensor alive inside this module until drop() is called.
 static std::vector<at::Tensor> g_held;
@@ -304,6 +486,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("bind_abi", &bind_abi);
   m.def("infonce", &infonce);
   m.def("bind_bn", &bind_bn);
+  m.def("bind_losses", &bind_losses);
+  m.def("row_loss", &row_loss);
   m.def("bn_train", &bn_train);
   m.def("hold", &hold);
   m.def("drop", &drop);

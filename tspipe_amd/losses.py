@@ -44,6 +44,24 @@ def _scale_saved_grad(grad: Tensor, grad_output: Tensor, rows: int, cols: int) -
     return grad
 
 
+_HOST_NODE = True   # tests switch this off to reach the Python autograd.Functions
+_KD, _MSE, _COSINE, _BYOL = 0, 1, 2, 3
+
+
+def _host_row_loss(kind: int, x1, y1, x2, y2, mask, labels, f, n):
+    """The plain case of a row loss through the C++ autograd node of the host
+    helper (the same entry points in the same order as the Python Functions
+    below, so the same bits; its backward needs no interpreter).  None when the
+    helper is not built or the call is not plain: then the Python Function takes
+    it, and raises the proper errors."""
+    if not _HOST_NODE:
+        return None
+    host = _lib.host_helper()
+    if host is None or type(x1) is not Tensor or not x1.is_cuda or not hasattr(host, "row_loss"):
+        return None
+    return host.row_loss(kind, x1, y1, x2, y2, mask, labels, f, n, _lib.current_stream_ptr(x1.device))
+
+
 # ---------------------------------------------------------------------------
 # KD soft-target loss
 # ---------------------------------------------------------------------------
@@ -128,6 +146,9 @@ def kd_soft_target_loss(out_s: Tensor, out_t: Tensor, T: float, weight: float = 
     the rows (last dimension = classes) selected by ``row_mask`` (all rows when
     ``None``); the formula of benchmarks/soft_target/kd_losses/st.py:18-23 and,
     with a mask, of benchmarks/distilbert/distiller.py:719-740."""
+    out = _host_row_loss(_KD, out_s, out_t, None, None, row_mask, None, [float(T), float(weight), 0.0, 0.0], [-100, 0])
+    if out is not None:
+        return out
     return _KDSoftTargetFn.apply(out_s, out_t, row_mask, float(T), float(weight))
 
 
@@ -151,6 +172,10 @@ def distil_ce_loss(s_logits: Tensor, t_logits: Tensor, row_mask: Tensor, tempera
     logits where ``row_mask`` (``[bs, seq]``) is set, KL with batchmean over the
     selected rows, times ``temperature**2`` and ``alpha_ce``.  No row is copied:
     the kernel reads the mask and writes a dense gradient with zeros elsewhere."""
+    out = _host_row_loss(_KD, s_logits, t_logits, None, None, row_mask, None,
+                         [float(temperature), float(alpha_ce), 0.0, 0.0], [-100, 0])
+    if out is not None:
+        return out
     return _KDSoftTargetFn.apply(s_logits, t_logits, row_mask, float(temperature), float(alpha_ce))
 
 
@@ -166,8 +191,13 @@ def kd_ce_loss(out_s: Tensor, out_t: Tensor, labels: Optional[Tensor], T: float,
     over the rows of ``row_mask`` (distiller.py:751-755; divided by the number
     of elements instead with ``mse_per_element``, as ``F.mse_loss`` does),
     accumulated into the same gradient buffer."""
-    return _KDSoftTargetFn.apply(out_s, out_t, row_mask, float(T), float(kd_weight), labels,
-                                 float(ce_weight) if labels is not None else 0.0, int(ignore_index),
+    ce = float(ce_weight) if labels is not None else 0.0
+    out = _host_row_loss(_KD, out_s, out_t, None, None, row_mask, labels,
+                         [float(T), float(kd_weight), ce, float(mse_weight)],
+                         [int(ignore_index), 1 if mse_per_element else 0])
+    if out is not None:
+        return out
+    return _KDSoftTargetFn.apply(out_s, out_t, row_mask, float(T), float(kd_weight), labels, ce, int(ignore_index),
                                  float(mse_weight), bool(mse_per_element))
 
 
@@ -317,6 +347,9 @@ def logits_mse_loss(out_s: Tensor, out_t: Tensor, row_mask: Optional[Tensor] = N
     ``per_element=False`` with a ``[bs, seq]`` mask is DistilBERT's
     ``MSELoss(reduction="sum")(s_slct, t_slct) / s_slct.size(0)``
     (benchmarks/distilbert/distiller.py:751-755)."""
+    out = _host_row_loss(_MSE, out_s, out_t, None, None, row_mask, None, [float(weight)], [1 if per_element else 0])
+    if out is not None:
+        return out
     return _LogitsMSEFn.apply(out_s, out_t, row_mask, float(weight), bool(per_element))
 
 
@@ -374,6 +407,9 @@ def cosine_embedding_loss(x: Tensor, y: Tensor, row_mask: Optional[Tensor] = Non
     """``weight * CosineEmbeddingLoss(reduction="mean")(x[rows], y[rows], +1)`` over
     the rows (last dimension = features) kept by ``row_mask``; gradient to ``x``
     only (benchmarks/distilbert/distiller.py:756-770)."""
+    out = _host_row_loss(_COSINE, x, y, None, None, row_mask, None, [float(weight)], [])
+    if out is not None:
+        return out
     return _CosineFn.apply(x, y, row_mask, float(weight))
 
 
@@ -494,11 +530,17 @@ def byol_loss(online_view_1: Tensor, online_view_2: Tensor, target_view_1: Tenso
               target_view_2: Tensor) -> Tensor:
     """``mean(rl(o1, t2) + rl(o2, t1))`` with ``rl(x, y) = 2 - 2 <x^, y^>``
     (benchmarks/byol/trainer.py:51-55, 192-196)."""
+    out = _host_row_loss(_BYOL, online_view_1, target_view_2, online_view_2, target_view_1, None, None, [], [])
+    if out is not None:
+        return out
     return _BYOLFn.apply(online_view_1, target_view_2, online_view_2, target_view_1)
 
 
 def regression_loss_mean(x: Tensor, y: Tensor) -> Tensor:
     """``regression_loss(x, y).mean()`` for a single pair (benchmarks/byol/trainer.py:51-55)."""
+    out = _host_row_loss(_BYOL, x, y, None, None, None, None, [], [])
+    if out is not None:
+        return out
     return _BYOLFn.apply(x, y, None, None)
 
 
