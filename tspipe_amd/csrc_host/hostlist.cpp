@@ -187,7 +187,11 @@ py::object infonce(const at::Tensor& q1, const at::Tensor& k1, const c10::option
   const int64_t c = q1.size(1);
   if ((c != 64 && c != 128 && c != 256) || dtype_code(q1.scalar_type()) < 0 || !(tau >= 0.03)) return py::none();
   if (k1.requires_grad() || (two && k2->requires_grad())) return py::none();
-  at::Tensor loss = InfoNCENode::apply(q1, k1, q2, k2, tau, stream);
+  // without gradient mode nothing is recorded, so no gradient buffer is wanted either
+  const bool record = at::GradMode::is_enabled();
+  c10::optional<at::Tensor> s2 = q2;
+  if (!record && two) s2 = q2->detach();
+  at::Tensor loss = InfoNCENode::apply(record ? q1 : q1.detach(), k1, s2, k2, tau, stream);
   return py::cast(loss);
 }
 
