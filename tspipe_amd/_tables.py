@@ -146,7 +146,7 @@ def stage_ema(t_ptrs: np.ndarray, s_ptrs: np.ndarray, o_ptrs: np.ndarray, numels
     n = len(numels)
     if chunk_elems == 0:
         chunk_elems = lib.ts_ema_auto_chunk(int(numels.sum()))
-    stream_id = torch.cuda.current_stream(device).cuda_stream
+    stream_id = _lib.current_stream_ptr(device)
     key = b"".join((t_ptrs[:n].tobytes(), s_ptrs[:n].tobytes(), o_ptrs[:n].tobytes(), numels[:n].tobytes(),
                     int(chunk_elems).to_bytes(8, "little"), int(stream_id).to_bytes(8, "little"),
                     bytes((dtype,))))

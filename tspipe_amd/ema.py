@@ -153,7 +153,7 @@ class _Arena:
         device = teachers[0].device
         # like a block of torch's caching allocator, the arena belongs to the
         # stream it was made on and is only handed out again on that stream
-        self.stream = torch.cuda.current_stream(device).cuda_stream if device.type == "cuda" else None
+        self.stream = _lib.current_stream_ptr(device) if device.type == "cuda" else None
         numels = np.array(list(map(torch.Tensor.numel, teachers)), dtype=np.int64)
         dtype = teachers[0].dtype
         mask = 16 // teachers[0].element_size() - 1  # elements per 16 bytes, minus one
@@ -251,15 +251,17 @@ def _acquire_arena(teachers: Sequence[torch.Tensor], shapes):
         arena = _Arena(teachers)
         return arena, list(arena.views)
     device = teachers[0].device
-    stream = torch.cuda.current_stream(device)
-    key = (device, stream.cuda_stream, shapes)
+    # (the raw handle: a torch Stream object per call costs more than the rest of this function)
+    key = (device, _lib.current_stream_ptr(device), shapes)
     with _pool_lock:
         arenas = _pool.setdefault(key, [])
         for arena in arenas:
             if arena.is_free():
                 # streams that were announced as readers of the old contents
-                for event in arena.readers:
-                    stream.wait_event(event)
+                if arena.readers:
+                    stream = torch.cuda.current_stream(device)
+                    for event in arena.readers:
+                        stream.wait_event(event)
                 arena.readers = []
                 return arena, list(arena.views)
         arena = _Arena(teachers)

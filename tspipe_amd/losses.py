@@ -613,7 +613,7 @@ def _infonce(q1: Tensor, k1: Tensor, q2: Optional[Tensor], k2: Optional[Tensor],
     interpreter lock; everything else, and every error, to the Python one."""
     host = _lib.host_helper()
     if host is not None and type(q1) is Tensor and q1.is_cuda and hasattr(host, "infonce"):
-        out = host.infonce(q1, k1, q2, k2, tau, torch.cuda.current_stream(q1.device).cuda_stream)
+        out = host.infonce(q1, k1, q2, k2, tau, _lib.current_stream_ptr(q1.device))
         if out is not None:
             return out
     return _InfoNCEFn.apply(q1, k1, q2, k2, tau)
