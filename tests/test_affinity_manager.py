@@ -113,3 +113,27 @@ def test_map_of_this_machine(device):
     assert 0 in lists and lists[0] and all(0 <= c < os.cpu_count() for c in lists[0])
     chosen = AffinityManager.get_gpu_affinity_map()
     assert 1 <= len(chosen[0]) <= 4 and chosen[0] == lists[0][:len(chosen[0])]
+
+
+def test_pure_functions_against_the_reference_recorded_cases():
+    """tests/golden/affinity_cases.json holds what the reference's parse_affinity and
+    num_cpus_for_gpu returned or raised (written by tests/golden/make_affinity_fixtures.py)."""
+    import json
+    here = os.path.dirname(os.path.abspath(__file__))
+    with open(os.path.join(here, "golden", "affinity_cases.json")) as fh:
+        cases = json.load(fh)
+
+    def attempt(fn, *args):
+        try:
+            return {"value": fn(*args)}
+        except Exception as exc:
+            return {"raises": type(exc).__name__}
+
+    assert len(cases["parse"]) >= 14 and len(cases["demand"]) >= 6
+    for case in cases["parse"]:
+        want = {k: v for k, v in case.items() if k != "text"}
+        assert attempt(AffinityManager.parse_affinity, case["text"]) == want, case["text"]
+    for case in cases["demand"]:
+        lists = {int(g): AffinityManager.parse_affinity(t) for g, t in case["lists"].items()}
+        for g, want in case["cores"].items():
+            assert attempt(AffinityManager.num_cpus_for_gpu, int(g), lists) == want, (case["lists"], g)
