@@ -1112,6 +1112,15 @@ def test_cpp_autograd_node_and_python_functions_of_the_row_losses_agree(device, 
         a = ta.kd_soft_target_loss(s.clone().requires_grad_(), t, 4.0)
     b = ta.kd_soft_target_loss(s, t, 4.0)
     assert a.grad_fn is None and b.grad_fn is None and bits_equal(a, b)
+    # one gradient buffer per forward: a second backward is refused by either kind of node
+    for node in (True, False):
+        monkeypatch.setattr(losses, "_HOST_NODE", node)
+        leaf = s.clone().requires_grad_()
+        loss = ta.kd_soft_target_loss(leaf, t, 4.0)
+        loss.backward(retain_graph=True)
+        with pytest.raises(RuntimeError, match="once per forward"):
+            loss.backward()
+    monkeypatch.setattr(losses, "_HOST_NODE", True)
     # calls that are not plain take the Python path and its errors
     with pytest.raises(ValueError):
         ta.kd_soft_target_loss(s, t[:, :, :50], 4.0)
