@@ -584,7 +584,7 @@ def test_kd_ce_mse_at_every_row_width_boundary(device, dtype):
             assert (sd.grad.cpu()[4] == 0).all(), case   # neither masked in nor labelled
 
 
-@pytest.mark.parametrize("rows", [77, 1027, 8195])
+@pytest.mark.parametrize("rows", [77, 1027, 2048, 2049, 8195])  # 2048: the last batch size whose workgroups count for themselves
 def test_kd_ce_counts_from_a_mask_that_starts_off_an_8_byte_boundary(device, rows):
     # short rows under a mask and with labels take a counting launch that reads the mask eight rows at a
     # time when it can; a mask that is a view three bytes into a buffer cannot, and must count the same
