@@ -895,6 +895,58 @@ def run_kernel_table(dev, with_cpu=True, with_eager=True):
             xg.grad = wg.grad = bg.grad = None
             y_c.backward(dy_c, retain_graph=True)
         cpu("bn_backward_32x256x56x56_f32", bn_bwd_cpu)
+    del xs, dys
+
+    # The late stages of a ResNet: many channels, planes of 7 x 7.  A plane is shorter than a wavefront's
+    # round of loads, so these shapes take the flat-tile kernels; the whole activation (25.7 MB) stays in
+    # the caches, and the call is a matter of launches and latency.
+    xs7 = torch.randn(256, 512, 7, 7, generator=dgen, device=dev) * 1.5 + 0.5
+    ys7, dy7, dx7 = torch.empty_like(xs7), torch.randn(256, 512, 7, 7, generator=dgen, device=dev), torch.empty_like(xs7)
+    g7, b7 = torch.rand(512, generator=g).to(dev) + 0.5, (torch.randn(512, generator=g) * 0.1).to(dev)
+    s7, q7, m7, i7, dg7, db7, ws7, par7 = z(512), z(512), z(512), z(512), z(512), z(512), z(4 * 512), {"p": 0}
+    one7 = xs7.numel() * 4
+
+    def fwd7():
+        _lib.check(lib.ts_bn_forward_train(xs7.data_ptr(), ys7.data_ptr(), g7.data_ptr(), b7.data_ptr(), 256, 512, 49,
+                                           s7.data_ptr(), q7.data_ptr(), m7.data_ptr(), i7.data_ptr(), ws7.data_ptr(),
+                                           par7["p"], 1e-5, stream), "ts_bn_forward_train")
+        par7["p"] ^= 1
+
+    def bwd7():
+        _lib.check(lib.ts_bn_backward(xs7.data_ptr(), dy7.data_ptr(), m7.data_ptr(), i7.data_ptr(), g7.data_ptr(),
+                                      dx7.data_ptr(), dg7.data_ptr(), db7.data_ptr(), ws7.data_ptr(), par7["p"], 256, 512,
+                                      49, 1, stream), "ts_bn_backward")
+        par7["p"] ^= 1
+    small_note = "planes of 49 values: the flat-tile kernels (a workgroup per 4 KB of the tensor as it lies in memory)"
+    out["bn_forward_train_256x512x7x7_f32"] = entry(3 * one7, _time_stream(fwd7), small_note, 2, working_set=2 * one7)
+    out["bn_backward_256x512x7x7_f32"] = entry(5 * one7, _time_stream(bwd7), small_note, 2, working_set=3 * one7)
+    ora7 = ts_oracle.DeferredBNOracle(512, chunks=1 << 30, weight=g7, bias=b7)
+    for attr in ("running_mean", "running_var", "num_batches_tracked", "sum", "sum_squares"):
+        setattr(ora7, attr, getattr(ora7, attr).to(dev))
+    eager("bn_forward_train_256x512x7x7_f32", lambda: ora7.forward(xs7))
+    if with_eager:
+        w7e, b7e, x7e = g7.clone().requires_grad_(), b7.clone().requires_grad_(), xs7.clone().requires_grad_()
+        y7e = torch.nn.functional.batch_norm(x7e, None, None, w7e, b7e, True, 0.0, 1e-5)
+
+        def bn7_bwd_eager():
+            x7e.grad = w7e.grad = b7e.grad = None
+            y7e.backward(dy7, retain_graph=True)
+        eager("bn_backward_256x512x7x7_f32", bn7_bwd_eager)
+        del w7e, b7e, x7e, y7e
+
+    # A gather of a few small pieces (per-micro-batch outputs, labels, embeddings): segments in the kernel's
+    # arguments, no table.  Host time is what such a call costs; the entry is the device side of it.
+    small = [torch.randn(64, 256, generator=dgen, device=dev) for _ in range(4)]
+    joined = torch.empty(256, 256, device=dev)
+    src_arr = (ctypes.c_void_p * 4)(*[t_.data_ptr() for t_ in small])
+    dst_arr = (ctypes.c_void_p * 4)(*[joined.data_ptr() + i * 65536 for i in range(4)])
+    len_arr = (ctypes.c_int64 * 4)(*([65536] * 4))
+
+    def few():
+        _lib.check(lib.ts_copy_few(src_arr, dst_arr, len_arr, 4, stream), "ts_copy_few")
+    out["gather_4x64KB_f32"] = entry(2 * 4 * 65536, _time_stream(few), "ts_copy_few: four segments in the kernel arguments",
+                                     1, working_set=2 * 4 * 65536)
+    eager("gather_4x64KB_f32", lambda: ts_oracle.gather(small))
     return out
 
 
