@@ -191,7 +191,13 @@ py::object infonce(const at::Tensor& q1, const at::Tensor& k1, const c10::option
   const bool record = at::GradMode::is_enabled();
   c10::optional<at::Tensor> s2 = q2;
   if (!record && two) s2 = q2->detach();
-  at::Tensor loss = InfoNCENode::apply(record ? q1 : q1.detach(), k1, s2, k2, tau, stream);
+  at::Tensor loss;
+  {
+    // allocations and launches need no interpreter: other Python threads (a pipeline's momentum
+    // update beside this loss) run meanwhile
+    py::gil_scoped_release no_gil;
+    loss = InfoNCENode::apply(record ? q1 : q1.detach(), k1, s2, k2, tau, stream);
+  }
   return py::cast(loss);
 }
 
@@ -290,7 +296,11 @@ py::object bn_train(const at::Tensor& x, const c10::optional<at::Tensor>& weight
     return py::none();
   const int64_t C = x.size(1);
   if (ws.numel() != 7 * C || ws.scalar_type() != at::kFloat || ws.device() != x.device()) return py::none();
-  at::Tensor y = BnTrainNode::apply(x, weight, bias, sum, sum_squares, ws, state, eps, stream);
+  at::Tensor y;
+  {
+    py::gil_scoped_release no_gil;
+    y = BnTrainNode::apply(x, weight, bias, sum, sum_squares, ws, state, eps, stream);
+  }
   return py::cast(y);
 }
 
@@ -471,7 +481,11 @@ py::object row_loss(int64_t kind, const at::Tensor& x1, const at::Tensor& y1, co
   const bool record = at::GradMode::is_enabled();
   c10::optional<at::Tensor> s2 = x2;
   if (!record && x2.has_value()) s2 = x2->detach();
-  at::Tensor loss = RowLossNode::apply(record ? x1 : x1.detach(), y1, s2, y2, mask, labels, kind, f, n, stream);
+  at::Tensor loss;
+  {
+    py::gil_scoped_release no_gil;
+    loss = RowLossNode::apply(record ? x1 : x1.detach(), y1, s2, y2, mask, labels, kind, f, n, stream);
+  }
   return py::cast(loss);
 }
 
