@@ -1129,3 +1129,52 @@ def test_cpp_autograd_node_and_python_functions_of_the_row_losses_agree(device, 
     strided = s.transpose(0, 1).requires_grad_()
     loss = ta.kd_soft_target_loss(strided, t.transpose(0, 1), 4.0)
     assert "RowLossNode" not in loss.grad_fn.name()
+
+
+def test_row_losses_from_two_threads_on_two_streams(device):
+    """The C++ node allocates and launches without the interpreter lock: two threads, each
+    on a stream of its own, get the same bits as one thread does."""
+    import threading
+    g = seeded(77)
+    s = (torch.randn(300, 100, generator=g) * 3).to(device)
+    t = (torch.randn(300, 100, generator=g) * 3).to(device)
+    y = torch.randint(0, 100, (300,), generator=g).to(device)
+    x = [torch.randn(256, 128, generator=g).to(device) for _ in range(4)]
+
+    def kd():
+        leaf = s.clone().requires_grad_()
+        loss = ta.kd_ce_loss(leaf, t, y, 4.0, 0.7, 1.0)
+        loss.backward()
+        return loss.detach(), leaf.grad
+
+    def byol():
+        a, b = x[0].clone().requires_grad_(), x[1].clone().requires_grad_()
+        loss = ta.byol_contrastive_loss(a, b, x[2], x[3])
+        loss.backward()
+        return loss.detach(), a.grad, b.grad
+
+    want = {"kd": kd(), "byol": byol()}
+    torch.cuda.synchronize()
+    got, errors = {"kd": [], "byol": []}, []
+
+    def worker(name, fn):
+        try:
+            stream = torch.cuda.Stream(device)
+            stream.wait_stream(torch.cuda.current_stream(device))
+            with torch.cuda.stream(stream):
+                for _ in range(40):
+                    got[name].append(fn())
+            stream.synchronize()
+        except BaseException as exc:
+            errors.append(exc)
+
+    threads = [threading.Thread(target=worker, args=(n, f)) for n, f in (("kd", kd), ("byol", byol))]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert not errors, errors
+    for name in got:
+        assert len(got[name]) == 40
+        for result in got[name]:
+            assert all(bits_equal(a, b) for a, b in zip(result, want[name])), name
