@@ -1,7 +1,8 @@
 // A consumer of the C ABI that knows nothing of Python or PyTorch: plain HIP
 // runtime calls for memory, include/tspipe_amd.h for everything else.  Checks
 // the EMA bit for bit against one-rounding-per-operation host arithmetic and
-// the KD soft-target loss against a double-precision evaluation, then prints
+// the KD soft-target loss against a double-precision evaluation, gathers a few
+// small pieces without a table, asks for a loss over zero rows, then prints
 // "c-abi consumer: ok".  Built by __graft_entry__.build(), run by the GPU tests.
 #include <hip/hip_runtime.h>
 
@@ -146,12 +147,74 @@ static int check_kd(hipStream_t stream) {
   return bad;
 }
 
+// A gather of a few small pieces without a table: odd byte counts, an empty segment, unaligned starts.
+static int check_copy_few(hipStream_t stream) {
+  const int64_t bytes[4] = {4099, 0, 65536, 7};
+  const int64_t src_off[4] = {0, 0, 3, 1}, total = 4099 + 65536 + 7;
+  std::vector<std::vector<unsigned char>> host(4);
+  const void* src[4];
+  void* dst[4];
+  unsigned char* joined = nullptr;
+  HIP_OK(hipMalloc((void**)&joined, (size_t)total + 16));
+  HIP_OK(hipMemset(joined, 0xee, (size_t)total + 16));
+  int64_t at = 0;
+  for (int i = 0; i < 4; ++i) {
+    host[i].resize((size_t)bytes[i]);
+    for (auto& v : host[i]) v = (unsigned char)(frand() * 127.f + 128.f);
+    unsigned char* d = nullptr;
+    HIP_OK(hipMalloc((void**)&d, (size_t)bytes[i] + 32));
+    if (bytes[i]) HIP_OK(hipMemcpy(d + src_off[i], host[i].data(), (size_t)bytes[i], hipMemcpyHostToDevice));
+    src[i] = d + src_off[i];
+    dst[i] = joined + at;
+    at += bytes[i];
+  }
+  TS_OK_(ts_copy_few(src, dst, bytes, 4, stream));
+  HIP_OK(hipStreamSynchronize(stream));
+  std::vector<unsigned char> got((size_t)total + 16);
+  HIP_OK(hipMemcpy(got.data(), joined, got.size(), hipMemcpyDeviceToHost));
+  int bad = 0;
+  at = 0;
+  for (int i = 0; i < 4; ++i) {
+    if (bytes[i] && std::memcmp(got.data() + at, host[i].data(), (size_t)bytes[i]) != 0) {
+      std::fprintf(stderr, "copy_few: segment %d differs\n", i);
+      ++bad;
+    }
+    at += bytes[i];
+  }
+  for (int64_t j = total; j < total + 16; ++j)
+    if (got[(size_t)j] != 0xee) {
+      std::fprintf(stderr, "copy_few: wrote past the end at %lld\n", (long long)j);
+      ++bad;
+      break;
+    }
+  if (ts_copy_few(src, dst, bytes, 17, stream) != TS_ERR_RANGE) ++bad;
+  return bad;
+}
+
+// A loss over zero rows is a mean over nothing: NaN, no error, input pointers not needed.
+static int check_kd_zero_rows(hipStream_t stream) {
+  void* ws;
+  float* dloss;
+  HIP_OK(hipMalloc(&ws, ts_kd_workspace_bytes(0, 100, TS_F32)));
+  HIP_OK(hipMalloc((void**)&dloss, 4));
+  HIP_OK(hipMemset(dloss, 0, 4));
+  TS_OK_(ts_kd_fwd_bwd(nullptr, nullptr, nullptr, 0, 100, 100, 100, 0.25f, 16.f, ws, dloss, nullptr, 100, TS_F32, stream));
+  HIP_OK(hipStreamSynchronize(stream));
+  float loss = 0.f;
+  HIP_OK(hipMemcpy(&loss, dloss, 4, hipMemcpyDeviceToHost));
+  if (!std::isnan(loss)) {
+    std::fprintf(stderr, "kd over zero rows gave %g, not NaN\n", loss);
+    return 1;
+  }
+  return 0;
+}
+
 int main() {
   std::printf("%s\n", ts_version());
   HIP_OK(hipSetDevice(0));
   hipStream_t stream;
   HIP_OK(hipStreamCreate(&stream));
-  const int bad = check_ema(stream) + check_kd(stream);
+  const int bad = check_ema(stream) + check_kd(stream) + check_copy_few(stream) + check_kd_zero_rows(stream);
   // error paths answer with a status, not a crash
   if (ts_ema_multi(nullptr, 1, 1024, 0.5f, 0.5f, stream) != TS_ERR_ARG) return 4;
   if (ts_ema_multi(nullptr, 0, 1000, 0.5f, 0.5f, stream) != TS_ERR_ARG) return 5;  // chunk not a multiple of 1024
